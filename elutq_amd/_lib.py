@@ -1,0 +1,60 @@
+"""ctypes binding of libelutq_hip.so (the C ABI declared in include/elutq_hip.h).
+
+The library is the only compute path: if it is missing or a symbol is absent this
+module raises; there is no PyTorch or CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libelutq_hip.so")
+
+_vp, _ci, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/elutq_hip.h
+SIGNATURES = {
+    "elutq_version": (_ci, []),
+    "elutq_status_string": (ctypes.c_char_p, [_ci]),
+    "elutq_hlq_planes_bytes": (_sz, [_ci, _ci, _ci]),
+    "elutq_hlq_scales_bytes": (_sz, [_ci, _ci, _ci, _ci]),
+    "elutq_hlq_zeros_bytes": (_sz, [_ci, _ci, _ci]),
+    "elutq_hlq_repack_host": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _vp, _vp]),
+    "elutq_hlq_unpack_host": (_ci, [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _vp, _vp]),
+    "elutq_hlq_workspace_bytes": (_sz, [_ci, _ci, _ci, _ci, _ci]),
+    "elutq_hlq_workspace_init": (_ci, [_vp, _sz, _vp]),
+    "elutq_hlq_gemv_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp]),
+    "elutq_hlq_gemv_f16_tuned": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _ci, _ci]),
+    "elutq_hlq_gemm_f16": (_ci, [_vp] * 6 + [_ci] * 5 + [_vp, _sz, _vp]),
+    "elutq_hlq_dequant_f16": (_ci, [_vp] * 4 + [_ci] * 4 + [_vp]),
+}
+
+_lib = None
+
+
+class ElutqError(RuntimeError):
+    def __init__(self, status: int, where: str):
+        self.status = status
+        msg = lib().elutq_status_string(status).decode()
+        super().__init__(f"{where}: {msg} (status {status})")
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m elutq_amd.build` "
+                "(there is no fallback path)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)          # AttributeError if the symbol is not exported
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def check(status: int, where: str) -> None:
+    if status != 0:
+        raise ElutqError(status, where)

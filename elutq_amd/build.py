@@ -1,0 +1,49 @@
+"""Builds libelutq_hip.so in-tree with hipcc for gfx950.
+
+    python -m elutq_amd.build            # compile (always)
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(_PKG, "csrc")
+LIB_PATH = os.path.join(_PKG, "libelutq_hip.so")
+SOURCES = ["hlq_gemv.hip", "hlq_gemm.hip", "hlq_misc.hip", "hlq_repack.cpp"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found (need ROCm with gfx950 support)")
+    return exe
+
+
+def build(verbose: bool = False) -> str:
+    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    tmp = LIB_PATH + ".tmp"
+    cmd = [hipcc(), *HIPCC_FLAGS, "-I", os.path.join(_PKG, "..", "include"), "-o", tmp, *srcs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

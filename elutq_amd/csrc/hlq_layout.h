@@ -1,0 +1,52 @@
+// Device-side layout of a repacked HLQ layer, shared by the host repack and the kernels.
+//
+// A "unit" is 128 consecutive k of one output column in one bit-plane: 128 bits = one
+// dwordx4 per lane.  Output columns are tiled in blocks of 64 (one wavefront, lane =
+// column), so a wave-wide dwordx4 load covers one unit of 64 columns = 1 KiB contiguous.
+//
+//   planes  uint4    [ncb][U][bits][64]        U = K/128, ncb = ceil(N/64)
+//   scales  uint32   [ncb][NT][bits][64]       one dword = fp16 scales of groups 2t, 2t+1
+//   zeros   uint32   [ncb][NT][64]             one dword = fp16 zeros  of groups 2t, 2t+1
+//
+// NT = ceil(NG/2) with NG = K/G groups per column ("task" t = the groups one meta dword
+// covers: two units at G = 128, one unit at G = 64).  Columns >= N and the odd group of
+// an odd NG are zero-filled.
+//
+// Inside a unit, dword d holds k = 32d .. 32d+31 LSB-first (bit i <-> k = 32d + i, the
+// byte order of the reference's w_quant.bin read as little-endian dwords), rotated left
+// by HLQ_ROT bits.  After the rotation the 4-bit field of chunk c (k = 4c..4c+3) sits at
+// bits 4c+2 .. 4c+5, so `byte_j & 0x3C` is 4 * (nibble of chunk 2j) -- a ready-made byte
+// offset into a table of 16 int32 entries -- and the same holds for chunk 2j+1 after a
+// further rotate right by 4.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+#define HLQ_CB 64
+#define HLQ_UNIT 128
+#define HLQ_ROT 2
+
+struct HlqGeo {
+    int K, N, bits, group;
+    int U;      // units per column
+    int NG;     // groups per column
+    int NT;     // tasks (meta dwords) per column
+    int UPT;    // units per task: 2 at G=128, 1 at G=64
+    int ncb;    // column blocks
+};
+
+static inline HlqGeo hlq_geo(int K, int N, int bits, int group)
+{
+    HlqGeo g;
+    g.K = K; g.N = N; g.bits = bits; g.group = group;
+    g.U = K / HLQ_UNIT;
+    g.NG = K / group;
+    g.NT = (g.NG + 1) / 2;
+    g.UPT = group == 64 ? 1 : 2;
+    g.ncb = (N + HLQ_CB - 1) / HLQ_CB;
+    return g;
+}
+
+static inline size_t hlq_planes_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.U * g.bits * HLQ_CB * 16; }
+static inline size_t hlq_scales_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * g.bits * HLQ_CB * 4; }
+static inline size_t hlq_zeros_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * HLQ_CB * 4; }

@@ -1,0 +1,187 @@
+"""HLQLinear: the quantized-linear module of the HLQ path on MI355X.
+
+On the Python side the reference has no quantized module: GPTQ/HLQ.py:173 writes the
+dequantized weight back into ``nn.Linear`` and the forward is ``x @ W_deq.T + bias``.
+HLQLinear keeps that ``nn.Linear`` surface (``in_features``, ``out_features``, optional
+``bias``, ``forward(x[..., K]) -> [..., N]``) but holds the packed planes / scales / zeros
+of the export files and runs the HIP LUT kernels through the C ABI, as the C++ runtime's
+``arm_gemm(m, k, n, input, output, temp, weight_tensor*, ...)`` does on the CPU
+(C++/ops/include/arm/arm_gemm.h:4-14).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import numpy as np
+import torch
+from torch import nn
+
+from . import _lib
+from .export_io import ExportedLinear, read_export_dir
+
+_workspaces: dict = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    """One zero-initialised scratch buffer per (device, stream); calls on a stream are
+    ordered, which is what the kernels' arrival counters need."""
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.zeros(max(nbytes, 1 << 21), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def repack_export_arrays(w_quant, w_scale, w_zero, group: int):
+    """Export-layout NumPy arrays -> (planes, scales, zeros) uint8 NumPy arrays in the
+    kernel layout (host-side permutation done by the library)."""
+    L = _lib.lib()
+    w_quant = np.ascontiguousarray(w_quant, dtype=np.uint8)
+    w_scale = np.ascontiguousarray(w_scale, dtype=np.float16)
+    w_zero = np.ascontiguousarray(w_zero, dtype=np.float16)
+    bits, n, k8 = w_quant.shape
+    k = k8 * 8
+    if w_scale.shape != (bits, n, k // group) or w_zero.shape != (n, k // group):
+        raise ValueError("w_scale / w_zero shapes do not match w_quant and the group size")
+    planes = np.empty(L.elutq_hlq_planes_bytes(k, n, bits), dtype=np.uint8)
+    scales = np.empty(L.elutq_hlq_scales_bytes(k, n, bits, group), dtype=np.uint8)
+    zeros = np.empty(L.elutq_hlq_zeros_bytes(k, n, group), dtype=np.uint8)
+    if planes.size == 0 or scales.size == 0:
+        raise ValueError(f"unsupported HLQ shape K={k} N={n} bits={bits} group={group} "
+                         "(need K % 128 == 0, bits 1..4, group 64 or 128)")
+    vp = ctypes.c_void_p
+    _lib.check(L.elutq_hlq_repack_host(w_quant.ctypes.data_as(vp), w_scale.ctypes.data_as(vp),
+                                       w_zero.ctypes.data_as(vp), k, n, bits, group,
+                                       planes.ctypes.data_as(vp), scales.ctypes.data_as(vp),
+                                       zeros.ctypes.data_as(vp)), "elutq_hlq_repack_host")
+    return planes, scales, zeros
+
+
+def unpack_to_export_arrays(planes, scales, zeros, k: int, n: int, bits: int, group: int):
+    """Inverse of repack_export_arrays."""
+    L = _lib.lib()
+    vp = ctypes.c_void_p
+    planes = np.ascontiguousarray(planes, dtype=np.uint8)
+    scales = np.ascontiguousarray(scales, dtype=np.uint8)
+    zeros = np.ascontiguousarray(zeros, dtype=np.uint8)
+    w_quant = np.empty((bits, n, k // 8), dtype=np.uint8)
+    w_scale = np.empty((bits, n, k // group), dtype=np.float16)
+    w_zero = np.empty((n, k // group), dtype=np.float16)
+    _lib.check(L.elutq_hlq_unpack_host(planes.ctypes.data_as(vp), scales.ctypes.data_as(vp),
+                                       zeros.ctypes.data_as(vp), k, n, bits, group,
+                                       w_quant.ctypes.data_as(vp), w_scale.ctypes.data_as(vp),
+                                       w_zero.ctypes.data_as(vp)), "elutq_hlq_unpack_host")
+    return w_quant, w_scale, w_zero
+
+
+class HLQLinear(nn.Module):
+    """``nn.Linear``-shaped module over HLQ-packed weights (fp16 activations)."""
+
+    def __init__(self, in_features: int, out_features: int, bits: int, group_size: int,
+                 planes: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor,
+                 bias: torch.Tensor | None = None):
+        super().__init__()
+        self.in_features, self.out_features = int(in_features), int(out_features)
+        self.bits, self.group_size = int(bits), int(group_size)
+        self.register_buffer("planes", planes)
+        self.register_buffer("scales", scales)
+        self.register_buffer("zeros", zeros)
+        self.register_buffer("bias", bias)
+        self._ws_bytes = _lib.lib().elutq_hlq_workspace_bytes(self.in_features, self.out_features,
+                                                              self.bits, self.group_size, 1)
+        if self._ws_bytes == 0:
+            raise ValueError(f"unsupported HLQ shape K={in_features} N={out_features} bits={bits} "
+                             f"group={group_size} (need K % 128 == 0, bits 1..4, group 64 or 128)")
+        self.ksplit, self.waves = 0, 0      # 0 = library default; set for tuning
+
+    # -- construction ------------------------------------------------------------------
+    @classmethod
+    def from_export_arrays(cls, w_quant, w_scale, w_zero, group_size: int, bias=None,
+                           device="cuda") -> "HLQLinear":
+        planes, scales, zeros = repack_export_arrays(w_quant, w_scale, w_zero, group_size)
+        bits, n, k8 = np.asarray(w_quant).shape
+        dev = torch.device(device)
+        b = None if bias is None else torch.from_numpy(np.ascontiguousarray(bias, dtype=np.float16)).to(dev)
+        return cls(k8 * 8, n, bits, group_size, torch.from_numpy(planes).to(dev),
+                   torch.from_numpy(scales).to(dev), torch.from_numpy(zeros).to(dev), b)
+
+    @classmethod
+    def from_export(cls, e: ExportedLinear, device="cuda") -> "HLQLinear":
+        return cls.from_export_arrays(e.w_quant, e.w_scale, e.w_zero, e.group, e.bias, device)
+
+    @classmethod
+    def from_export_dir(cls, path: str, device="cuda", group_size: int | None = None) -> "HLQLinear":
+        return cls.from_export(read_export_dir(path, group_size), device)
+
+    # -- compute -----------------------------------------------------------------------
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.shape[-1] != self.in_features:
+            raise ValueError(f"expected last dim {self.in_features}, got {tuple(x.shape)}")
+        if not x.is_cuda:
+            raise RuntimeError("HLQLinear runs on the GPU only (there is no CPU path)")
+        in_dtype = x.dtype
+        x2 = x.reshape(-1, self.in_features)
+        if x2.dtype != torch.float16:
+            x2 = x2.to(torch.float16)
+        x2 = x2.contiguous()
+        m = x2.shape[0]
+        y = torch.empty((m, self.out_features), dtype=torch.float16, device=x.device)
+        if m:
+            ws = _workspace(x.device, self._ws_bytes)
+            stream = torch.cuda.current_stream(x.device).cuda_stream
+            L = _lib.lib()
+            bias = self.bias.data_ptr() if self.bias is not None else None
+            if m == 1:
+                rc = L.elutq_hlq_gemv_f16_tuned(self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
+                                                bias, x2.data_ptr(), y.data_ptr(), self.in_features,
+                                                self.out_features, self.bits, self.group_size,
+                                                ws.data_ptr(), ws.numel(), stream, self.ksplit, self.waves)
+                _lib.check(rc, "elutq_hlq_gemv_f16")
+            else:
+                rc = L.elutq_hlq_gemm_f16(self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
+                                          bias, x2.data_ptr(), y.data_ptr(), m, self.in_features,
+                                          self.out_features, self.bits, self.group_size,
+                                          ws.data_ptr(), ws.numel(), stream)
+                _lib.check(rc, "elutq_hlq_gemm_f16")
+        y = y.reshape(*x.shape[:-1], self.out_features)
+        return y if in_dtype == torch.float16 else y.to(in_dtype)
+
+    def dequantize(self) -> torch.Tensor:
+        """Dense fp16 W [N, K] (``dequantize_with_scales``, GPTQ/quant.py:176-183)."""
+        w = torch.empty((self.out_features, self.in_features), dtype=torch.float16, device=self.planes.device)
+        stream = torch.cuda.current_stream(self.planes.device).cuda_stream
+        rc = _lib.lib().elutq_hlq_dequant_f16(self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
+                                              w.data_ptr(), self.in_features, self.out_features, self.bits,
+                                              self.group_size, stream)
+        _lib.check(rc, "elutq_hlq_dequant_f16")
+        return w
+
+    def extra_repr(self) -> str:
+        return (f"in_features={self.in_features}, out_features={self.out_features}, bits={self.bits}, "
+                f"group_size={self.group_size}, bias={self.bias is not None}")
+
+
+def replace_linear(model: nn.Module, export_root: str, device="cuda", group_size: int | None = None) -> int:
+    """Swaps every ``nn.Linear`` that has an export directory for an HLQLinear.
+
+    Directories follow the reference: ``<export_root>/<layer id>/<name>`` with ``name`` the
+    module path inside the decoder layer (``self_attn.q_proj`` ... ``mlp.down_proj``,
+    GPTQ/llama.py:90-95, GPTQ/HLQ.py:73).  Returns the number of modules replaced."""
+    replaced = 0
+    for full_name, mod in list(model.named_modules()):
+        if not isinstance(mod, nn.Linear):
+            continue
+        parts = full_name.split(".")
+        idx = next((i for i, p in enumerate(parts) if p.isdigit()), None)
+        if idx is None:
+            continue
+        path = os.path.join(export_root, parts[idx], ".".join(parts[idx + 1:]))
+        if not os.path.exists(os.path.join(path, "weight_config.json")):
+            continue
+        new = HLQLinear.from_export_dir(path, device, group_size)
+        parent = model.get_submodule(".".join(parts[:-1])) if len(parts) > 1 else model
+        setattr(parent, parts[-1], new)
+        replaced += 1
+    return replaced

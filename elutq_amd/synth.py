@@ -1,0 +1,80 @@
+"""Seeded synthetic HLQ layers with the distributions the benchmark configs name.
+
+All tensors are drawn on the CPU from ``torch.Generator().manual_seed(seed)`` and
+rounded to fp16 before anything uses them, so every machine sees the same bits:
+
+  x       randn(M, K)                                            -> fp16
+  planes  randint(0, 2, [B, N, K])  (i.i.d. Bernoulli 0.5)
+  w2      s0 ~ U(0.005, 0.02) per (n, group);  s1 = 2*s0*U(0.8, 1.2)
+  w3/w4   s0 ~ U(0.003, 0.01);                 s_b = 2^b*s0*U(0.8, 1.2), b >= 1
+  zero    z = -(sum_b s_b)/2 * U(0.9, 1.1)
+
+The arrays come back in the reference's export layout (GPTQ/HLQ.py:207-251):
+w_quant uint8 [B, N, K/8] packed LSB-first along K, w_scale fp16 [B, N, K/G],
+w_zero fp16 [N, K/G].
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+
+@dataclass
+class SynthLayer:
+    k: int
+    n: int
+    bits: int
+    group: int
+    w_quant: np.ndarray     # uint8 [B, N, K/8]
+    w_scale: np.ndarray     # fp16  [B, N, K/G]
+    w_zero: np.ndarray      # fp16  [N, K/G]
+    bias: np.ndarray | None  # fp16 [N]
+    x: np.ndarray           # fp16  [M, K]
+
+
+def pack_bits_lsb_first(planes: np.ndarray) -> np.ndarray:
+    """0/1 uint8 [..., K] -> uint8 [..., K/8]; bit j of byte i is element 8*i+j
+    (the order Pack_T_MAC_Weight writes, GPTQ/HLQ.py:239-251)."""
+    return np.packbits(np.asarray(planes, dtype=np.uint8), axis=-1, bitorder="little")
+
+
+def make_layer(k: int, n: int, bits: int = 2, group: int = 128, m: int = 1, seed: int = 0,
+               bias: bool = False) -> SynthLayer:
+    assert k % group == 0 and k % 8 == 0
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(m, k, generator=g).to(torch.float16)
+    planes = torch.randint(0, 2, (bits, n, k), generator=g, dtype=torch.uint8)
+    ng = k // group
+
+    def uni(lo, hi):
+        return torch.rand(n, ng, generator=g) * (hi - lo) + lo
+
+    s0 = uni(0.005, 0.02) if bits == 2 else uni(0.003, 0.01)
+    scales = [s0]
+    for b in range(1, bits):
+        scales.append((2.0 ** b) * s0 * uni(0.8, 1.2))
+    s = torch.stack(scales, 0)                                   # [B, N, K/G] fp32
+    z = -(s.sum(0)) / 2 * uni(0.9, 1.1)
+    bvec = None
+    if bias:
+        bvec = (torch.randn(n, generator=g) * 0.1).to(torch.float16).numpy()
+    return SynthLayer(k=k, n=n, bits=bits, group=group,
+                      w_quant=pack_bits_lsb_first(planes.numpy()),
+                      w_scale=s.to(torch.float16).numpy(),
+                      w_zero=z.to(torch.float16).numpy(),
+                      bias=bvec, x=x.numpy())
+
+
+# (K, N) of the LLaMA-3-8B projections and of the LLaMA-2-13B prefill shapes.
+LLAMA3_8B_SHAPES = {
+    "q_proj": (4096, 4096), "k_proj": (4096, 1024), "v_proj": (4096, 1024), "o_proj": (4096, 4096),
+    "gate_proj": (4096, 14336), "up_proj": (4096, 14336), "down_proj": (14336, 4096),
+}
+LLAMA2_13B_PREFILL_SHAPES = [(5120, 5120), (5120, 13824), (13824, 5120)]
+
+
+def algorithmic_bytes(k: int, n: int, bits: int, group: int, m: int = 1) -> int:
+    """planes + fp16 per-plane scales + fp16 zeros + x + y."""
+    return k * n * bits // 8 + 2 * bits * n * (k // group) + 2 * n * (k // group) + 2 * m * k + 2 * m * n

@@ -1,0 +1,124 @@
+/*
+ * elutq_hip.h -- C ABI of libelutq_hip.so: the HLQ bit-serial LUT GEMV / small-batch
+ * GEMM for AMD MI355X (gfx950).
+ *
+ * HLQ stores a linear layer's weight W[N][K] as
+ *     W[n][k] = sum_b  s[b][n][k/G] * B_b[n][k]  +  z[n][k/G]
+ * with `bits` binary planes B_b, fp16 per-plane group scales s and an fp16 group
+ * zero z, groups of G = 64 or 128 consecutive k.
+ *
+ * The entry points replace, one for one, the reference's CPU operator for this
+ * path (file:line under the reference tree, Nkniexin/ELUTQ):
+ *
+ *   elutq_hlq_repack_*      load_Parameter(..LINEAR..)        C++/ops/src/arm/parameters.cpp:8-70
+ *                           t_mac_g4_rearrange_weight_normal_impl
+ *                                                            C++/ops/src/arm/arm_t_mac_kernal.cpp:472-552
+ *   elutq_hlq_gemv_f16      arm_gemm(m == 1, bit <= 4)        C++/ops/include/arm/arm_gemm.h:4-14
+ *                           MultiThread_arm_gemv_w_lowbit_activation_fp_impl
+ *                                                            C++/ops/src/arm/arm_gemm.cpp:312-360
+ *   elutq_hlq_gemm_f16      arm_gemm(m  > 1, bit <= 4)        C++/ops/src/arm/arm_gemm.cpp:362-387
+ *   elutq_hlq_dequant_f16   dequantize_with_scales            GPTQ/quant.py:176-183
+ *
+ * Conventions
+ *   - plain C types only; every `d_` pointer is DEVICE memory owned by the caller,
+ *     every `h_` pointer is HOST memory owned by the caller;
+ *   - compute calls are asynchronous on `stream` (a hipStream_t passed as void*,
+ *     NULL = the default stream), never synchronise, never allocate, and are
+ *     capturable in a HIP graph;
+ *   - every function returns ELUTQ_OK (0) or a negative elutq_status; nothing throws;
+ *   - a workspace is private to one in-flight call: calls that share a workspace
+ *     must be ordered on one stream.  It must be zero-filled once after allocation
+ *     (elutq_hlq_workspace_init); the kernels leave it zeroed where that matters.
+ */
+#ifndef ELUTQ_HIP_H
+#define ELUTQ_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum elutq_status {
+    ELUTQ_OK = 0,
+    ELUTQ_ERR_NULL = -1,       /* a required pointer is NULL */
+    ELUTQ_ERR_SHAPE = -2,      /* K % 128 != 0, K % group != 0, K, N or M < 1 */
+    ELUTQ_ERR_BITS = -3,       /* bits outside 1..4 */
+    ELUTQ_ERR_GROUP = -4,      /* group not 64 or 128 */
+    ELUTQ_ERR_WORKSPACE = -5,  /* workspace smaller than elutq_hlq_workspace_bytes() */
+    ELUTQ_ERR_HIP = -6,        /* a HIP runtime call failed (launch, attribute) */
+    ELUTQ_ERR_TUNING = -7      /* explicit ksplit / waves arguments out of range */
+} elutq_status;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int elutq_version(void);
+
+/* Static description of a status code. */
+const char *elutq_status_string(int status);
+
+/* Sizes, in bytes, of the three device buffers holding a repacked layer. */
+size_t elutq_hlq_planes_bytes(int K, int N, int bits);
+size_t elutq_hlq_scales_bytes(int K, int N, int bits, int group);
+size_t elutq_hlq_zeros_bytes(int K, int N, int group);
+
+/*
+ * Host-side repack: the reference's export files, byte for byte
+ * (GPTQ/HLQ.py:207-251: w_quant.bin uint8 [bits][N][K/8] packed LSB-first along K,
+ * w_scale.bin fp16 [bits][N][K/G], w_zero.bin fp16 [N][K/G]) -> the layout the
+ * kernels read.  Output buffers are host memory of the sizes above; copy them to
+ * the device unchanged.  Pure permutation, no arithmetic.
+ */
+int elutq_hlq_repack_host(const uint8_t *h_w_quant, const uint16_t *h_w_scale,
+                          const uint16_t *h_w_zero, int K, int N, int bits, int group,
+                          void *h_planes_out, void *h_scales_out, void *h_zeros_out);
+
+/* Inverse of elutq_hlq_repack_host (kernel layout -> export layout). */
+int elutq_hlq_unpack_host(const void *h_planes, const void *h_scales, const void *h_zeros,
+                          int K, int N, int bits, int group,
+                          uint8_t *h_w_quant_out, uint16_t *h_w_scale_out, uint16_t *h_w_zero_out);
+
+/* Workspace size for a call with up to M activation rows. */
+size_t elutq_hlq_workspace_bytes(int K, int N, int bits, int group, int M);
+
+/* Zero-fills a freshly allocated workspace (asynchronous on `stream`). */
+int elutq_hlq_workspace_init(void *d_workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * y[N] = W x + bias, batch 1.  d_x fp16 [K], d_y fp16 [N], d_bias fp16 [N] or NULL.
+ * Replaces arm_gemm(m = 1, ...) for bit <= 4, use_sparse = false.
+ */
+int elutq_hlq_gemv_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
+                       const void *d_bias, const void *d_x, void *d_y,
+                       int K, int N, int bits, int group,
+                       void *d_workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Same computation with the launch shape chosen by the caller: `ksplit` slices of K
+ * per column block (1..number of group pairs) and `waves` wavefronts per workgroup
+ * (1..16); 0 = library default.  For tuning and for tests that must reach every
+ * reduction path; results do not depend on these beyond fp32 summation order.
+ */
+int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const void *d_zeros,
+                             const void *d_bias, const void *d_x, void *d_y,
+                             int K, int N, int bits, int group,
+                             void *d_workspace, size_t workspace_bytes, void *stream,
+                             int ksplit, int waves);
+
+/*
+ * y[M][N] = x[M][K] W^T + bias, row-major fp16, 1 <= M.  Replaces arm_gemm(m > 1, ...),
+ * which the reference defines as one GEMV per row.
+ */
+int elutq_hlq_gemm_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
+                       const void *d_bias, const void *d_x, void *d_y,
+                       int M, int K, int N, int bits, int group,
+                       void *d_workspace, size_t workspace_bytes, void *stream);
+
+/* W[N][K] fp16 row-major from the repacked buffers (dequantize_with_scales). */
+int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
+                          void *d_w_out, int K, int N, int bits, int group, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ELUTQ_HIP_H */

@@ -1,0 +1,272 @@
+"""CPU oracle for the HLQ bit-serial LUT GEMV/GEMM path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, in NumPy, what the reference (Nkniexin/ELUTQ) computes on
+the path "packed --export files -> loader repack -> LUT GEMV/GEMM".  It is the
+checker the HIP kernels are compared with; nothing in the shipped package may
+import it (only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg).
+
+Reference lines each function follows (paths relative to the reference root):
+
+  pack_planes / unpack_planes   GPTQ/HLQ.py:239-251   (Pack_T_MAC_Weight, LSB-first)
+  export_arrays                 GPTQ/HLQ.py:207-236   (w_zero / w_scale / w_quant files)
+  weight_config                 GPTQ/HLQ.py:175-193   (weight_config.json keys)
+  dequantize                    GPTQ/quant.py:176-183 (W = sum_b q_b*s_b + z)
+  rearrange_reference           C++/ops/src/arm/arm_t_mac_kernal.cpp:472-552
+  lut_float                     C++/ops/src/arm/arm_t_mac_kernal.cpp:95-138
+  gemv_fp16_chain               C++/ops/src/arm/arm_gemm.cpp:248-308 +
+                                C++/ops/src/arm/arm_t_mac_kernal.cpp:364-469
+  gemm_rows                     C++/ops/src/arm/arm_gemm.cpp:362-387
+
+Parity pins (tests/test_oracle_*.py): the reference ships no tests, golden
+vectors or fixtures for this path, so every function is pinned by mathematics:
+pack_planes against numpy.packbits(bitorder="little") and hand vectors;
+dequantize/gemv against an independent einsum in float64 and the closed forms
+(all-zero planes, all-one planes, unit-vector activations, single set bit);
+rearrange_reference by bijectivity and by brute-force index enumeration on tiny
+shapes; lut_float by brute force over the 16 subsets; gemv_fp16_chain against
+the C restatement (oracle/lut_gemv_ref.c, an independent implementation that
+indexes the rearranged buffers the way the reference kernel does) bit-for-bit,
+and against integer-only inputs where every fp16 operation is exact so the
+chain must equal the float64 result bit-for-bit.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+__all__ = [
+    "pack_planes", "unpack_planes", "export_arrays", "weight_config",
+    "dequantize", "gemv_f64", "gemm_f64", "rearrange_reference",
+    "lut_float", "gemv_fp16_chain", "gemm_rows", "rel_err",
+]
+
+
+# --------------------------------------------------------------------------- #
+# a1: bit-plane packing (GPTQ/HLQ.py:239-251)
+# --------------------------------------------------------------------------- #
+def pack_planes(planes: np.ndarray) -> np.ndarray:
+    """uint8 0/1 planes [B, N, K] -> uint8 [B, N, K/8]; bit j of byte i is
+    planes[b, n, 8*i + j] (LSB first), exactly the triple loop of
+    Pack_T_MAC_Weight."""
+    planes = np.asarray(planes)
+    assert planes.ndim == 3 and planes.shape[2] % 8 == 0
+    b, n, k = planes.shape
+    p = planes.astype(np.uint8).reshape(b, n, k // 8, 8)
+    out = np.zeros((b, n, k // 8), dtype=np.uint8)
+    for j in range(8):
+        out |= (p[..., j] & 1) << j
+    return out
+
+
+def unpack_planes(packed: np.ndarray) -> np.ndarray:
+    """Inverse of pack_planes: uint8 [B, N, K/8] -> uint8 0/1 [B, N, K]."""
+    packed = np.asarray(packed, dtype=np.uint8)
+    b, n, k8 = packed.shape
+    out = np.zeros((b, n, k8, 8), dtype=np.uint8)
+    for j in range(8):
+        out[..., j] = (packed >> j) & 1
+    return out.reshape(b, n, k8 * 8)
+
+
+# --------------------------------------------------------------------------- #
+# a2: on-disk arrays (GPTQ/HLQ.py:207-236) and json (GPTQ/HLQ.py:175-193)
+# --------------------------------------------------------------------------- #
+def export_arrays(q: np.ndarray, scale: np.ndarray, zero: np.ndarray):
+    """Quantizer-side tensors -> the three file payloads.
+
+    q     uint8 [N, K, B]    (0/1; quant.py:204)
+    scale float [N, K/G, B]  (quant.py:205)
+    zero  float [N, K/G, 1]  (quant.py:206)
+
+    returns (w_quant uint8 [B,N,K/8], w_scale fp16 [B,N,K/G], w_zero fp16 [N,K/G])
+    whose .tobytes() are the contents of w_quant.bin / w_scale.bin / w_zero.bin.
+    """
+    q = np.asarray(q)
+    scale = np.asarray(scale)
+    zero = np.asarray(zero)
+    assert q.ndim == 3 and scale.ndim == 3 and zero.ndim == 3
+    w_zero = zero.astype(np.float16)[..., 0].copy()                    # [N, K/G]   (no permute)
+    w_scale = np.ascontiguousarray(scale.astype(np.float16).transpose(2, 0, 1))  # [B, N, K/G]
+    planes = np.ascontiguousarray(q.astype(np.uint8).transpose(2, 0, 1))         # [B, N, K]
+    w_quant = pack_planes(planes)
+    return w_quant, w_scale, w_zero
+
+
+def weight_config(k: int, n: int, bits: int, has_bias: bool, groupsize: int | None = None) -> dict:
+    """Keys written at GPTQ/HLQ.py:177-193.  The exporter never writes
+    'groupsize' although the loader reads it (parameters.cpp:17); pass
+    groupsize to add it the way a fixed exporter would."""
+    cfg = {
+        "weight_data_len": int(k * n * bits // 8),
+        "base_bit": int(bits),
+        "use_sparse": False,
+        "in_channel": int(k),
+        "out_channel": int(n),
+        "has_bias": bool(has_bias),
+    }
+    if groupsize is not None:
+        cfg["groupsize"] = int(groupsize)
+    return cfg
+
+
+# --------------------------------------------------------------------------- #
+# a4: dequantize (GPTQ/quant.py:176-183) and the float64 matmul oracle
+# --------------------------------------------------------------------------- #
+def dequantize(w_quant: np.ndarray, w_scale: np.ndarray, w_zero: np.ndarray, group: int,
+               dtype=np.float64) -> np.ndarray:
+    """Export arrays -> dense W [N, K]:  W[n,k] = sum_b bit_b[n,k]*s[b,n,k//G] + z[n,k//G]."""
+    planes = unpack_planes(w_quant).astype(dtype)           # [B, N, K]
+    b, n, k = planes.shape
+    assert k % group == 0
+    s = np.repeat(np.asarray(w_scale).astype(dtype), group, axis=2)     # [B, N, K]
+    z = np.repeat(np.asarray(w_zero).astype(dtype), group, axis=1)      # [N, K]
+    return (planes * s).sum(axis=0) + z
+
+
+def gemv_f64(x, w_quant, w_scale, w_zero, group, bias=None) -> np.ndarray:
+    """y[n] = sum_k x[k] W[n,k] (+ bias) in float64 from fp16-valued inputs."""
+    w = dequantize(w_quant, w_scale, w_zero, group, np.float64)
+    y = w @ np.asarray(x).astype(np.float64).reshape(-1)
+    if bias is not None:
+        y = y + np.asarray(bias).astype(np.float64)
+    return y
+
+
+def gemm_f64(x, w_quant, w_scale, w_zero, group, bias=None) -> np.ndarray:
+    """x [M, K] -> y [M, N] in float64."""
+    w = dequantize(w_quant, w_scale, w_zero, group, np.float64)
+    y = np.asarray(x).astype(np.float64) @ w.T
+    if bias is not None:
+        y = y + np.asarray(bias).astype(np.float64)[None, :]
+    return y
+
+
+# --------------------------------------------------------------------------- #
+# a7: the loader's permutation (arm_t_mac_kernal.cpp:472-552)
+# --------------------------------------------------------------------------- #
+def rearrange_reference(w_quant, w_scale, w_zero, group: int, n_thread: int):
+    """Returns flat (weight u8, scale f16, zero f16) in the reference's run-time
+    layout: planes [thread][bit][tile32][K/8][32], scales [thread][bit][tile32][g][32],
+    zeros [tile32][g][32]."""
+    w_quant = np.asarray(w_quant, dtype=np.uint8)
+    w_scale = np.asarray(w_scale, dtype=np.float16)
+    w_zero = np.asarray(w_zero, dtype=np.float16)
+    bits, n, k8 = w_quant.shape
+    ng = w_zero.shape[1]
+    assert w_scale.shape == (bits, n, ng) and ng * group == k8 * 8
+    chunk = (n + n_thread - 1) // n_thread
+    wq, ws = [], []
+    for t in range(n_thread):
+        start, end = t * chunk, min((t + 1) * chunk, n)
+        if start >= end:
+            continue
+        assert (end - start) % 32 == 0, "reference requires 32-channel tiles per thread chunk"
+        for b in range(bits):
+            blk = w_quant[b, start:end].reshape(-1, 32, k8)        # [tile, r, kb]
+            wq.append(blk.transpose(0, 2, 1).reshape(-1))          # [tile, kb, r]
+    for t in range(n_thread):
+        start, end = t * chunk, min((t + 1) * chunk, n)
+        if start >= end:
+            continue
+        for b in range(bits):
+            blk = w_scale[b, start:end].reshape(-1, 32, ng)
+            ws.append(blk.transpose(0, 2, 1).reshape(-1))
+    wz = w_zero.reshape(-1, 32, ng).transpose(0, 2, 1).reshape(-1)
+    return np.concatenate(wq), np.concatenate(ws), np.ascontiguousarray(wz)
+
+
+# --------------------------------------------------------------------------- #
+# a8: fp16 LUT (arm_t_mac_kernal.cpp:95-138)
+# --------------------------------------------------------------------------- #
+def lut_float(x: np.ndarray) -> np.ndarray:
+    """x fp16 [K] -> fp16 [K/4, 16]; LUT[c][m] = sequential fp16 sum of x[4c+i]
+    over the set bits i of m in ascending i (temp[g] += activation[i+..])."""
+    x = np.asarray(x, dtype=np.float16).reshape(-1, 4)
+    lut = np.zeros((x.shape[0], 16), dtype=np.float16)
+    for m in range(16):
+        acc = np.zeros(x.shape[0], dtype=np.float16)
+        for i in range(4):
+            if m >> i & 1:
+                acc = (acc.astype(np.float32) + x[:, i].astype(np.float32)).astype(np.float16)
+        lut[:, m] = acc
+    return lut
+
+
+def _h(a):
+    return np.asarray(a, dtype=np.float32).astype(np.float16)
+
+
+def _mac16(acc, a, b, fused):
+    """fp16 acc + a*b: one rounding if fused (fmla), two otherwise."""
+    if fused:
+        return (acc.astype(np.float64) + a.astype(np.float64) * b.astype(np.float64)).astype(np.float16)
+    prod = (a.astype(np.float32) * b.astype(np.float32)).astype(np.float16)
+    return (acc.astype(np.float32) + prod.astype(np.float32)).astype(np.float16)
+
+
+# --------------------------------------------------------------------------- #
+# a9/a10: the live fp16 GEMV chain (arm_gemm.cpp:248-308, kernal.cpp:364-469)
+# --------------------------------------------------------------------------- #
+def gemv_fp16_chain(x, w_quant, w_scale, w_zero, group, bias=None, fused=True) -> np.ndarray:
+    """Follows the reference op for op with every fp16 rounding point:
+       xs[g]  sequential fp16 sum of the group's activations
+       y[n]   sequential over g of fp16 (y + xs[g]*z[n,g])
+       per plane: acc_g sequential fp16 sum of LUT[lo nibble] then LUT[hi nibble] per byte;
+                  c = acc_0*s_0, then c += acc_g*s_g;  y = fp16(y + c)
+       y += bias.
+    'fused' selects fmla (one rounding per multiply-add), which is what
+    -O3 -ffp-contract=fast yields for `v += a*b` on float16x8_t."""
+    x = np.asarray(x, dtype=np.float16).reshape(-1)
+    w_quant = np.asarray(w_quant, dtype=np.uint8)
+    w_scale = np.asarray(w_scale, dtype=np.float16)
+    w_zero = np.asarray(w_zero, dtype=np.float16)
+    bits, n, k8 = w_quant.shape
+    k = k8 * 8
+    ng = k // group
+    xs = np.zeros(ng, dtype=np.float16)
+    for g in range(ng):
+        a = np.float16(0)
+        for j in range(group):
+            a = np.float16(np.float32(a) + np.float32(x[g * group + j]))
+        xs[g] = a
+    y = np.zeros(n, dtype=np.float16)
+    for g in range(ng):
+        y = _mac16(y, np.full(n, xs[g], dtype=np.float16), w_zero[:, g], fused)
+    lut = lut_float(x)
+    for b in range(bits):
+        c = None
+        for g in range(ng):
+            acc = np.zeros(n, dtype=np.float16)
+            for l in range(0, group, 8):
+                byte = w_quant[b, :, (g * group + l) // 8]
+                c0 = (g * group + l) // 4
+                acc = _h(acc.astype(np.float32) + lut[c0, byte & 15].astype(np.float32))
+                acc = _h(acc.astype(np.float32) + lut[c0 + 1, byte >> 4].astype(np.float32))
+            if g == 0:
+                c = _h(acc.astype(np.float32) * w_scale[b, :, 0].astype(np.float32))
+            else:
+                c = _mac16(c, acc, w_scale[b, :, g], fused)
+        y = _h(y.astype(np.float32) + c.astype(np.float32))
+    if bias is not None:
+        y = _h(y.astype(np.float32) + np.asarray(bias, dtype=np.float16).astype(np.float32))
+    return y
+
+
+def gemm_rows(x, w_quant, w_scale, w_zero, group, bias=None, fused=True) -> np.ndarray:
+    """m > 1 in the reference is a row loop over the GEMV (arm_gemm.cpp:380-385)."""
+    x = np.asarray(x, dtype=np.float16)
+    return np.stack([gemv_fp16_chain(r, w_quant, w_scale, w_zero, group, bias, fused) for r in x])
+
+
+# --------------------------------------------------------------------------- #
+# tolerance metric used by every parity test
+# --------------------------------------------------------------------------- #
+def rel_err(y, ref, floor_frac: float = 0.05) -> float:
+    """max_i |y_i - ref_i| / max(|ref_i|, floor_frac * rms(ref)).
+
+    The floor keeps outputs that cross zero from dominating: without it a
+    correctly rounded fp16 result next to 0 has unbounded relative error."""
+    y = np.asarray(y, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    rms = float(np.sqrt(np.mean(ref * ref))) if ref.size else 0.0
+    den = np.maximum(np.abs(ref), max(floor_frac * rms, 1e-30))
+    return float(np.max(np.abs(y - ref) / den)) if ref.size else 0.0

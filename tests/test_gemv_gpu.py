@@ -1,0 +1,165 @@
+"""GPU parity of the HIP LUT GEMV (through the C ABI) against the CPU oracle.
+
+Tolerances (fp16 outputs):
+  * vs the float64 dequantize-then-matmul oracle:  rel_err <= 1e-2 with
+    rel_err = max_i |y_i - ref_i| / max(|ref_i|, 0.05 rms(ref))   (oracle.hlq_oracle.rel_err);
+  * vs the C restatement of the reference's all-fp16 chain: max|y - y_ref| <= 2e-2 rms,
+    the reference chain itself being that far from the exact result;
+  * bit-exact where the arithmetic is exact (integer-valued inputs, unit vectors).
+"""
+import numpy as np
+import pytest
+import torch
+
+from elutq_amd.hlq_linear import HLQLinear
+from elutq_amd.synth import LLAMA3_8B_SHAPES, make_layer
+from oracle import hlq_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def to_mod(L, dev, ksplit=0, waves=0):
+    m = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, L.group, L.bias, dev)
+    m.ksplit, m.waves = ksplit, waves
+    return m
+
+
+def run(m, x, dev):
+    y = m(torch.from_numpy(np.ascontiguousarray(x)).to(dev))
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("k,n,bits,group", [
+    (256, 64, 2, 128), (512, 128, 2, 128), (1024, 256, 3, 128), (1024, 192, 2, 64),
+    (384, 70, 2, 128), (128, 1, 1, 128), (640, 100, 4, 64), (2048, 512, 4, 128), (384, 64, 3, 64),
+])
+@pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 1), (1, 4), (2, 2), (3, 8)])
+def test_gemv_matches_oracle(cuda, k, n, bits, group, ksplit, waves):
+    L = make_layer(k, n, bits=bits, group=group, seed=k + n + bits, bias=(n % 3 == 0))
+    nt = (k // group + 1) // 2
+    ks = min(ksplit, nt)
+    y = run(to_mod(L, cuda, ks, waves), L.x, cuda)[0]
+    ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, group, L.bias)
+    assert y.shape == (n,) and y.dtype == np.float16
+    assert O.rel_err(y, ref) <= TOL, (k, n, bits, group, ks, waves)
+    # exact integer tables + fp32 accumulation: only the final fp16 rounding is left
+    assert np.max(np.abs(y.astype(np.float64) - ref)) <= 2.0 ** -10 * max(1.0, np.max(np.abs(ref)))
+
+
+@pytest.mark.parametrize("bits,group", [(2, 128), (3, 128), (2, 64)])
+def test_gemv_close_to_reference_fp16_chain(cuda, lutref, bits, group):
+    L = make_layer(1024, 256, bits=bits, group=group, seed=21, bias=True)
+    y = run(to_mod(L, cuda), L.x, cuda)[0].astype(np.float64)
+    yref = lutref.RefWeight(L.w_quant, L.w_scale, L.w_zero, group, 4, L.bias).gemv(L.x[0]).astype(np.float64)
+    rms = np.sqrt(np.mean(yref ** 2))
+    assert np.max(np.abs(y - yref)) <= 2e-2 * rms
+
+
+@pytest.mark.parametrize("bits,group,ksplit", [(2, 128, 1), (2, 128, 2), (3, 64, 0), (4, 128, 3)])
+def test_gemv_bit_exact_on_integer_inputs(cuda, lutref, bits, group, ksplit):
+    """x in {-2..2}, power-of-two scales, quarter-integer zeros: every partial sum is exactly
+    representable, so GPU == float64 == the reference's fp16 chain, bit for bit."""
+    r = np.random.default_rng(5)
+    k, n = 768, 128
+    x = r.integers(-2, 3, (1, k)).astype(np.float16)
+    wq = O.pack_planes(r.integers(0, 2, (bits, n, k), dtype=np.uint8))
+    ws = np.stack([np.full((n, k // group), 2.0 ** (b - 3), np.float16) for b in range(bits)])
+    wz = (r.integers(-3, 1, (n, k // group)) / 4).astype(np.float16)
+    y64 = O.gemv_f64(x[0], wq, ws, wz, group)
+    m = HLQLinear.from_export_arrays(wq, ws, wz, group, None, cuda)
+    m.ksplit = ksplit
+    y = run(m, x, cuda)[0]
+    assert np.array_equal(y.astype(np.float64), y64)
+    yc = lutref.RefWeight(wq, ws, wz, group, 4).gemv(x[0])
+    assert np.array_equal(y.view(np.uint16), yc.view(np.uint16))
+
+
+def test_gemv_closed_forms(cuda):
+    L = make_layer(512, 128, bits=2, group=128, seed=31)
+    x64 = L.x[0].astype(np.float64)
+    xs = x64.reshape(-1, 128).sum(1)
+    z, s = L.w_zero.astype(np.float64), L.w_scale.astype(np.float64)
+    zero = HLQLinear.from_export_arrays(np.zeros_like(L.w_quant), L.w_scale, L.w_zero, 128, None, cuda)
+    assert O.rel_err(run(zero, L.x, cuda)[0], z @ xs) <= 2e-3
+    ones = HLQLinear.from_export_arrays(np.full_like(L.w_quant, 255), L.w_scale, L.w_zero, 128, None, cuda)
+    assert O.rel_err(run(ones, L.x, cuda)[0], (s.sum(0) + z) @ xs) <= 2e-3
+    # x = e_k returns column k of W, rounded once to fp16
+    m = to_mod(L, cuda)
+    w = O.dequantize(L.w_quant, L.w_scale, L.w_zero, 128)
+    for kk in (0, 127, 128, 300, 511):
+        e = np.zeros((1, 512), np.float16)
+        e[0, kk] = 1
+        y = run(m, e, cuda)[0]
+        assert np.array_equal(y, w[:, kk].astype(np.float32).astype(np.float16)), kk
+
+
+def test_gemv_linearity_scaling_and_determinism(cuda):
+    L = make_layer(1024, 256, bits=2, group=128, seed=41)
+    m = to_mod(L, cuda)
+    y1 = run(m, L.x, cuda)
+    assert np.array_equal(y1, run(m, L.x, cuda))              # same bits run to run
+    y2 = run(m, (L.x * np.float16(4)).astype(np.float16), cuda)   # power-of-two scaling is exact
+    ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, 128)
+    assert O.rel_err(y2[0], 4 * ref) <= 2e-3
+    # tiny and large activations (per-unit power-of-two table scale)
+    for f in (2.0 ** -10, 2.0 ** 8):
+        xf = (L.x.astype(np.float32) * f).astype(np.float16)
+        r = O.gemv_f64(xf[0], L.w_quant, L.w_scale, L.w_zero, 128)
+        assert O.rel_err(run(m, xf, cuda)[0], r) <= 2e-3
+    # a unit of exact zeros next to live units
+    xz = L.x.copy()
+    xz[0, 128:256] = 0
+    assert O.rel_err(run(m, xz, cuda)[0], O.gemv_f64(xz[0], L.w_quant, L.w_scale, L.w_zero, 128)) <= 2e-3
+
+
+def test_gemv_wide_dynamic_range_in_one_unit(cuda):
+    """One activation 2^13 times the rest: the small ones are still summed exactly
+    (fixed point covers 2^-13 max|x| without rounding)."""
+    L = make_layer(256, 64, bits=2, group=128, seed=43)
+    x = (L.x.astype(np.float32) * 2.0 ** -6).astype(np.float16)
+    x[0, 5] = np.float16(64.0)
+    y = run(to_mod(L, cuda), x, cuda)[0]
+    assert O.rel_err(y, O.gemv_f64(x[0], L.w_quant, L.w_scale, L.w_zero, 128)) <= 2e-3
+
+
+def test_rows_are_gemvs_and_leading_dims(cuda):
+    L = make_layer(512, 192, bits=3, group=128, m=6, seed=51, bias=True)
+    m = to_mod(L, cuda)
+    y = run(m, L.x, cuda)
+    ref = O.gemm_f64(L.x, L.w_quant, L.w_scale, L.w_zero, 128, L.bias)
+    assert y.shape == (6, 192) and O.rel_err(y, ref) <= TOL
+    y3 = m(torch.from_numpy(L.x).to(cuda).reshape(2, 3, 512))
+    assert y3.shape == (2, 3, 192) and np.array_equal(y3.cpu().numpy().reshape(6, 192), y)
+    assert m(torch.empty(0, 512, dtype=torch.float16, device=cuda)).shape == (0, 192)
+    with pytest.raises(ValueError):
+        m(torch.zeros(1, 256, dtype=torch.float16, device=cuda))
+
+
+def test_dequantize_matches_oracle(cuda):
+    for bits, group, n in ((2, 128, 64), (3, 64, 70), (4, 128, 130)):
+        L = make_layer(384, n, bits=bits, group=group, seed=61)
+        w = to_mod(L, cuda).dequantize().cpu().numpy()
+        planes = O.unpack_planes(L.w_quant).astype(np.float32)
+        v = np.repeat(L.w_zero.astype(np.float32), group, axis=1)
+        for b in range(bits):                                    # fp32, plane order, one final rounding
+            v = v + planes[b] * np.repeat(L.w_scale[b].astype(np.float32), group, axis=1)
+        assert np.array_equal(w, v.astype(np.float16))
+
+
+@pytest.mark.parametrize("name", ["q_proj", "k_proj", "gate_proj", "down_proj"])
+@pytest.mark.parametrize("bits,group", [(2, 128), (3, 128), (2, 64)])
+def test_llama3_8b_shapes_full_size(cuda, name, bits, group):
+    """BASELINE shapes at full size: oracle comparison plus size-independent properties."""
+    k, n = LLAMA3_8B_SHAPES[name]
+    L = make_layer(k, n, bits=bits, group=group, seed=7)
+    m = to_mod(L, cuda)
+    y = run(m, L.x, cuda)[0]
+    w = O.dequantize(L.w_quant, L.w_scale, L.w_zero, group, np.float32)
+    ref = w.astype(np.float64) @ L.x[0].astype(np.float64)
+    assert O.rel_err(y, ref) <= TOL
+    assert np.array_equal(y, run(m, L.x, cuda)[0])
+    # y(x) + y(-x) == 0 exactly (integer tables negate exactly, fp32 sums are sign symmetric)
+    yn = run(m, (-L.x).astype(np.float16), cuda)[0]
+    assert np.array_equal(yn.view(np.uint16) ^ 0x8000, y.view(np.uint16)) or np.array_equal(-yn, y)

@@ -1,0 +1,132 @@
+"""CPU-only tests of the host side: the C-ABI library loads and exports every symbol the
+header declares, the host repack is a bijection with the documented layout, the export
+directory reader/writer round-trips, and argument checks return the documented codes.
+No GPU compute is called here."""
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+from elutq_amd import _lib
+from elutq_amd.export_io import read_export_dir, write_export_dir
+from elutq_amd.hlq_linear import repack_export_arrays, unpack_to_export_arrays
+from elutq_amd.synth import algorithmic_bytes, make_layer
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "elutq_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(elutq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = header_symbols()
+    assert "elutq_hlq_gemv_f16" in names and "elutq_hlq_repack_host" in names and len(names) >= 12
+    L = _lib.lib()
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in include/elutq_hip.h but not exported"
+    assert set(names) == set(_lib.SIGNATURES), "ctypes table and header disagree"
+    assert L.elutq_version() >= 100
+    assert L.elutq_status_string(0) == b"ok"
+    assert b"group" in L.elutq_status_string(-4)
+
+
+def test_size_queries_and_argument_errors():
+    L = _lib.lib()
+    assert L.elutq_hlq_planes_bytes(4096, 4096, 2) == 4096 * 4096 * 2 // 8
+    assert L.elutq_hlq_scales_bytes(4096, 4096, 2, 128) == 2 * 2 * 4096 * 32
+    assert L.elutq_hlq_zeros_bytes(4096, 4096, 128) == 2 * 4096 * 32
+    # columns are padded to 64, an odd number of groups to an even one
+    assert L.elutq_hlq_planes_bytes(384, 70, 3) == 128 * 3 * 3 * 16 * 8 // 8
+    assert L.elutq_hlq_zeros_bytes(384, 70, 128) == 128 * 2 * 4
+    assert L.elutq_hlq_planes_bytes(100, 64, 2) == 0          # K % 128
+    assert L.elutq_hlq_workspace_bytes(4096, 4096, 2, 32, 1) == 0
+    assert L.elutq_hlq_workspace_bytes(4096, 4096, 2, 128, 1) >= 64 * 1024
+    one = ctypes.c_void_p(1)
+    g = lambda K, N, b, G: L.elutq_hlq_gemv_f16(one, one, one, None, one, one, K, N, b, G, None, 0, None)
+    assert g(4096, 64, 5, 128) == -3
+    assert g(4096, 64, 2, 32) == -4
+    assert g(4000, 64, 2, 128) == -2
+    assert g(4096, 0, 2, 128) == -2
+    assert L.elutq_hlq_gemv_f16(None, one, one, None, one, one, 4096, 64, 2, 128, None, 0, None) == -1
+    assert L.elutq_hlq_gemm_f16(one, one, one, None, one, one, 0, 4096, 64, 2, 128, None, 0, None) == -2
+    assert L.elutq_hlq_repack_host(None, None, None, 128, 64, 2, 128, None, None, None) == -1
+    with pytest.raises(_lib.ElutqError, match="group must be 64 or 128"):
+        _lib.check(-4, "t")
+
+
+@pytest.mark.parametrize("k,n,bits,group", [(256, 64, 2, 128), (384, 70, 3, 128), (128, 1, 1, 64),
+                                             (512, 200, 4, 64), (1024, 128, 2, 64)])
+def test_repack_roundtrip_and_layout(k, n, bits, group):
+    L = make_layer(k, n, bits=bits, group=group, seed=3)
+    planes, scales, zeros = repack_export_arrays(L.w_quant, L.w_scale, L.w_zero, group)
+    wq, ws, wz = unpack_to_export_arrays(planes, scales, zeros, k, n, bits, group)
+    assert np.array_equal(wq, L.w_quant)
+    assert np.array_equal(ws.view(np.uint16), L.w_scale.view(np.uint16))
+    assert np.array_equal(wz.view(np.uint16), L.w_zero.view(np.uint16))
+    # documented layout, checked independently of the library's inverse:
+    ncb, U, NG = (n + 63) // 64, k // 128, k // group
+    NT = (NG + 1) // 2
+    p = planes.view(np.uint32).reshape(ncb, U, bits, 64, 4)
+    rot = lambda v, r: ((int(v) >> r) | (int(v) << (32 - r))) & 0xFFFFFFFF
+    rs = np.random.default_rng(0)
+    for _ in range(50):
+        col, u, b, d, i = rs.integers(n), rs.integers(U), rs.integers(bits), rs.integers(4), rs.integers(32)
+        kk = u * 128 + d * 32 + i
+        want = (L.w_quant[b, col, kk // 8] >> (kk % 8)) & 1
+        natural = rot(p[col // 64, u, b, col % 64, d], 2)          # undo the rotate-left by 2
+        assert (natural >> i) & 1 == want
+    s = scales.view(np.uint16).reshape(ncb, NT, bits, 64, 2)
+    z = zeros.view(np.uint16).reshape(ncb, NT, 64, 2)
+    for _ in range(50):
+        col, g, b = rs.integers(n), rs.integers(NG), rs.integers(bits)
+        assert s[col // 64, g // 2, b, col % 64, g % 2] == L.w_scale.view(np.uint16)[b, col, g]
+        assert z[col // 64, g // 2, col % 64, g % 2] == L.w_zero.view(np.uint16)[col, g]
+    # padding columns are zero
+    if n % 64:
+        assert not p[-1, :, :, n % 64:, :].any() and not s[-1, :, :, n % 64:, :].any()
+
+
+def test_repack_rejects_bad_shapes():
+    L = make_layer(256, 64, seed=1)
+    with pytest.raises(ValueError):
+        repack_export_arrays(L.w_quant, L.w_scale, L.w_zero, 64)       # wrong group for these scales
+    with pytest.raises(ValueError):
+        repack_export_arrays(L.w_quant[:, :, :8], L.w_scale[:, :, :1], L.w_zero[:, :1], 64)   # K = 64
+
+
+def test_export_dir_roundtrip(tmp_path):
+    L = make_layer(256, 96, bits=3, group=64, seed=5, bias=True)
+    d = tmp_path / "0" / "self_attn.q_proj"
+    write_export_dir(str(d), L.w_quant, L.w_scale, L.w_zero, L.bias)
+    cfg = json.load(open(d / "weight_config.json"))
+    assert cfg == {"weight_data_len": 256 * 96 * 3 // 8, "base_bit": 3, "use_sparse": False,
+                   "in_channel": 256, "out_channel": 96, "has_bias": True}       # no groupsize key
+    assert os.path.getsize(d / "w_quant.bin") == 256 * 96 * 3 // 8
+    assert os.path.getsize(d / "w_scale.bin") == 2 * 3 * 96 * 4
+    assert os.path.getsize(d / "w_zero.bin") == 2 * 96 * 4
+    e = read_export_dir(str(d))                      # group derived from the w_zero.bin size
+    assert (e.k, e.n, e.bits, e.group) == (256, 96, 3, 64)
+    assert np.array_equal(e.w_quant, L.w_quant) and np.array_equal(e.w_scale, L.w_scale)
+    assert np.array_equal(e.w_zero, L.w_zero) and np.array_equal(e.bias, L.bias)
+    write_export_dir(str(d), L.w_quant, L.w_scale, L.w_zero, None, groupsize=64)
+    assert read_export_dir(str(d)).group == 64 and read_export_dir(str(d)).bias is None
+    # truncated file -> error, not garbage
+    with open(d / "w_scale.bin", "r+b") as f:
+        f.truncate(10)
+    with pytest.raises(ValueError):
+        read_export_dir(str(d))
+
+
+def test_algorithmic_bytes_table():
+    assert algorithmic_bytes(4096, 4096, 2, 128) == 4_997_120
+    assert algorithmic_bytes(4096, 1024, 2, 128) == 1_255_424
+    assert algorithmic_bytes(4096, 14336, 2, 128) == 17_469_440
+    assert algorithmic_bytes(14336, 4096, 2, 128) == 17_469_440
+    assert algorithmic_bytes(4096, 4096, 3, 128) == 7_356_416
+    assert algorithmic_bytes(4096, 4096, 2, 64) == 5_783_552
