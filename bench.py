@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Benchmark of the HLQ LUT GEMV hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-decode]
+
+Workload (BASELINE config 2): the LLaMA-3-8B layer-shape sweep at HLQ w2g128, batch 1.
+One "step" streams the seven projections (q, k, v, o, gate, up, down) of all 32 layers --
+224 GEMVs over 224 distinct random weight sets, 2.07 GB of packed planes + scales + zeros,
+far more than the 256 MB Infinity Cache, so every step reads its weights from HBM.  Inputs
+are resident in HBM before the timed region.  The step is captured once in a HIP graph and
+replayed, so the figure is GPU throughput, not Python launch rate.
+
+Prints ONE JSON line.  `value` is algorithmic bytes per step / time per step in GB/s
+(bytes = planes + fp16 scales + fp16 zeros + x + y per GEMV).  `per_shape` holds the
+per-shape latency / bandwidth of the four distinct (K, N), each measured over a ring of
+weight sets larger than 512 MB.  `roofline` is for the dominant kernel (the 4096x14336
+gate/up GEMV); `cpu_baseline` times the C port of the reference's CPU LUT kernel
+(oracle/lut_gemv_ref.c, AVX2 build) on this machine's host cores over a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+BITS, GROUP = 2, 128
+N_LAYERS = 32
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    p.add_argument("--no-decode", action="store_true", help="skip the decode tokens/s leg")
+    p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    return p.parse_args()
+
+
+class Gemv:
+    """Direct C-ABI launcher on preallocated buffers (no allocation in the timed loop)."""
+
+    def __init__(self, lib, mod, x, y, ws):
+        self.lib, self.mod, self.x, self.y, self.ws = lib, mod, x, y, ws
+        self.args = (mod.planes.data_ptr(), mod.scales.data_ptr(), mod.zeros.data_ptr(), None,
+                     x.data_ptr(), y.data_ptr(), mod.in_features, mod.out_features, mod.bits,
+                     mod.group_size, ws.data_ptr(), ws.numel())
+
+    def __call__(self, stream):
+        rc = self.lib.elutq_hlq_gemv_f16(*self.args, stream)
+        if rc:
+            raise RuntimeError(f"elutq_hlq_gemv_f16 failed: {rc}")
+
+
+def time_graph(torch, launch_all, replays, warmup):
+    """Captures launch_all(stream) once, replays it; returns seconds per replay (HIP events on
+    the replay stream)."""
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        launch_all(s.cuda_stream)            # eager warm-up on the capture stream
+    s.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        launch_all(torch.cuda.current_stream().cuda_stream)
+    for _ in range(warmup):
+        g.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        g.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / replays
+
+
+def cpu_baseline(budget_s):
+    """C port of the reference CPU LUT GEMV (AVX2 pshufb lookups, fp32 accumulation) on the
+    host cores: one layer's seven GEMVs, repeated within the time budget."""
+    import numpy as np
+    from elutq_amd.synth import LLAMA3_8B_SHAPES, algorithmic_bytes, make_layer
+    from oracle import lutref
+    if not os.path.exists(os.path.join(ROOT, "oracle", "liblutref.so")):
+        lutref.build()
+    ncpu = os.cpu_count() or 1
+    out = {}
+    weights = {}
+    for (k, n) in sorted(set(LLAMA3_8B_SHAPES.values())):
+        weights[(k, n)] = make_layer(k, n, bits=BITS, group=GROUP, seed=k + n)
+    for threads in sorted({4, min(16, ncpu)}):
+        refs = {kn: lutref.RefWeight(L.w_quant, L.w_scale, L.w_zero, GROUP, threads) for kn, L in weights.items()}
+        seq = [(refs[kn], weights[kn].x[0]) for kn in LLAMA3_8B_SHAPES.values()]
+        nbytes = sum(algorithmic_bytes(k, n, BITS, GROUP) for (k, n) in LLAMA3_8B_SHAPES.values())
+        for rw, x in seq:
+            rw.gemv_fast(x)
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            for rw, x in seq:
+                rw.gemv_fast(x)
+            reps += 1
+            if time.perf_counter() - t0 > budget_s / 2:
+                break
+        dt = (time.perf_counter() - t0) / reps
+        out[threads] = {"GBps": nbytes / dt / 1e9, "ms_per_layer": dt * 1e3, "reps": reps}
+    return out, ncpu
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print(f"bench.py: this build measures ONE GPU (the path needs no collective); --gpus {a.gpus} is not supported",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    from elutq_amd import _lib
+    from elutq_amd.synth import LLAMA3_8B_SHAPES, algorithmic_bytes, make_device_layer
+
+    lib = _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    ws_bytes = max(lib.elutq_hlq_workspace_bytes(k, n, BITS, GROUP, 1) for (k, n) in LLAMA3_8B_SHAPES.values())
+    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+    xs = {k: torch.randn(1, k, device=dev).to(torch.float16) for k in {k for k, _ in LLAMA3_8B_SHAPES.values()}}
+    ys = {n: torch.empty(1, n, dtype=torch.float16, device=dev) for n in {n for _, n in LLAMA3_8B_SHAPES.values()}}
+
+    # ---- the sweep: 32 layers x 7 projections, all weight sets distinct -----------------
+    calls = []
+    step_bytes = 0
+    seed = 0
+    for layer in range(N_LAYERS):
+        for name, (k, n) in LLAMA3_8B_SHAPES.items():
+            mod = make_device_layer(k, n, BITS, GROUP, seed=seed, device=dev)
+            seed += 1
+            calls.append(Gemv(lib, mod, xs[k], ys[n], ws))
+            step_bytes += algorithmic_bytes(k, n, BITS, GROUP)
+    torch.cuda.synchronize()
+
+    def launch_step(stream):
+        for c in calls:
+            c(stream)
+
+    sec_step = time_graph(torch, launch_step, a.steps, a.warmup)
+    value = step_bytes / sec_step / 1e9
+
+    # ---- per shape, each over a ring of weight sets > 512 MB ------------------------------
+    per_shape = {}
+    by_shape = {}
+    for c in calls:
+        by_shape.setdefault((c.mod.in_features, c.mod.out_features), []).append(c)
+    for (k, n), lst in sorted(by_shape.items()):
+        nbytes = algorithmic_bytes(k, n, BITS, GROUP)
+        need = -(-512 * 2 ** 20 // nbytes)
+        extra = []
+        while len(lst) + len(extra) < need:
+            mod = make_device_layer(k, n, BITS, GROUP, seed=10_000 + len(extra) + k, device=dev)
+            extra.append(Gemv(lib, mod, xs[k], ys[n], ws))
+        ring = lst + extra
+
+        def launch_ring(stream, ring=ring):
+            for c in ring:
+                c(stream)
+
+        reps = max(3, min(a.steps, int(20000 / len(ring)) + 1))
+        sec = time_graph(torch, launch_ring, reps, 2) / len(ring)
+        per_shape[f"{k}x{n}"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                                 "bytes": nbytes, "ring_sets": len(ring)}
+        del extra, ring
+        torch.cuda.empty_cache()
+
+    dom = per_shape["4096x14336"]
+    roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": dom["GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                "kernel": "hlq_gemv_kernel<2,false> K=4096 N=14336", "us_per_launch": dom["us"],
+                "bytes_per_launch": dom["bytes"]}
+
+    out = {
+        "metric": "LUT-GEMV HBM GB/s at LLaMA3-8B shapes bs1 (HLQ w2g128)",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": sec_step * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 activations, int32 fixed-point tables, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "LLaMA-3-8B layer-shape sweep, HLQ w2g128, batch 1: 32 layers x (q,k,v,o,gate,up,down) = 224 GEMVs over distinct weights per step",
+                   "bits": BITS, "group": GROUP, "bytes_per_step": step_bytes, "gemvs_per_step": len(calls)},
+        "frac_hbm_peak": value / HBM_PEAK_GBPS,
+        "per_shape": per_shape,
+        "roofline": roofline,
+    }
+
+    if not a.no_decode:
+        try:
+            from elutq_amd.llama_decode import bench_decode
+            out["decode"] = bench_decode(dev)
+        except ImportError:
+            out["decode"] = None
+
+    if not a.no_cpu:
+        res, ncpu = cpu_baseline(a.cpu_seconds)
+        tmax = max(res)
+        out["cpu_baseline"] = {"value": res[tmax]["GBps"], "unit": "GB/s", "cores": tmax, "kind": "port",
+                               "sample": f"one layer (7 GEMVs, {res[tmax]['reps']} repeats) of the same sweep, AVX2 port of the reference kernel with fp32 accumulators, {tmax} OpenMP threads of {ncpu} host CPUs",
+                               "ms_per_layer": res[tmax]["ms_per_layer"],
+                               "at_4_threads_GBps": res[4]["GBps"] if 4 in res else None}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -28,6 +28,7 @@
 
 namespace {
 
+constexpr int MAX_LDS = 160 * 1024;
 constexpr int TBL_BYTES = 64;                    // 16 int32 entries
 constexpr int UNIT_LUT_BYTES = 32 * TBL_BYTES;   // 32 chunks per unit
 
@@ -41,8 +42,19 @@ struct GemvArgs {
     float *partial;          // [ksplit][ncb*64]   (ksplit > 1)
     unsigned *counters;      // [ncb], zero between calls
     int N, U, NT, ncb;
-    int ksplit, tps;         // slices per column block, tasks per slice
+    int ksplit, ups;         // slices per column block, units per slice
 };
+
+#ifdef HLQ_TIMING
+// Profiling builds only: per-stage wall-clock stamps (100 MHz) of wave 0 of every workgroup.
+__device__ unsigned long long *g_hlq_stamps = nullptr;
+#define HLQ_STAMP(i)                                                                              \
+    do {                                                                                          \
+        if (g_hlq_stamps && threadIdx.x == 0) g_hlq_stamps[(size_t)blockIdx.x * 8 + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define HLQ_STAMP(i) do { } while (0)
+#endif
 
 typedef __attribute__((address_space(3))) const int lds_cint;
 
@@ -90,100 +102,85 @@ __device__ __forceinline__ int lookup_dword(uint32_t w, uint32_t (&a)[8], uint32
     return acc;
 }
 
-template <int BITS, bool G64>
-struct Task {
-    static constexpr int UPT = G64 ? 1 : 2;
-    uint4 w[UPT][BITS];
-    uint32_t sc[BITS];
-    uint32_t zz;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// A sub-task is one unit of one plane: 128 k of 64 columns = one dwordx4 per lane, plus the
+// meta dword(s) that scale it.
+struct Sub {
+    uint4 w;
+    uint32_t sc;   // fp16 scales of the group pair this unit belongs to (this plane)
+    uint32_t zz;   // fp16 zeros of the pair; loaded for plane 0 only, which folds the zero point
 };
 
 template <int BITS, bool G64>
-__device__ __forceinline__ void load_task(Task<BITS, G64> &t, const GemvArgs &a, int cb, int task, int lane)
+__device__ __forceinline__ void load_sub(Sub &t, const GemvArgs &a, int cb, int u, int b, int lane)
 {
-    constexpr int UPT = Task<BITS, G64>::UPT;
-#pragma unroll
-    for (int ul = 0; ul < UPT; ul++) {
-        const int u = task * UPT + ul;
-        if (u < a.U) {
-            const uint4 *p = a.planes + (((size_t)cb * a.U + u) * BITS) * HLQ_CB + lane;
-#pragma unroll
-            for (int b = 0; b < BITS; b++) t.w[ul][b] = p[b * HLQ_CB];
-        } else {
-#pragma unroll
-            for (int b = 0; b < BITS; b++) t.w[ul][b] = make_uint4(0, 0, 0, 0);
-        }
-    }
-    const size_t m = (size_t)cb * a.NT + task;
-#pragma unroll
-    for (int b = 0; b < BITS; b++) t.sc[b] = a.scales[(m * BITS + b) * HLQ_CB + lane];
-    t.zz = a.zeros[m * HLQ_CB + lane];
+    const u32x4 v = __builtin_nontemporal_load((const u32x4 *)(a.planes + (((size_t)cb * a.U + u) * BITS + b) * HLQ_CB + lane));
+    t.w = make_uint4(v.x, v.y, v.z, v.w);
+    const size_t m = (size_t)cb * a.NT + (G64 ? u : (u >> 1));
+    t.sc = a.scales[(m * BITS + b) * HLQ_CB + lane];
+    t.zz = 0;
+    if (b == 0) t.zz = a.zeros[m * HLQ_CB + lane];
 }
 
-// One unit (128 k of 64 columns, all planes).  `lu` = unit index inside the slice.
-template <int BITS, bool G64, int HALF>
-__device__ __forceinline__ float process_unit(const uint4 (&w)[BITS], const uint32_t (&sc)[BITS], uint32_t zz,
-                                              int lu, uint32_t lut_base, const float *xs, const float *invs,
-                                              uint32_t mask, float acc)
+// The two 64-k halves of a unit have their own table scale (2^-p) and activation sum; at
+// G = 64 they are also two quantization groups (lo / hi half of the meta dwords), at G = 128
+// one group (the half of the meta dwords selected by the unit's parity).
+template <bool G64>
+__device__ __forceinline__ float process_sub(const Sub &t, int lu, int b, int odd, uint32_t lut_base,
+                                             const float2 *xs_inv, uint32_t mask, float acc)
 {
     uint32_t a[8];
     const uint32_t ub = lut_base + (uint32_t)lu * UNIT_LUT_BYTES;
 #pragma unroll
     for (int j = 0; j < 8; j++) a[j] = ub;
-    const float inv = invs[lu];
-    if (G64) {
-        float p0 = 0.f, p1 = 0.f;
-#pragma unroll
-        for (int b = 0; b < BITS; b++) {
-            int i0 = lookup_dword<0>(w[b].x, a, mask, 0);
-            i0 = lookup_dword<1>(w[b].y, a, mask, i0);
-            int i1 = lookup_dword<2>(w[b].z, a, mask, 0);
-            i1 = lookup_dword<3>(w[b].w, a, mask, i1);
-            p0 = fmaf((float)i0, h2f_lo(sc[b]), p0);
-            p1 = fmaf((float)i1, h2f_hi(sc[b]), p1);
-        }
-        acc = fmaf(inv, p0 + p1, acc);
-        acc = fmaf(h2f_lo(zz), xs[2 * lu], acc);
-        acc = fmaf(h2f_hi(zz), xs[2 * lu + 1], acc);
-    } else {
-        float p = 0.f;
-#pragma unroll
-        for (int b = 0; b < BITS; b++) {
-            int i0 = lookup_dword<0>(w[b].x, a, mask, 0);
-            i0 = lookup_dword<1>(w[b].y, a, mask, i0);
-            i0 = lookup_dword<2>(w[b].z, a, mask, i0);
-            i0 = lookup_dword<3>(w[b].w, a, mask, i0);
-            p = fmaf((float)i0, HALF ? h2f_hi(sc[b]) : h2f_lo(sc[b]), p);
-        }
-        acc = fmaf(inv, p, acc);
-        acc = fmaf(HALF ? h2f_hi(zz) : h2f_lo(zz), xs[lu], acc);
+    const float2 h0 = xs_inv[2 * lu], h1 = xs_inv[2 * lu + 1];      // .x = sum of x, .y = 2^-p
+    int i0 = lookup_dword<0>(t.w.x, a, mask, 0);
+    i0 = lookup_dword<1>(t.w.y, a, mask, i0);
+    int i1 = lookup_dword<2>(t.w.z, a, mask, 0);
+    i1 = lookup_dword<3>(t.w.w, a, mask, i1);
+    const uint32_t sc = G64 ? t.sc : (odd ? (t.sc >> 16) * 0x10001u : (t.sc & 0xffffu) * 0x10001u);
+    acc = fmaf((float)i0 * h0.y, h2f_lo(sc), acc);
+    acc = fmaf((float)i1 * h1.y, h2f_hi(sc), acc);
+    if (b == 0) {
+        const uint32_t zz = G64 ? t.zz : (odd ? (t.zz >> 16) * 0x10001u : (t.zz & 0xffffu) * 0x10001u);
+        acc = fmaf(h2f_lo(zz), h0.x, acc);
+        acc = fmaf(h2f_hi(zz), h1.x, acc);
     }
     return acc;
 }
 
-// Subset-sum tables of the slice's units, as int32 fixed point; xs = group sums of x
-// (fp32), invs = 2^-p per unit.  32 consecutive threads build one unit.
-template <bool G64>
-__device__ __forceinline__ void build_luts(const uint16_t *x, int u0, int nU, unsigned char *lut, float *xs,
-                                           float *invs, int tid, int nthreads)
+// DPP lane exchanges inside a row of 16 lanes (no LDS traffic).
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v)
 {
-    const int nchunks = nU * 32;
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// all-reduce over the 16 lanes of a row: xor 1, xor 2 (quad_perm), then half-row and row mirrors
+#define HLQ_ROW_REDUCE(v, OP)             \
+    v = OP(v, dpp_f<0xB1>(v));            \
+    v = OP(v, dpp_f<0x4E>(v));            \
+    v = OP(v, dpp_f<0x141>(v));           \
+    v = OP(v, dpp_f<0x140>(v))
+__device__ __forceinline__ float op_add(float a, float b) { return a + b; }
+__device__ __forceinline__ float op_max(float a, float b) { return fmaxf(a, b); }
+
+// Subset-sum tables of the slice's units as int32 fixed point.  One thread per chunk of
+// 4 activations; the 16 threads of a DPP row cover one 64-k half unit, whose max|x| sets
+// the power-of-two table scale and whose sum feeds the zero-point fold.  `raw` holds the
+// chunk of the first pass (loaded by the caller ahead of the weight loads).
+__device__ __forceinline__ void build_luts(const uint16_t *x, uint2 raw, int nchunks, unsigned char *lut,
+                                           float2 *xs_inv, int tid, int nthreads)
+{
     for (int ci = tid; ci < nchunks; ci += nthreads) {
-        const int lu = ci >> 5, c = ci & 31;
-        const uint2 raw = *(const uint2 *)(x + (size_t)(u0 + lu) * HLQ_UNIT + c * 4);
+        if (ci != tid) raw = *(const uint2 *)(x + (size_t)ci * 4);
         const float x0 = h2f_lo(raw.x), x1 = h2f_hi(raw.x), x2 = h2f_lo(raw.y), x3 = h2f_hi(raw.y);
         float amax = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3)));
         float s = (x0 + x1) + (x2 + x3);
-#pragma unroll
-        for (int o = 1; o <= 8; o <<= 1) {
-            s += __shfl_xor(s, o, 32);
-            amax = fmaxf(amax, __shfl_xor(amax, o, 32));
-        }
-        const float s16 = s;
-        s += __shfl_xor(s, 16, 32);
-        amax = fmaxf(amax, __shfl_xor(amax, 16, 32));
-        // amax < 2^(eb-126): scale by 2^(149-eb) so |x * scale| < 2^23, a 4-subset < 2^25,
-        // 32 lookups < 2^30.
+        HLQ_ROW_REDUCE(s, op_add);
+        HLQ_ROW_REDUCE(amax, op_max);
+        // amax < 2^(eb-126): scale by 2^(149-eb) so |x * scale| < 2^23, a 4-subset < 2^25 and
+        // the 16 lookups of a half unit < 2^29.
         const uint32_t eb = (__float_as_uint(amax) >> 23) & 0xffu;
         const float scale = eb ? __uint_as_float((276u - eb) << 23) : 1.0f;
         const float inv = eb ? __uint_as_float((eb - 22u) << 23) : 1.0f;
@@ -195,68 +192,74 @@ __device__ __forceinline__ void build_luts(const uint16_t *x, int u0, int nU, un
         dst[1] = make_int4(i2, e5, e6, e7);
         dst[2] = make_int4(i3, i3 + i0, i3 + i1, i3 + e3);
         dst[3] = make_int4(i3 + i2, i3 + e5, i3 + e6, i3 + e7);
-        if (c == 0) invs[lu] = inv;
-        if (G64) {
-            if ((c & 15) == 0) xs[2 * lu + (c >> 4)] = s16;
-        } else {
-            if (c == 0) xs[lu] = s;
-        }
+        if ((ci & 15) == 0) xs_inv[ci >> 4] = make_float2(s, inv);
     }
 }
+
+constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 
 template <int BITS, bool G64>
 __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 {
     extern __shared__ __align__(256) unsigned char smem[];
-    constexpr int UPT = G64 ? 1 : 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
     const int cb = blockIdx.x / a.ksplit, slice = blockIdx.x - cb * a.ksplit;
-    const int t0 = slice * a.tps, t1 = min(t0 + a.tps, a.NT);
-    const int u0 = t0 * UPT, nU = min(t1 * UPT, a.U) - u0;
-    const int maxU = a.tps * UPT;
+    const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
+    const int nst = nU * BITS;                                             // sub-tasks of this workgroup
 
     unsigned char *lut = smem;
-    float *xs = (float *)(smem + (size_t)maxU * UNIT_LUT_BYTES);   // [maxU * (G64 ? 2 : 1)]
-    float *invs = xs + maxU * 2;                                     // [maxU]
-    float *red = invs + maxU;                                        // [nw][64]
-    int *flag = (int *)(red + nw * HLQ_CB);
+    float2 *xs_inv = (float2 *)(smem + (size_t)a.ups * UNIT_LUT_BYTES);   // [2 * ups]
+    float *red = (float *)(xs_inv + 2 * a.ups);                            // [nw][64]
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
-    // Issue the first task's loads before the tables are built: HBM latency overlaps the build.
-    Task<BITS, G64> cur;
-    int t = t0 + wave;
-    bool have = t < t1;
-    if (have) load_task<BITS, G64>(cur, a, cb, t, lane);
+    HLQ_STAMP(0);
+    // Activations first (they are needed first and come from cache), then the weight
+    // stream: its HBM latency overlaps the table build.
+    const uint16_t *xsl = a.x + (size_t)u0 * HLQ_UNIT;
+    const int nchunks = nU * 32;
+    uint2 raw = make_uint2(0, 0);
+    if (tid < nchunks) raw = *(const uint2 *)(xsl + (size_t)tid * 4);
 
-    build_luts<G64>(a.x, u0, nU, lut, xs, invs, tid, blockDim.x);
+    Sub slot[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; d++) {
+        const int st = wave + d * nw;
+        if (st < nst) load_sub<BITS, G64>(slot[d], a, cb, u0 + st / BITS, st % BITS, lane);
+    }
+
+    build_luts(xsl, raw, nchunks, lut, xs_inv, tid, blockDim.x);
+    HLQ_STAMP(1);
     __syncthreads();
+    HLQ_STAMP(2);
 
     const uint32_t mask = 0x3Cu;
     float acc = 0.f;
-    while (have) {
-        const int tn = t + nw;
-        const bool hn = tn < t1;
-        Task<BITS, G64> nxt;
-        if (hn) load_task<BITS, G64>(nxt, a, cb, tn, lane);
-        const int lu = (t - t0) * UPT;
-        acc = process_unit<BITS, G64, 0>(cur.w[0], cur.sc, cur.zz, lu, lut_base, xs, invs, mask, acc);
-        if (!G64) {
-            if (t * UPT + 1 < a.U)
-                acc = process_unit<BITS, G64, 1>(cur.w[UPT - 1], cur.sc, cur.zz, lu + 1, lut_base, xs, invs, mask, acc);
+    for (int base = wave; base < nst; base += DEPTH * nw) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) {
+            const int st = base + d * nw;
+            if (st < nst) {
+                const int lu = st / BITS, b = st % BITS;
+                acc = process_sub<G64>(slot[d], lu, b, (u0 + lu) & 1, lut_base, xs_inv, mask, acc);
+                const int sn = st + DEPTH * nw;
+                if (sn < nst) load_sub<BITS, G64>(slot[d], a, cb, u0 + sn / BITS, sn % BITS, lane);
+            }
         }
-        if (hn) cur = nxt;
-        t = tn;
-        have = hn;
     }
 
+    HLQ_STAMP(3);
     // Combine the waves of this workgroup, then the slices of this column block.
-    red[wave * HLQ_CB + lane] = acc;
-    __syncthreads();
     const int n = cb * HLQ_CB + lane;
-    float total = 0.f;
-    if (wave == 0) {
-        for (int w = 0; w < nw; w++) total += red[w * HLQ_CB + lane];
+    float total = acc;
+    if (nw > 1) {
+        red[wave * HLQ_CB + lane] = acc;
+        __syncthreads();
+        if (wave == 0) {
+            total = 0.f;
+            for (int w = 0; w < nw; w++) total += red[w * HLQ_CB + lane];
+        }
     }
+    HLQ_STAMP(4);
     if (a.ksplit == 1) {
         if (wave == 0 && n < a.N) {
             if (a.bias) total += (float)__builtin_bit_cast(_Float16, a.bias[n]);
@@ -264,42 +267,58 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
         }
         return;
     }
+    // Slices meet through device memory.  Partial sums are written and read with
+    // agent-scope atomics (they bypass the per-XCD L2s' non-coherent lines), the writer
+    // waits for its stores to be acknowledged before it takes a ticket, and the reader's
+    // loads depend on the ticket it drew -- so no cache write-back / invalidate is needed.
     const size_t npad = (size_t)a.ncb * HLQ_CB;
     if (wave == 0) {
-        a.partial[(size_t)slice * npad + n] = total;
-        __threadfence();
-    }
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned ticket = atomicAdd(&a.counters[cb], 1u);
-        *flag = (ticket == (unsigned)a.ksplit - 1u);
-    }
-    __syncthreads();
-    if (*flag && wave == 0) {
-        __threadfence();
-        float sum = 0.f;
-        for (int s = 0; s < a.ksplit; s++) sum += __builtin_nontemporal_load(&a.partial[(size_t)s * npad + n]);
-        if (n < a.N) {
-            if (a.bias) sum += (float)__builtin_bit_cast(_Float16, a.bias[n]);
-            a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
+        __hip_atomic_store(&a.partial[(size_t)slice * npad + n], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        HLQ_STAMP(5);
+        unsigned ticket = 0;
+        if (lane == 0)
+            ticket = __hip_atomic_fetch_add(&a.counters[cb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ticket = __builtin_amdgcn_readfirstlane(ticket);
+        HLQ_STAMP(6);
+        if (ticket == (unsigned)a.ksplit - 1u) {
+            // eight independent loads in flight at a time, summed in slice order
+            float sum = 0.f;
+            for (int s0 = 0; s0 < a.ksplit; s0 += 8) {
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) {
+                    const int s = min(s0 + j, a.ksplit - 1);
+                    v[j] = __hip_atomic_load(&a.partial[(size_t)s * npad + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    if (s0 + j < a.ksplit) sum += v[j];
+            }
+            if (n < a.N) {
+                if (a.bias) sum += (float)__builtin_bit_cast(_Float16, a.bias[n]);
+                a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
+            }
+            if (lane == 0) __hip_atomic_store(&a.counters[cb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            HLQ_STAMP(7);
         }
-        if (lane == 0) a.counters[cb] = 0u;
     }
 }
 
-size_t gemv_lds_bytes(int tps, int upt, int waves)
+size_t gemv_lds_bytes(int ups, int waves)
 {
-    const int maxU = tps * upt;
-    return (size_t)maxU * UNIT_LUT_BYTES + (size_t)maxU * 3 * sizeof(float) + (size_t)waves * HLQ_CB * sizeof(float) + 16;
+    return (size_t)ups * UNIT_LUT_BYTES + (size_t)ups * 2 * sizeof(float2) + (size_t)waves * HLQ_CB * sizeof(float) + 16;
 }
 
 template <int BITS, bool G64>
 int launch_gemv(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
     auto kern = hlq_gemv_kernel<BITS, G64>;
-    if (lds > 64 * 1024) {
-        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+    static bool big_lds_enabled = false;      // per template instance; the setting is sticky
+    if (lds > 64 * 1024 && !big_lds_enabled) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS) != hipSuccess)
             return ELUTQ_ERR_HIP;
+        big_lds_enabled = true;
     }
     hipLaunchKernelGGL(kern, dim3(a.ncb * a.ksplit), dim3(waves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
@@ -325,35 +344,41 @@ int check_shape(int K, int N, int bits, int group)
     return ELUTQ_OK;
 }
 
-constexpr int MAX_LDS = 160 * 1024;
 constexpr int WS_COUNTER_BYTES = 64 * 1024;   // one arrival counter per column block, N <= 2^20
 constexpr int NUM_CU = 256;
 
-// Launch shape: enough workgroups to cover every CU a few times over, slices no
-// smaller than one task per wave.
+// Launch shape (measured on MI355X): about one workgroup per CU, as few K slices as that
+// allows (every slice adds a trip through device memory to the tail of the kernel), and
+// 16 waves per workgroup so that every SIMD has several waves to hide LDS latency with.
 void choose_shape(const HlqGeo &g, int &ksplit, int &waves)
 {
-    if (waves <= 0) waves = 4;
     if (ksplit <= 0) {
-        const int want = (4 * NUM_CU + g.ncb - 1) / g.ncb;              // slices for ~4 workgroups per CU
-        const int most = (g.NT + waves - 1) / waves;                    // at least one task per wave
-        ksplit = want < 1 ? 1 : want;
-        if (ksplit > most) ksplit = most;
+        ksplit = NUM_CU / g.ncb;
+        if (ksplit > 4) ksplit = 4;
         if (ksplit < 1) ksplit = 1;
+        if (ksplit > g.U) ksplit = g.U;
     }
+    if (waves <= 0) waves = g.ncb * ksplit > 300 ? 8 : 16;
 }
 
 }  // namespace
 
 extern "C" {
 
+#ifdef HLQ_TIMING
+int elutq_debug_set_stamps(void *d_buf)
+{
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_hlq_stamps), &d_buf, sizeof(d_buf)) == hipSuccess ? 0 : -1;
+}
+#endif
+
 size_t elutq_hlq_workspace_bytes(int K, int N, int bits, int group, int M)
 {
     if (check_shape(K, N, bits, group) != ELUTQ_OK || M < 1) return 0;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     // arrival counters (fixed region, so layers of any shape can share one workspace) +
-    // partial sums for the finest split (one task per slice)
-    return (size_t)WS_COUNTER_BYTES + (size_t)g.NT * g.ncb * HLQ_CB * sizeof(float);
+    // partial sums for the finest split (one unit per slice)
+    return (size_t)WS_COUNTER_BYTES + (size_t)g.U * g.ncb * HLQ_CB * sizeof(float);
 }
 
 int elutq_hlq_workspace_init(void *d_workspace, size_t workspace_bytes, void *stream)
@@ -370,12 +395,12 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
     if (rc != ELUTQ_OK) return rc;
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
     const HlqGeo g = hlq_geo(K, N, bits, group);
-    if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.NT) return ELUTQ_ERR_TUNING;
+    if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return ELUTQ_ERR_TUNING;
     choose_shape(g, ksplit, waves);
-    int tps = (g.NT + ksplit - 1) / ksplit;
-    // shrink the slice count so that no slice is empty, and the slice so its tables fit in LDS
-    while (gemv_lds_bytes(tps, g.UPT, waves) > (size_t)MAX_LDS) tps = (tps + 1) / 2;
-    ksplit = (g.NT + tps - 1) / tps;
+    int ups = (g.U + ksplit - 1) / ksplit;
+    // shrink the slice so its tables fit in LDS, then the slice count so that no slice is empty
+    while (gemv_lds_bytes(ups, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
+    ksplit = (g.U + ups - 1) / ups;
 
     GemvArgs a;
     a.planes = (const uint4 *)d_planes;
@@ -385,7 +410,7 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
     a.x = (const uint16_t *)d_x;
     a.y = (uint16_t *)d_y;
     a.N = N; a.U = g.U; a.NT = g.NT; a.ncb = g.ncb;
-    a.ksplit = ksplit; a.tps = tps;
+    a.ksplit = ksplit; a.ups = ups;
     a.partial = nullptr; a.counters = nullptr;
     if (ksplit > 1) {
         if (!d_workspace) return ELUTQ_ERR_NULL;
@@ -395,7 +420,7 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
         a.counters = (unsigned *)d_workspace;
         a.partial = (float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
-    return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(tps, g.UPT, waves), (hipStream_t)stream);
+    return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, waves), (hipStream_t)stream);
 }
 
 int elutq_hlq_gemv_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,

@@ -78,3 +78,40 @@ LLAMA2_13B_PREFILL_SHAPES = [(5120, 5120), (5120, 13824), (13824, 5120)]
 def algorithmic_bytes(k: int, n: int, bits: int, group: int, m: int = 1) -> int:
     """planes + fp16 per-plane scales + fp16 zeros + x + y."""
     return k * n * bits // 8 + 2 * bits * n * (k // group) + 2 * n * (k // group) + 2 * m * k + 2 * m * n
+
+
+def make_device_layer(k: int, n: int, bits: int = 2, group: int = 128, seed: int = 0, device="cuda",
+                      bias: bool = False):
+    """Random HLQLinear drawn on the GPU directly in the kernel layout, for benchmarks.
+
+    Planes are uniform random bytes (i.i.d. Bernoulli(0.5) bits in any bit order); scales and
+    zeros follow the same per-(column, group) distributions as make_layer.  The values are
+    not those of make_layer(seed): use make_layer when a CPU oracle must see the same bits.
+    """
+    import torch
+
+    from . import _lib
+    from .hlq_linear import HLQLinear
+
+    L = _lib.lib()
+    dev = torch.device(device)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    pb, sb, zb = (L.elutq_hlq_planes_bytes(k, n, bits), L.elutq_hlq_scales_bytes(k, n, bits, group),
+                  L.elutq_hlq_zeros_bytes(k, n, group))
+    if not pb or not sb:
+        raise ValueError(f"unsupported HLQ shape K={k} N={n} bits={bits} group={group}")
+    planes = torch.randint(0, 256, (pb,), generator=g, dtype=torch.uint8, device=dev)
+    ncb, nt = (n + 63) // 64, (k // group + 1) // 2
+
+    def uni(lo, hi):
+        return torch.rand(ncb, nt, 64, 2, generator=g, device=dev) * (hi - lo) + lo
+
+    s0 = uni(0.005, 0.02) if bits == 2 else uni(0.003, 0.01)
+    sc = [s0] + [(2.0 ** b) * s0 * uni(0.8, 1.2) for b in range(1, bits)]
+    s = torch.stack(sc, 2)                                    # [ncb, nt, bits, 64, 2]
+    z = -(s.sum(2)) / 2 * uni(0.9, 1.1)                       # [ncb, nt, 64, 2]
+    scales = s.to(torch.float16).contiguous().view(torch.uint8).reshape(-1)
+    zeros = z.to(torch.float16).contiguous().view(torch.uint8).reshape(-1)
+    assert scales.numel() == sb and zeros.numel() == zb
+    b = (torch.randn(n, generator=g, device=dev) * 0.1).to(torch.float16) if bias else None
+    return HLQLinear(k, n, bits, group, planes, scales, zeros, b)

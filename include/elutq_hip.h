@@ -95,7 +95,7 @@ int elutq_hlq_gemv_f16(const void *d_planes, const void *d_scales, const void *d
 
 /*
  * Same computation with the launch shape chosen by the caller: `ksplit` slices of K
- * per column block (1..number of group pairs) and `waves` wavefronts per workgroup
+ * per column block (1..K/128) and `waves` wavefronts per workgroup
  * (1..16); 0 = library default.  For tuning and for tests that must reach every
  * reduction path; results do not depend on these beyond fp32 summation order.
  */

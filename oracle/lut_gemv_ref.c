@@ -3,7 +3,7 @@
  * TEST INFRASTRUCTURE ONLY: the checker for the HIP kernels and the timed host
  * baseline.  Nothing in the shipped package links or loads this file.
  *
- * The reference (Nkniexin/ELUTQ, C++/ops/src/arm/*.cpp) is ARM-NEON only and
+ * The reference (Nkniexin/ELUTQ, the .cpp files under C++/ops/src/arm) is ARM-NEON only and
  * cannot be compiled on x86, so its algorithm is restated here in portable C,
  * operation for operation, with the same fp16 rounding points:
  *

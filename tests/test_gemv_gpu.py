@@ -38,8 +38,7 @@ def run(m, x, dev):
 @pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 1), (1, 4), (2, 2), (3, 8)])
 def test_gemv_matches_oracle(cuda, k, n, bits, group, ksplit, waves):
     L = make_layer(k, n, bits=bits, group=group, seed=k + n + bits, bias=(n % 3 == 0))
-    nt = (k // group + 1) // 2
-    ks = min(ksplit, nt)
+    ks = min(ksplit, k // 128)
     y = run(to_mod(L, cuda, ks, waves), L.x, cuda)[0]
     ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, group, L.bias)
     assert y.shape == (n,) and y.dtype == np.float16
