@@ -28,7 +28,7 @@
 
 namespace {
 
-constexpr int MAX_LDS = 160 * 1024;
+constexpr int MAX_LDS = HLQ_MAX_LDS;
 constexpr int TBL_BYTES = 64;                    // 16 int32 entries
 constexpr int UNIT_LUT_BYTES = 32 * TBL_BYTES;   // 32 chunks per unit
 
@@ -344,8 +344,8 @@ int check_shape(int K, int N, int bits, int group)
     return ELUTQ_OK;
 }
 
-constexpr int WS_COUNTER_BYTES = 64 * 1024;   // one arrival counter per column block, N <= 2^20
-constexpr int NUM_CU = 256;
+constexpr int WS_COUNTER_BYTES = HLQ_WS_COUNTER_BYTES;   // one arrival counter per column block, N <= 2^20
+constexpr int NUM_CU = HLQ_NUM_CU;
 
 // Launch shape (measured on MI355X): about one workgroup per CU, as few K slices as that
 // allows (every slice adds a trip through device memory to the tail of the kernel), and
@@ -377,8 +377,10 @@ size_t elutq_hlq_workspace_bytes(int K, int N, int bits, int group, int M)
     if (check_shape(K, N, bits, group) != ELUTQ_OK || M < 1) return 0;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     // arrival counters (fixed region, so layers of any shape can share one workspace) +
-    // partial sums for the finest split (one unit per slice)
-    return (size_t)WS_COUNTER_BYTES + (size_t)g.U * g.ncb * HLQ_CB * sizeof(float);
+    // partial sums: GEMV at its finest split (one unit per slice), GEMM at the split it uses
+    const size_t gemv = (size_t)WS_COUNTER_BYTES + (size_t)g.U * g.ncb * HLQ_CB * sizeof(float);
+    const size_t gemm = M > 1 ? hlq_gemm_ws_bytes(g, M > 64 ? 64 : M) : 0;
+    return gemv > gemm ? gemv : gemm;
 }
 
 int elutq_hlq_workspace_init(void *d_workspace, size_t workspace_bytes, void *stream)

@@ -25,6 +25,10 @@
 #define HLQ_CB 64
 #define HLQ_UNIT 128
 #define HLQ_ROT 2
+#define HLQ_NUM_CU 256                 /* MI355X */
+#define HLQ_MAX_LDS (160 * 1024)       /* per workgroup on gfx950 */
+#define HLQ_WS_COUNTER_BYTES (64 * 1024) /* head of every workspace: one arrival counter per column block */
+#define HLQ_GEMM_CH 4                  /* units staged per chunk = waves per GEMM workgroup */
 
 struct HlqGeo {
     int K, N, bits, group;
@@ -50,3 +54,23 @@ static inline HlqGeo hlq_geo(int K, int N, int bits, int group)
 static inline size_t hlq_planes_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.U * g.bits * HLQ_CB * 16; }
 static inline size_t hlq_scales_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * g.bits * HLQ_CB * 4; }
 static inline size_t hlq_zeros_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * HLQ_CB * 4; }
+
+// K slices the GEMM launcher uses for a shape: about one workgroup per CU, whole chunks.
+static inline void hlq_gemm_split(const HlqGeo &g, int &ksplit, int &ups)
+{
+    int ks = (HLQ_NUM_CU + g.ncb - 1) / g.ncb;
+    const int most = (g.U + HLQ_GEMM_CH - 1) / HLQ_GEMM_CH;
+    if (ks > most) ks = most;
+    if (ks < 1) ks = 1;
+    ups = (g.U + ks - 1) / ks;
+    ups = (ups + HLQ_GEMM_CH - 1) / HLQ_GEMM_CH * HLQ_GEMM_CH;
+    ksplit = (g.U + ups - 1) / ups;
+}
+
+static inline size_t hlq_gemm_ws_bytes(const HlqGeo &g, int M)
+{
+    int ks, ups;
+    hlq_gemm_split(g, ks, ups);
+    const int mpad = M <= 32 ? 32 : 64;
+    return (size_t)HLQ_WS_COUNTER_BYTES + (ks > 1 ? (size_t)ks * mpad * g.ncb * HLQ_CB * sizeof(float) : 0);
+}

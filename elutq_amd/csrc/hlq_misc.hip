@@ -83,19 +83,4 @@ int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
 
-// m > 1 in the reference is one GEMV per row (arm_gemm.cpp:380-385).
-int elutq_hlq_gemm_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
-                       const void *d_x, void *d_y, int M, int K, int N, int bits, int group, void *d_workspace,
-                       size_t workspace_bytes, void *stream)
-{
-    if (M < 1) return ELUTQ_ERR_SHAPE;
-    for (int i = 0; i < M; i++) {
-        int rc = elutq_hlq_gemv_f16(d_planes, d_scales, d_zeros, d_bias, (const uint16_t *)d_x + (size_t)i * K,
-                                    (uint16_t *)d_y + (size_t)i * N, K, N, bits, group, d_workspace, workspace_bytes,
-                                    stream);
-        if (rc != ELUTQ_OK) return rc;
-    }
-    return ELUTQ_OK;
-}
-
 }  // extern "C"

@@ -94,7 +94,15 @@ class HLQLinear(nn.Module):
         if self._ws_bytes == 0:
             raise ValueError(f"unsupported HLQ shape K={in_features} N={out_features} bits={bits} "
                              f"group={group_size} (need K % 128 == 0, bits 1..4, group 64 or 128)")
+        self._ws_cache: dict = {}
         self.ksplit, self.waves = 0, 0      # 0 = library default; set for tuning
+
+    def _ws_bytes_for(self, m: int) -> int:
+        key = 64 if m > 32 else 32
+        if key not in self._ws_cache:
+            self._ws_cache[key] = _lib.lib().elutq_hlq_workspace_bytes(
+                self.in_features, self.out_features, self.bits, self.group_size, key)
+        return self._ws_cache[key]
 
     # -- construction ------------------------------------------------------------------
     @classmethod
@@ -129,7 +137,8 @@ class HLQLinear(nn.Module):
         m = x2.shape[0]
         y = torch.empty((m, self.out_features), dtype=torch.float16, device=x.device)
         if m:
-            ws = _workspace(x.device, self._ws_bytes)
+            need = self._ws_bytes if m == 1 else self._ws_bytes_for(m)
+            ws = _workspace(x.device, need)
             stream = torch.cuda.current_stream(x.device).cuda_stream
             L = _lib.lib()
             bias = self.bias.data_ptr() if self.bias is not None else None
