@@ -43,6 +43,10 @@ def parse():
     p.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     p.add_argument("--no-decode", action="store_true", help="skip the decode tokens/s leg")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    p.add_argument("--mode", choices=["full", "kernel", "copy"], default="full",
+                   help="kernel: only the dominant GEMV (4096x14336) over its weight ring, for counter runs; "
+                        "copy: a plain 64 MiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE")
+    p.add_argument("--launches", type=int, default=256, help="launches in --mode kernel / copy")
     return p.parse_args()
 
 
@@ -115,6 +119,35 @@ def cpu_baseline(budget_s):
     return out, ncpu
 
 
+def counter_mode(a, torch, lib, dev):
+    """Eager launches of one kernel only, so a rocprofv3 --pmc run sees nothing else of size."""
+    from elutq_amd.synth import algorithmic_bytes, make_device_layer
+    if a.mode == "copy":
+        n = 64 * 2 ** 20
+        src = torch.randint(0, 255, (n,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(a.launches):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"mode": "copy", "bytes_read": n, "bytes_written": n, "launches": a.launches}))
+        return
+    k, n = 4096, 14336
+    nbytes = algorithmic_bytes(k, n, BITS, GROUP)
+    ring = [make_device_layer(k, n, BITS, GROUP, seed=i, device=dev) for i in range(-(-512 * 2 ** 20 // nbytes))]
+    x = torch.randn(1, k, device=dev).to(torch.float16)
+    y = torch.empty(1, n, dtype=torch.float16, device=dev)
+    ws = torch.zeros(lib.elutq_hlq_workspace_bytes(k, n, BITS, GROUP, 1), dtype=torch.uint8, device=dev)
+    calls = [Gemv(lib, m, x, y, ws) for m in ring]
+    stream = torch.cuda.current_stream().cuda_stream
+    torch.cuda.synchronize()
+    for i in range(a.launches):
+        calls[i % len(calls)](stream)
+    torch.cuda.synchronize()
+    print(json.dumps({"mode": "kernel", "shape": f"{k}x{n}", "algorithmic_bytes": nbytes, "launches": a.launches,
+                      "ring_sets": len(ring)}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -131,6 +164,9 @@ def main():
     lib = _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.mode != "full":
+        counter_mode(a, torch, lib, dev)
+        return
     ws_bytes = max(lib.elutq_hlq_workspace_bytes(k, n, BITS, GROUP, 1) for (k, n) in LLAMA3_8B_SHAPES.values())
     ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
     xs = {k: torch.randn(1, k, device=dev).to(torch.float16) for k in {k for k, _ in LLAMA3_8B_SHAPES.values()}}
@@ -182,7 +218,11 @@ def main():
 
     dom = per_shape["4096x14336"]
     roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": dom["GBps"] / HBM_PEAK_GBPS, "traffic": None,
+                "frac": dom["GBps"] / HBM_PEAK_GBPS,
+                # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+                # `bench.py --mode kernel`, each scaled by what the same counter reads for `--mode copy`
+                # (summary under profiles/); a property of the kernel's access pattern, not of this run.
+                "traffic": 17_648_000,
                 "kernel": "hlq_gemv_kernel<2,false> K=4096 N=14336", "us_per_launch": dom["us"],
                 "bytes_per_launch": dom["bytes"]}
 

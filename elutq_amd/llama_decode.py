@@ -1,0 +1,239 @@
+"""Batch-1 decode step of a LLaMA-shaped model whose linear layers are HLQLinear.
+
+Counterpart of the caller of the hot path in the reference runtime, ``llama::forward`` +
+the decode loop of ``main.cpp`` (C++/examples/models/llama.cpp:150-774,
+C++/examples/main.cpp:81-110): embedding, then per layer RMSNorm -> q/k/v -> RoPE -> KV-cache
+append -> single-token GQA attention -> o -> residual -> RMSNorm -> gate/up -> SiLU*up ->
+down -> residual, final RMSNorm, fp16 lm_head, greedy argmax.  Semantics follow the
+reference ops: RMSNorm in fp32 with fp16 output (arm_rmsnorm.cpp:25-84), half-split RoPE
+pairs (j, j + d/2) with theta = pos * base^(-2j/d) and no frequency rescaling
+(arm_rotary.cpp:31-46), fp32 softmax, GQA map h_kv = h * n_kv / n_q
+(arm_attention.cpp:199-274), SiLU*up in fp32 (arm_activation.cpp:36-49).
+
+Everything except the HLQ projections is plain PyTorch-ROCm glue; the step is captured in a
+HIP graph (token id and position live in device tensors), so one replay = one token.
+q|k|v and gate|up are fused along N, which in the kernel layout is a concatenation of the
+packed buffers.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from .hlq_linear import HLQLinear
+from .synth import make_device_layer
+
+
+@dataclass
+class LlamaShape:
+    n_layers: int = 32
+    hidden: int = 4096
+    n_heads: int = 32
+    n_kv_heads: int = 8
+    ffn: int = 14336
+    vocab: int = 128256
+    rms_eps: float = 1e-5
+    rope_base: float = 500000.0
+    max_seq: int = 640
+    bits: int = 2
+    group: int = 128
+
+    @property
+    def head_dim(self) -> int:
+        return self.hidden // self.n_heads
+
+
+def fuse_along_n(mods: list[HLQLinear]) -> HLQLinear:
+    """One HLQLinear computing the concatenation of the outputs.  The kernel layout is
+    column-block major, so this is a concatenation of the packed buffers (every N but the
+    last must be a multiple of 64)."""
+    k, bits, group = mods[0].in_features, mods[0].bits, mods[0].group_size
+    for m in mods:
+        assert (m.in_features, m.bits, m.group_size) == (k, bits, group)
+    for m in mods[:-1]:
+        assert m.out_features % 64 == 0
+    bias = None
+    if any(m.bias is not None for m in mods):
+        bias = torch.cat([m.bias if m.bias is not None else
+                          torch.zeros(m.out_features, dtype=torch.float16, device=m.planes.device) for m in mods])
+    return HLQLinear(k, sum(m.out_features for m in mods), bits, group,
+                     torch.cat([m.planes for m in mods]), torch.cat([m.scales for m in mods]),
+                     torch.cat([m.zeros for m in mods]), bias)
+
+
+def rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(torch.float16)
+
+
+class DecoderLayer(nn.Module):
+    def __init__(self, s: LlamaShape, linears: dict, norms: tuple, fuse: bool = True):
+        super().__init__()
+        self.s = s
+        self.fused = fuse
+        if fuse:
+            self.qkv = fuse_along_n([linears["q_proj"], linears["k_proj"], linears["v_proj"]])
+            self.gate_up = fuse_along_n([linears["gate_proj"], linears["up_proj"]])
+        else:
+            self.q_proj, self.k_proj, self.v_proj = linears["q_proj"], linears["k_proj"], linears["v_proj"]
+            self.gate_proj, self.up_proj = linears["gate_proj"], linears["up_proj"]
+        self.o_proj, self.down_proj = linears["o_proj"], linears["down_proj"]
+        self.register_buffer("ln1", norms[0])
+        self.register_buffer("ln2", norms[1])
+        self.register_buffer("k_cache", torch.zeros(s.max_seq, s.n_kv_heads, s.head_dim, dtype=torch.float16,
+                                                    device=norms[0].device))
+        self.register_buffer("v_cache", torch.zeros_like(self.k_cache))
+
+    def forward(self, x, pos, cos, sin, mask):
+        """x [1, hidden] fp16; pos int64 [1] (device); cos/sin [1, head_dim/2] fp32 at pos;
+        mask [1, 1, max_seq] additive fp32 (0 up to pos, -inf beyond)."""
+        s = self.s
+        d, nq, nkv = s.head_dim, s.n_heads, s.n_kv_heads
+        h = rms_norm(x, self.ln1, s.rms_eps)
+        if self.fused:
+            qkv = self.qkv(h)
+            q, k, v = qkv.split([nq * d, nkv * d, nkv * d], dim=-1)
+        else:
+            q, k, v = self.q_proj(h), self.k_proj(h), self.v_proj(h)
+        q = rope(q.view(nq, d), cos, sin)
+        k = rope(k.view(nkv, d), cos, sin)
+        self.k_cache.index_copy_(0, pos, k.unsqueeze(0))
+        self.v_cache.index_copy_(0, pos, v.reshape(1, nkv, d))
+        # single-token GQA attention over the whole cache buffer, masked beyond pos
+        qg = q.view(nkv, nq // nkv, d).float()
+        kc = self.k_cache.permute(1, 2, 0).float()                 # [nkv, d, L]
+        scores = torch.matmul(qg, kc) * (d ** -0.5) + mask         # [nkv, nq/nkv, L]
+        p = torch.softmax(scores, dim=-1)
+        ctx = torch.matmul(p, self.v_cache.permute(1, 0, 2).float())   # [nkv, nq/nkv, d]
+        attn = ctx.to(torch.float16).reshape(1, nq * d)
+        x = x + self.o_proj(attn)
+        h = rms_norm(x, self.ln2, s.rms_eps)
+        if self.fused:
+            g, u = self.gate_up(h).split([s.ffn, s.ffn], dim=-1)
+        else:
+            g, u = self.gate_proj(h), self.up_proj(h)
+        act = (F.silu(g.float()) * u.float()).to(torch.float16)
+        return x + self.down_proj(act)
+
+
+def rope(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """Half-split rotation: pairs (j, j + d/2)."""
+    d2 = t.shape[-1] // 2
+    a, b = t[..., :d2].float(), t[..., d2:].float()
+    return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1).to(torch.float16)
+
+
+class LlamaDecoder(nn.Module):
+    """Random-init LLaMA-shaped decoder for the decode benchmark and its parity test."""
+
+    def __init__(self, s: LlamaShape, device="cuda", seed: int = 0, fuse: bool = True):
+        super().__init__()
+        self.s = s
+        dev = torch.device(device)
+        g = torch.Generator(device=dev).manual_seed(seed)
+        d = s.head_dim
+        shapes = {"q_proj": (s.hidden, s.n_heads * d), "k_proj": (s.hidden, s.n_kv_heads * d),
+                  "v_proj": (s.hidden, s.n_kv_heads * d), "o_proj": (s.n_heads * d, s.hidden),
+                  "gate_proj": (s.hidden, s.ffn), "up_proj": (s.hidden, s.ffn), "down_proj": (s.ffn, s.hidden)}
+        layers = []
+        sd = seed * 100_003
+        for _ in range(s.n_layers):
+            lin = {}
+            for name, (k, n) in shapes.items():
+                lin[name] = make_device_layer(k, n, s.bits, s.group, seed=sd, device=dev)
+                sd += 1
+            norms = tuple((1.0 + 0.1 * torch.randn(s.hidden, generator=g, device=dev)).to(torch.float16) for _ in range(2))
+            layers.append(DecoderLayer(s, lin, norms, fuse))
+        self.layers = nn.ModuleList(layers)
+        self.register_buffer("embed", (torch.randn(s.vocab, s.hidden, generator=g, device=dev) * 0.5).to(torch.float16))
+        self.register_buffer("lm_head", (torch.randn(s.vocab, s.hidden, generator=g, device=dev) * 0.02).to(torch.float16))
+        self.register_buffer("norm", (1.0 + 0.1 * torch.randn(s.hidden, generator=g, device=dev)).to(torch.float16))
+        inv = s.rope_base ** (-torch.arange(0, d, 2, device=dev, dtype=torch.float32) / d)
+        ang = torch.arange(s.max_seq, device=dev, dtype=torch.float32)[:, None] * inv[None, :]
+        self.register_buffer("cos_t", ang.cos())
+        self.register_buffer("sin_t", ang.sin())
+        self.register_buffer("arange", torch.arange(s.max_seq, device=dev))
+        # state of the decode loop (device resident so a captured step can advance it)
+        self.register_buffer("token", torch.zeros(1, dtype=torch.long, device=dev))
+        self.register_buffer("pos", torch.zeros(1, dtype=torch.long, device=dev))
+        self._graph = None
+
+    @torch.no_grad()
+    def fill_cache(self, n_tokens: int, seed: int = 1) -> None:
+        """Random fp16 KV entries for positions [0, n_tokens): the 'context already decoded'."""
+        g = torch.Generator(device=self.embed.device).manual_seed(seed)
+        for layer in self.layers:
+            layer.k_cache[:n_tokens] = torch.randn(n_tokens, self.s.n_kv_heads, self.s.head_dim, generator=g,
+                                                   device=self.embed.device).to(torch.float16)
+            layer.v_cache[:n_tokens] = torch.randn(n_tokens, self.s.n_kv_heads, self.s.head_dim, generator=g,
+                                                   device=self.embed.device).to(torch.float16)
+        self.pos.fill_(n_tokens)
+
+    @torch.no_grad()
+    def step(self) -> torch.Tensor:
+        """One decode step from the device-resident (token, pos); stores the greedy next token
+        and pos + 1 back.  Returns the logits [1, vocab] (fp16)."""
+        x = self.embed.index_select(0, self.token)
+        cos = self.cos_t.index_select(0, self.pos)
+        sin = self.sin_t.index_select(0, self.pos)
+        mask = torch.where(self.arange <= self.pos, 0.0, float("-inf")).view(1, 1, -1)
+        for layer in self.layers:
+            x = layer(x, self.pos, cos, sin, mask)
+        logits = F.linear(rms_norm(x, self.norm, self.s.rms_eps), self.lm_head)
+        self.token.copy_(logits.argmax(-1))
+        self.pos.add_(1)
+        return logits
+
+    @torch.no_grad()
+    def capture(self) -> None:
+        """Captures step() in a HIP graph (after eager warm-up steps that size the scratch)."""
+        state = (self.token.clone(), self.pos.clone())
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            for _ in range(2):
+                self.step()
+        s.synchronize()
+        self.token.copy_(state[0])
+        self.pos.copy_(state[1])
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            self._logits = self.step()
+        self._graph = g
+        self.token.copy_(state[0])
+        self.pos.copy_(state[1])
+        torch.cuda.synchronize()
+
+    def replay(self) -> None:
+        self._graph.replay()
+
+
+def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | None = None) -> dict:
+    """Decode tokens/s of the random-init model: n_gen greedy tokens after an n_ctx-token
+    cache; the first generated token is excluded, as in the reference
+    ((generate_num - 1) / elapsed, main.cpp:110)."""
+    s = shape or LlamaShape()
+    model = LlamaDecoder(s, device=device, seed=0)
+    model.fill_cache(n_ctx)
+    model.token.fill_(1)
+    model.capture()
+    model.replay()                           # token 1 (excluded)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n_gen - 1):
+        model.replay()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    hlq_bytes = sum(m.planes.numel() + m.scales.numel() + m.zeros.numel()
+                    for m in model.modules() if isinstance(m, HLQLinear))
+    lm_bytes = model.lm_head.numel() * 2
+    kv_bytes = 2 * s.n_layers * n_ctx * s.n_kv_heads * s.head_dim * 2
+    ms = dt / (n_gen - 1) * 1e3
+    return {"tokens_per_s": (n_gen - 1) / dt, "ms_per_token": ms, "n_ctx": n_ctx, "n_gen": n_gen,
+            "bytes_per_token": hlq_bytes + lm_bytes + kv_bytes,
+            "GBps": (hlq_bytes + lm_bytes + kv_bytes) / (ms * 1e-3) / 1e9,
+            "model": f"LLaMA-3-8B-shaped random init, {s.n_layers} layers, HLQ w{s.bits}g{s.group}, fp16 lm_head",
+            "glue": "PyTorch-ROCm ops (RMSNorm, RoPE, attention, SiLU) + hipBLASLt lm_head, one HIP graph per token"}
