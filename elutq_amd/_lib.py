@@ -26,9 +26,19 @@ SIGNATURES = {
     "elutq_hlq_workspace_init": (_ci, [_vp, _sz, _vp]),
     "elutq_hlq_gemv_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp]),
     "elutq_hlq_gemv_f16_tuned": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _ci, _ci]),
+    "elutq_hlq_gemv_fused_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
+    "elutq_decode_rope_attn_f16": (_ci, [_vp] * 5 + [_ci] * 4 + [ctypes.c_float, _vp]),
     "elutq_hlq_gemm_f16": (_ci, [_vp] * 6 + [_ci] * 5 + [_vp, _sz, _vp]),
     "elutq_hlq_dequant_f16": (_ci, [_vp] * 4 + [_ci] * 4 + [_vp]),
 }
+
+
+
+class GemvFusion(ctypes.Structure):
+    """struct elutq_gemv_fusion of include/elutq_hip.h."""
+    _fields_ = [("prologue", ctypes.c_int), ("eps", ctypes.c_float),
+                ("d_norm_weight", ctypes.c_void_p), ("d_residual", ctypes.c_void_p)]
+
 
 _lib = None
 

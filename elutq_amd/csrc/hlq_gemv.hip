@@ -43,6 +43,11 @@ struct GemvArgs {
     unsigned *counters;      // [ncb], zero between calls
     int N, U, NT, ncb;
     int ksplit, ups;         // slices per column block, units per slice
+    // optional fusion with the ops around the projection in a decoder layer
+    int prologue;            // 0: x as is; 1: rmsnorm(x) * norm_w; 2: silu(x[0:K]) * x[K:2K]
+    float eps;
+    const uint16_t *norm_w;  // fp16 [K]      (prologue 1)
+    const uint16_t *residual;  // fp16 [N] added to the output, or null
 };
 
 #ifdef HLQ_TIMING
@@ -165,16 +170,43 @@ __device__ __forceinline__ float dpp_f(float v)
 __device__ __forceinline__ float op_add(float a, float b) { return a + b; }
 __device__ __forceinline__ float op_max(float a, float b) { return fmaxf(a, b); }
 
+// The four activations of a chunk after the optional prologue, as fp32 values that are
+// exactly representable in fp16 (the fused ops round to fp16 where the unfused pipeline
+// would have stored fp16: RMSNorm output, arm_rmsnorm.cpp:25-84; SiLU(gate)*up,
+// arm_activation.cpp:36-49).
+__device__ __forceinline__ void chunk_values(int prologue, uint2 raw, uint2 raw2, float rstd, float (&v)[4])
+{
+    v[0] = h2f_lo(raw.x); v[1] = h2f_hi(raw.x); v[2] = h2f_lo(raw.y); v[3] = h2f_hi(raw.y);
+    if (prologue == 0) return;
+    const float w[4] = {h2f_lo(raw2.x), h2f_hi(raw2.x), h2f_lo(raw2.y), h2f_hi(raw2.y)};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float t;
+        if (prologue == 1) t = v[i] * rstd * w[i];
+        else t = v[i] / (1.0f + __expf(-v[i])) * w[i];
+        v[i] = (float)(_Float16)t;
+    }
+}
+
+__device__ __forceinline__ void load_chunk(const GemvArgs &a, int K, size_t k, uint2 &raw, uint2 &raw2)
+{
+    raw = *(const uint2 *)(a.x + k);
+    if (a.prologue == 1) raw2 = *(const uint2 *)(a.norm_w + k);
+    else if (a.prologue == 2) raw2 = *(const uint2 *)(a.x + (size_t)K + k);
+}
+
 // Subset-sum tables of the slice's units as int32 fixed point.  One thread per chunk of
 // 4 activations; the 16 threads of a DPP row cover one 64-k half unit, whose max|x| sets
-// the power-of-two table scale and whose sum feeds the zero-point fold.  `raw` holds the
-// chunk of the first pass (loaded by the caller ahead of the weight loads).
-__device__ __forceinline__ void build_luts(const uint16_t *x, uint2 raw, int nchunks, unsigned char *lut,
-                                           float2 *xs_inv, int tid, int nthreads)
+// the power-of-two table scale and whose sum feeds the zero-point fold.  `raw`/`raw2` hold
+// the chunk of the first pass (loaded by the caller ahead of the weight loads).
+__device__ __forceinline__ void build_luts(const GemvArgs &a, int K, size_t k0, uint2 raw, uint2 raw2, float rstd,
+                                           int nchunks, unsigned char *lut, float2 *xs_inv, int tid, int nthreads)
 {
     for (int ci = tid; ci < nchunks; ci += nthreads) {
-        if (ci != tid) raw = *(const uint2 *)(x + (size_t)ci * 4);
-        const float x0 = h2f_lo(raw.x), x1 = h2f_hi(raw.x), x2 = h2f_lo(raw.y), x3 = h2f_hi(raw.y);
+        if (ci != tid) load_chunk(a, K, k0 + (size_t)ci * 4, raw, raw2);
+        float v[4];
+        chunk_values(a.prologue, raw, raw2, rstd, v);
+        const float x0 = v[0], x1 = v[1], x2 = v[2], x3 = v[3];
         float amax = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3)));
         float s = (x0 + x1) + (x2 + x3);
         HLQ_ROW_REDUCE(s, op_add);
@@ -196,6 +228,30 @@ __device__ __forceinline__ void build_luts(const uint16_t *x, uint2 raw, int nch
     }
 }
 
+// 1 / rms of the whole activation vector (every workgroup computes it for itself: 2K bytes
+// from cache), for the fused RMSNorm prologue.  `red` is LDS scratch of >= 64 floats.
+__device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *red, int tid, int nthreads)
+{
+    float ssq = 0.f;
+    for (int i = tid; i < K / 4; i += nthreads) {
+        const uint2 r = *(const uint2 *)(a.x + (size_t)i * 4);
+        const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
+        ssq += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
+    }
+    HLQ_ROW_REDUCE(ssq, op_add);
+    if ((tid & 15) == 0) red[tid >> 4] = ssq;
+    __syncthreads();
+    if (tid < 64) {
+        float v = tid < (nthreads >> 4) ? red[tid] : 0.f;
+        HLQ_ROW_REDUCE(v, op_add);
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        if (tid == 0) red[64] = v;
+    }
+    __syncthreads();
+    return rsqrtf(red[64] / (float)K + a.eps);
+}
+
 constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 
 template <int BITS, bool G64>
@@ -215,10 +271,11 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
     HLQ_STAMP(0);
     // Activations first (they are needed first and come from cache), then the weight
     // stream: its HBM latency overlaps the table build.
-    const uint16_t *xsl = a.x + (size_t)u0 * HLQ_UNIT;
+    const int K = a.U * HLQ_UNIT;
+    const size_t k0 = (size_t)u0 * HLQ_UNIT;
     const int nchunks = nU * 32;
-    uint2 raw = make_uint2(0, 0);
-    if (tid < nchunks) raw = *(const uint2 *)(xsl + (size_t)tid * 4);
+    uint2 raw = make_uint2(0, 0), raw2 = make_uint2(0, 0);
+    if (tid < nchunks) load_chunk(a, K, k0 + (size_t)tid * 4, raw, raw2);
 
     Sub slot[DEPTH];
 #pragma unroll
@@ -227,7 +284,9 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
         if (st < nst) load_sub<BITS, G64>(slot[d], a, cb, u0 + st / BITS, st % BITS, lane);
     }
 
-    build_luts(xsl, raw, nchunks, lut, xs_inv, tid, blockDim.x);
+    float rstd = 1.f;
+    if (a.prologue == 1) rstd = block_rstd(a, K, red, tid, blockDim.x);
+    build_luts(a, K, k0, raw, raw2, rstd, nchunks, lut, xs_inv, tid, blockDim.x);
     HLQ_STAMP(1);
     __syncthreads();
     HLQ_STAMP(2);
@@ -263,6 +322,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
     if (a.ksplit == 1) {
         if (wave == 0 && n < a.N) {
             if (a.bias) total += (float)__builtin_bit_cast(_Float16, a.bias[n]);
+            if (a.residual) total += (float)__builtin_bit_cast(_Float16, a.residual[n]);
             a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)total);
         }
         return;
@@ -297,6 +357,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
             }
             if (n < a.N) {
                 if (a.bias) sum += (float)__builtin_bit_cast(_Float16, a.bias[n]);
+                if (a.residual) sum += (float)__builtin_bit_cast(_Float16, a.residual[n]);
                 a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
             }
             if (lane == 0) __hip_atomic_store(&a.counters[cb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -307,7 +368,8 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 
 size_t gemv_lds_bytes(int ups, int waves)
 {
-    return (size_t)ups * UNIT_LUT_BYTES + (size_t)ups * 2 * sizeof(float2) + (size_t)waves * HLQ_CB * sizeof(float) + 16;
+    const int red = waves * HLQ_CB > 80 ? waves * HLQ_CB : 80;      // cross-wave sums; >= 65 floats for block_rstd
+    return (size_t)ups * UNIT_LUT_BYTES + (size_t)ups * 2 * sizeof(float2) + (size_t)red * sizeof(float) + 16;
 }
 
 template <int BITS, bool G64>
@@ -389,9 +451,10 @@ int elutq_hlq_workspace_init(void *d_workspace, size_t workspace_bytes, void *st
     return hipMemsetAsync(d_workspace, 0, workspace_bytes, (hipStream_t)stream) == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
 
-int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
                              const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
-                             size_t workspace_bytes, void *stream, int ksplit, int waves)
+                             size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,
+                             int waves)
 {
     int rc = check_shape(K, N, bits, group);
     if (rc != ELUTQ_OK) return rc;
@@ -414,6 +477,15 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
     a.N = N; a.U = g.U; a.NT = g.NT; a.ncb = g.ncb;
     a.ksplit = ksplit; a.ups = ups;
     a.partial = nullptr; a.counters = nullptr;
+    a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr;
+    if (fusion) {
+        if (fusion->prologue < 0 || fusion->prologue > 2) return ELUTQ_ERR_TUNING;
+        if (fusion->prologue == 1 && !fusion->d_norm_weight) return ELUTQ_ERR_NULL;
+        a.prologue = fusion->prologue;
+        a.eps = fusion->eps;
+        a.norm_w = (const uint16_t *)fusion->d_norm_weight;
+        a.residual = (const uint16_t *)fusion->d_residual;
+    }
     if (ksplit > 1) {
         if (!d_workspace) return ELUTQ_ERR_NULL;
         if ((size_t)g.ncb * sizeof(unsigned) > (size_t)WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
@@ -425,12 +497,20 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, waves), (hipStream_t)stream);
 }
 
+int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                             const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
+                             size_t workspace_bytes, void *stream, int ksplit, int waves)
+{
+    return elutq_hlq_gemv_fused_f16(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace,
+                                    workspace_bytes, stream, nullptr, ksplit, waves);
+}
+
 int elutq_hlq_gemv_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
                        const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
                        size_t workspace_bytes, void *stream)
 {
-    return elutq_hlq_gemv_f16_tuned(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace,
-                                    workspace_bytes, stream, 0, 0);
+    return elutq_hlq_gemv_fused_f16(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace,
+                                    workspace_bytes, stream, nullptr, 0, 0);
 }
 
 }  // extern "C"

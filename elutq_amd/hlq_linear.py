@@ -157,6 +157,27 @@ class HLQLinear(nn.Module):
         y = y.reshape(*x.shape[:-1], self.out_features)
         return y if in_dtype == torch.float16 else y.to(in_dtype)
 
+    def gemv_fused(self, x: torch.Tensor, out: torch.Tensor, ws: torch.Tensor, prologue: int = 0,
+                   norm_weight: torch.Tensor | None = None, eps: float = 0.0,
+                   residual: torch.Tensor | None = None) -> torch.Tensor:
+        """Batch-1 GEMV into a caller-owned `out`, optionally fused with the RMSNorm in front of
+        the projection (prologue 1), the SiLU(gate)*up in front of it (prologue 2; x holds 2K
+        values) and a residual added to the result.  No allocation: `ws` is the caller's
+        zero-initialised workspace.  See elutq_hlq_gemv_fused_f16 in include/elutq_hip.h."""
+        f = _lib.GemvFusion(prologue, eps, norm_weight.data_ptr() if norm_weight is not None else None,
+                            residual.data_ptr() if residual is not None else None)
+        rc = _lib.lib().elutq_hlq_gemv_fused_f16(
+            self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
+            self.bias.data_ptr() if self.bias is not None else None, x.data_ptr(), out.data_ptr(),
+            self.in_features, self.out_features, self.bits, self.group_size, ws.data_ptr(), ws.numel(),
+            torch.cuda.current_stream(x.device).cuda_stream, ctypes.byref(f), self.ksplit, self.waves)
+        _lib.check(rc, "elutq_hlq_gemv_fused_f16")
+        return out
+
+    @property
+    def workspace_bytes(self) -> int:
+        return self._ws_bytes
+
     def dequantize(self) -> torch.Tensor:
         """Dense fp16 W [N, K] (``dequantize_with_scales``, GPTQ/quant.py:176-183)."""
         w = torch.empty((self.out_features, self.in_features), dtype=torch.float16, device=self.planes.device)

@@ -24,6 +24,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
+from . import _lib
 from .hlq_linear import HLQLinear
 from .synth import make_device_layer
 
@@ -120,6 +121,34 @@ class DecoderLayer(nn.Module):
         return x + self.down_proj(act)
 
 
+class FusedBuffers:
+    """Static activations of the fused decode path (nothing is allocated per token)."""
+
+    def __init__(self, s: LlamaShape, ws_bytes: int, device):
+        d = s.head_dim
+        f16 = dict(dtype=torch.float16, device=device)
+        self.xa = torch.zeros(1, s.hidden, **f16)
+        self.xb = torch.zeros(1, s.hidden, **f16)
+        self.qkv = torch.zeros(1, (s.n_heads + 2 * s.n_kv_heads) * d, **f16)
+        self.attn = torch.zeros(1, s.n_heads * d, **f16)
+        self.gu = torch.zeros(1, 2 * s.ffn, **f16)
+        self.ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=device)
+
+
+def fused_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tensor) -> None:
+    """One decoder layer in five launches: rmsnorm+qkv | rope+cache+attention | o+residual |
+    rmsnorm+gate|up | silu*up+down+residual.  The residual stream enters and leaves in b.xa."""
+    s = layer.s
+    layer.qkv.gemv_fused(b.xa, b.qkv, b.ws, prologue=1, norm_weight=layer.ln1, eps=s.rms_eps)
+    rc = _lib.lib().elutq_decode_rope_attn_f16(
+        b.qkv.data_ptr(), layer.k_cache.data_ptr(), layer.v_cache.data_ptr(), pos.data_ptr(), b.attn.data_ptr(),
+        s.n_heads, s.n_kv_heads, s.head_dim, s.max_seq, s.rope_base, torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "elutq_decode_rope_attn_f16")
+    layer.o_proj.gemv_fused(b.attn, b.xb, b.ws, residual=b.xa)
+    layer.gate_up.gemv_fused(b.xb, b.gu, b.ws, prologue=1, norm_weight=layer.ln2, eps=s.rms_eps)
+    layer.down_proj.gemv_fused(b.gu, b.xa, b.ws, prologue=2, residual=b.xb)
+
+
 def rope(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
     """Half-split rotation: pairs (j, j + d/2)."""
     d2 = t.shape[-1] // 2
@@ -130,9 +159,13 @@ def rope(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
 class LlamaDecoder(nn.Module):
     """Random-init LLaMA-shaped decoder for the decode benchmark and its parity test."""
 
-    def __init__(self, s: LlamaShape, device="cuda", seed: int = 0, fuse: bool = True):
+    def __init__(self, s: LlamaShape, device="cuda", seed: int = 0, fuse: bool = True, impl: str = "hip"):
+        """impl "hip": five fused launches per layer through the C ABI (needs fuse=True);
+        impl "torch": the same step with PyTorch ops around plain HLQLinear calls."""
         super().__init__()
+        assert impl in ("hip", "torch") and (fuse or impl == "torch")
         self.s = s
+        self.impl = impl
         dev = torch.device(device)
         g = torch.Generator(device=dev).manual_seed(seed)
         d = s.head_dim
@@ -161,6 +194,10 @@ class LlamaDecoder(nn.Module):
         self.register_buffer("token", torch.zeros(1, dtype=torch.long, device=dev))
         self.register_buffer("pos", torch.zeros(1, dtype=torch.long, device=dev))
         self._graph = None
+        self._buf = None
+        if impl == "hip":
+            ws = max(m.workspace_bytes for m in self.modules() if isinstance(m, HLQLinear))
+            self._buf = FusedBuffers(s, ws, dev)
 
     @torch.no_grad()
     def fill_cache(self, n_tokens: int, seed: int = 1) -> None:
@@ -177,12 +214,19 @@ class LlamaDecoder(nn.Module):
     def step(self) -> torch.Tensor:
         """One decode step from the device-resident (token, pos); stores the greedy next token
         and pos + 1 back.  Returns the logits [1, vocab] (fp16)."""
-        x = self.embed.index_select(0, self.token)
-        cos = self.cos_t.index_select(0, self.pos)
-        sin = self.sin_t.index_select(0, self.pos)
-        mask = torch.where(self.arange <= self.pos, 0.0, float("-inf")).view(1, 1, -1)
-        for layer in self.layers:
-            x = layer(x, self.pos, cos, sin, mask)
+        if self.impl == "hip":
+            b = self._buf
+            torch.index_select(self.embed, 0, self.token, out=b.xa)
+            for layer in self.layers:
+                fused_layer_step(layer, b, self.pos)
+            x = b.xa
+        else:
+            x = self.embed.index_select(0, self.token)
+            cos = self.cos_t.index_select(0, self.pos)
+            sin = self.sin_t.index_select(0, self.pos)
+            mask = torch.where(self.arange <= self.pos, 0.0, float("-inf")).view(1, 1, -1)
+            for layer in self.layers:
+                x = layer(x, self.pos, cos, sin, mask)
         logits = F.linear(rms_norm(x, self.norm, self.s.rms_eps), self.lm_head)
         self.token.copy_(logits.argmax(-1))
         self.pos.add_(1)
@@ -211,12 +255,13 @@ class LlamaDecoder(nn.Module):
         self._graph.replay()
 
 
-def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | None = None) -> dict:
+def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | None = None,
+                 impl: str = "hip") -> dict:
     """Decode tokens/s of the random-init model: n_gen greedy tokens after an n_ctx-token
     cache; the first generated token is excluded, as in the reference
     ((generate_num - 1) / elapsed, main.cpp:110)."""
     s = shape or LlamaShape()
-    model = LlamaDecoder(s, device=device, seed=0)
+    model = LlamaDecoder(s, device=device, seed=0, impl=impl)
     model.fill_cache(n_ctx)
     model.token.fill_(1)
     model.capture()
@@ -236,4 +281,6 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
             "bytes_per_token": hlq_bytes + lm_bytes + kv_bytes,
             "GBps": (hlq_bytes + lm_bytes + kv_bytes) / (ms * 1e-3) / 1e9,
             "model": f"LLaMA-3-8B-shaped random init, {s.n_layers} layers, HLQ w{s.bits}g{s.group}, fp16 lm_head",
-            "glue": "PyTorch-ROCm ops (RMSNorm, RoPE, attention, SiLU) + hipBLASLt lm_head, one HIP graph per token"}
+            "glue": ("5 launches per layer (rmsnorm+qkv | rope+cache+attention | o+residual | rmsnorm+gate|up | "
+                     "silu*up+down+residual), " if impl == "hip" else "PyTorch-ROCm ops around the HLQ GEMVs, ")
+                    + "torch embedding / final norm / hipBLASLt fp16 lm_head / argmax, one HIP graph per token"}

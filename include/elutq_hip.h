@@ -106,6 +106,31 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
                              int ksplit, int waves);
 
 /*
+ * Batch-1 GEMV fused with the ops that surround a projection in a decoder layer, so a
+ * decode step needs one launch where the reference runs two or three operators:
+ *   prologue 1  x <- fp16(rmsnorm(x) * norm_weight)     launch_pre_rms_norm + arm_gemm
+ *                                                       (C++/ops/src/arm/arm_rmsnorm.cpp:25-84)
+ *   prologue 2  x <- fp16(silu(x[0:K]) * x[K:2K])        gated_silu + arm_gemm; d_x holds 2K values
+ *                                                       (C++/ops/src/arm/arm_activation.cpp:22-53)
+ *   d_residual  y <- y + residual (fp16 [N])            the residual add folded into the next
+ *                                                       norm in the reference (arm_rmsnorm.cpp:43-85)
+ * `fusion` is a HOST pointer (read before the call returns) or NULL for a plain GEMV.
+ * ksplit / waves as in elutq_hlq_gemv_f16_tuned.
+ */
+typedef struct elutq_gemv_fusion {
+    int prologue;               /* 0, 1 or 2 */
+    float eps;                  /* RMSNorm epsilon (prologue 1) */
+    const void *d_norm_weight;  /* fp16 [K] (prologue 1) */
+    const void *d_residual;     /* fp16 [N] or NULL */
+} elutq_gemv_fusion;
+
+int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
+                             const void *d_bias, const void *d_x, void *d_y,
+                             int K, int N, int bits, int group,
+                             void *d_workspace, size_t workspace_bytes, void *stream,
+                             const elutq_gemv_fusion *fusion, int ksplit, int waves);
+
+/*
  * y[M][N] = x[M][K] W^T + bias, row-major fp16, 1 <= M.  Replaces arm_gemm(m > 1, ...),
  * which the reference defines as one GEMV per row.
  */
@@ -113,6 +138,20 @@ int elutq_hlq_gemm_f16(const void *d_planes, const void *d_scales, const void *d
                        const void *d_bias, const void *d_x, void *d_y,
                        int M, int K, int N, int bits, int group,
                        void *d_workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Decode-step glue between the q|k|v projection and the o projection, one launch per layer:
+ * half-split RoPE on q and k at position *d_pos, append of k and v to the caches at that
+ * position, single-token grouped-query attention over positions 0..*d_pos, fp16 output
+ * [n_heads * head_dim].  Replaces launch_llama_qkv_apply_rotary + arm_cache + arm_attention
+ * (C++/ops/src/arm/arm_rotary.cpp:4-89, arm_cache.cpp:17-22, arm_attention.cpp:162-316).
+ * d_qkv fp16 [n_heads*d | n_kv_heads*d | n_kv_heads*d]; caches fp16 [max_seq][n_kv_heads][d];
+ * d_pos a DEVICE int64 (so a captured graph can advance it); head_dim even, <= 128.
+ * If *d_pos is outside [0, max_seq) the kernel does nothing.
+ */
+int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,
+                               void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                               float rope_base, void *stream);
 
 /* W[N][K] fp16 row-major from the repacked buffers (dequantize_with_scales). */
 int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void *d_zeros,

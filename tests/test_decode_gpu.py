@@ -45,10 +45,10 @@ def test_fuse_along_n_is_concatenation(cuda):
     assert torch.equal(f.dequantize(), torch.cat([a.dequantize(), b.dequantize(), c.dequantize()]))
 
 
-@pytest.mark.parametrize("fuse", [True, False])
-def test_decode_step_matches_dense_model(cuda, fuse):
-    hlq = LlamaDecoder(SMALL, device=cuda, seed=3, fuse=fuse)
-    ref = densify(LlamaDecoder(SMALL, device=cuda, seed=3, fuse=fuse))
+@pytest.mark.parametrize("fuse,impl", [(True, "hip"), (True, "torch"), (False, "torch")])
+def test_decode_step_matches_dense_model(cuda, fuse, impl):
+    hlq = LlamaDecoder(SMALL, device=cuda, seed=3, fuse=fuse, impl=impl)
+    ref = densify(LlamaDecoder(SMALL, device=cuda, seed=3, fuse=fuse, impl="torch"))
     for m in (hlq, ref):
         m.fill_cache(20, seed=5)
         m.token.fill_(7)
@@ -64,9 +64,27 @@ def test_decode_step_matches_dense_model(cuda, fuse):
     assert (k0 - k1).abs().max() <= 1e-2 * k1.abs().max()
 
 
-def test_graph_replay_equals_eager(cuda):
-    eager = LlamaDecoder(SMALL, device=cuda, seed=4)
-    graph = LlamaDecoder(SMALL, device=cuda, seed=4)
+def test_fused_launches_match_torch_glue(cuda):
+    """The five fused launches per layer against the same HLQ model run with PyTorch glue:
+    same tokens, logits within fp16 rounding of the intermediate activations."""
+    a = LlamaDecoder(SMALL, device=cuda, seed=6, impl="hip")
+    b = LlamaDecoder(SMALL, device=cuda, seed=6, impl="torch")
+    for m in (a, b):
+        m.fill_cache(33, seed=8)
+        m.token.fill_(11)
+    for step in range(5):
+        la, lb = a.step().float(), b.step().float()
+        assert (la - lb).abs().max() <= 1e-2 * lb.pow(2).mean().sqrt(), step
+        assert int(a.token) == int(b.token)
+    for la_, lb_ in zip(a.layers, b.layers):
+        assert (la_.k_cache[33:38].float() - lb_.k_cache[33:38].float()).abs().max() <= 2e-2
+        assert torch.equal(la_.k_cache[:33], lb_.k_cache[:33])
+
+
+@pytest.mark.parametrize("impl", ["hip", "torch"])
+def test_graph_replay_equals_eager(cuda, impl):
+    eager = LlamaDecoder(SMALL, device=cuda, seed=4, impl=impl)
+    graph = LlamaDecoder(SMALL, device=cuda, seed=4, impl=impl)
     for m in (eager, graph):
         m.fill_cache(10, seed=2)
         m.token.fill_(3)
