@@ -60,7 +60,7 @@ __global__ __launch_bounds__(ATTN_WAVES * 64) void rope_attn_kernel(const AttnAr
 
     const float inv_freq = exp2f(-(float)(2 * j) / (float)d * a.log2_base);
     float sn, cs;
-    sincosf((float)pos * inv_freq, &sn, &cs);
+    __sincosf((float)pos * inv_freq, &sn, &cs);
     const uint16_t *qp = a.qkv + (size_t)h * d, *kp = a.qkv + (size_t)a.nq * d + (size_t)g * d;
     const uint16_t *vp = a.qkv + (size_t)(a.nq + a.nkv) * d + (size_t)g * d;
     const float qa = h2f(qp[j]), qb = h2f(qp[j + half]), ka = h2f(kp[j]), kb = h2f(kp[j + half]);
@@ -129,6 +129,131 @@ __global__ __launch_bounds__(ATTN_WAVES * 64) void rope_attn_kernel(const AttnAr
     }
 }
 
+
+// ---------------------------------------------------------------------------------------
+// head_dim 128: coalesced variant.  A wave instruction covers 4 cache rows x 16 segments of
+// 8 dims (one dwordx4 per lane, 1 KiB contiguous per kv head row group); the 16 lanes of a
+// DPP row reduce their partial dot products among themselves, so no LDS permutes are
+// needed, and every (wave, row) pair runs its own running-max softmax stream over the
+// positions it sees.  Batches of FAST_BATCH row groups are loaded before any is used.
+// ---------------------------------------------------------------------------------------
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+constexpr int FAST_WAVES = 8;
+constexpr int FAST_BATCH = 8;
+constexpr int FAST_D = 128;
+
+__device__ __forceinline__ float dot8(const uint4 &q, const uint4 &k)
+{
+    float s = 0.f;
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, q.x), __builtin_bit_cast(half2v, k.x), s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, q.y), __builtin_bit_cast(half2v, k.y), s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, q.z), __builtin_bit_cast(half2v, k.z), s, false);
+    s = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, q.w), __builtin_bit_cast(half2v, k.w), s, false);
+    s += dpp_f<0xB1>(s);
+    s += dpp_f<0x4E>(s);
+    s += dpp_f<0x141>(s);
+    s += dpp_f<0x140>(s);
+    return s;
+}
+
+__device__ __forceinline__ void stream_update(float s, bool valid, const uint4 &v, float &m, float &l, float (&acc)[8])
+{
+    const float mx = valid ? fmaxf(m, s) : m;
+    const float corr = (m == mx) ? 1.f : __expf(m - mx);
+    const float e = valid ? __expf(s - mx) : 0.f;
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    l = fmaf(l, corr, e);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        acc[2 * i] = fmaf(e, h2f((uint16_t)(w[i] & 0xffffu)), acc[2 * i] * corr);
+        acc[2 * i + 1] = fmaf(e, h2f((uint16_t)(w[i] >> 16)), acc[2 * i + 1] * corr);
+    }
+    m = mx;
+}
+
+__global__ __launch_bounds__(FAST_WAVES * 64) void rope_attn_d128_kernel(const AttnArgs a)
+{
+    constexpr int D = FAST_D, HALF = D / 2, STREAMS = FAST_WAVES * 4;
+    __shared__ __align__(16) uint16_t sq[D], sk[D], sv[D];
+    __shared__ float sm_m[STREAMS], sm_l[STREAMS];
+    __shared__ float sm_o[STREAMS][D];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int h = blockIdx.x, grp = a.nq / a.nkv, g = h / grp;
+    const int pos = (int)*a.pos;
+    if (pos < 0 || pos >= a.max_seq) return;
+
+    if (tid < HALF) {                                    // rotary pair (tid, tid + 64) of q and of the new k
+        const int j = tid;
+        const float inv_freq = exp2f(-(float)(2 * j) / (float)D * a.log2_base);
+        float sn, cs;
+        __sincosf((float)pos * inv_freq, &sn, &cs);
+        const uint16_t *qp = a.qkv + (size_t)h * D, *kp = a.qkv + (size_t)a.nq * D + (size_t)g * D;
+        const uint16_t *vp = a.qkv + (size_t)(a.nq + a.nkv) * D + (size_t)g * D;
+        const float qa = h2f(qp[j]), qb = h2f(qp[j + HALF]), ka = h2f(kp[j]), kb = h2f(kp[j + HALF]);
+        sq[j] = f2h(qa * cs - qb * sn); sq[j + HALF] = f2h(qb * cs + qa * sn);
+        sk[j] = f2h(ka * cs - kb * sn); sk[j + HALF] = f2h(kb * cs + ka * sn);
+        sv[j] = vp[j]; sv[j + HALF] = vp[j + HALF];
+    }
+    __syncthreads();
+    if (h % grp == 0 && tid < D / 8) {                   // one workgroup per kv head appends the new row
+        const size_t row = ((size_t)pos * a.nkv + g) * D;
+        ((uint4 *)(a.kc + row))[tid] = ((const uint4 *)sk)[tid];
+        ((uint4 *)(a.vc + row))[tid] = ((const uint4 *)sv)[tid];
+    }
+
+    const int seg = lane & 15, r = lane >> 4;
+    const uint4 qv = ((const uint4 *)sq)[seg];
+    const float scale = rsqrtf((float)D);
+    const int ngroups = (pos + 3) >> 2;                  // row groups of the cached positions 0..pos-1
+    float m = -INFINITY, l = 0.f, acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.f;
+
+    for (int gb = wave; gb < ngroups; gb += FAST_WAVES * FAST_BATCH) {
+        uint4 kk[FAST_BATCH], vv[FAST_BATCH];
+        bool ok[FAST_BATCH];
+#pragma unroll
+        for (int b = 0; b < FAST_BATCH; b++) {
+            const int p = (gb + FAST_WAVES * b) * 4 + r;
+            ok[b] = p < pos;
+            const size_t row = ((size_t)(ok[b] ? p : 0) * a.nkv + g) * D;
+            kk[b] = ((const uint4 *)(a.kc + row))[seg];
+            vv[b] = ((const uint4 *)(a.vc + row))[seg];
+        }
+        // keep the whole batch of loads ahead of the first use (the scheduler would otherwise
+        // sink each load to its consumer and serialise the memory round trips)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int b = 0; b < FAST_BATCH; b++) {
+            const float s = dot8(qv, kk[b]) * scale;
+            stream_update(s, ok[b], vv[b], m, l, acc);
+        }
+    }
+    if (wave == 0) {                                     // the token being decoded, from LDS (row 0 only)
+        const float s = dot8(qv, ((const uint4 *)sk)[seg]) * scale;
+        stream_update(s, r == 0, ((const uint4 *)sv)[seg], m, l, acc);
+    }
+    const int stream = wave * 4 + r;
+    if (seg == 0) { sm_m[stream] = m; sm_l[stream] = l; }
+#pragma unroll
+    for (int i = 0; i < 8; i++) sm_o[stream][seg * 8 + i] = acc[i];
+    __syncthreads();
+    if (tid < D) {
+        float M = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < STREAMS; s++) M = fmaxf(M, sm_m[s]);
+        float L = 0.f, o = 0.f;
+#pragma unroll
+        for (int s = 0; s < STREAMS; s++) {
+            const float f = __expf(sm_m[s] - M);
+            L = fmaf(sm_l[s], f, L);
+            o = fmaf(sm_o[s][tid], f, o);
+        }
+        a.out[(size_t)h * D + tid] = f2h(o / L);
+    }
+}
+
 }  // namespace
 
 extern "C" int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,
@@ -147,6 +272,9 @@ extern "C" int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, vo
     a.out = (uint16_t *)d_out;
     a.nq = n_heads; a.nkv = n_kv_heads; a.d = head_dim; a.max_seq = max_seq;
     a.log2_base = log2f(rope_base);
-    hipLaunchKernelGGL(rope_attn_kernel, dim3(n_heads), dim3(ATTN_WAVES * 64), 0, (hipStream_t)stream, a);
+    if (head_dim == FAST_D)
+        hipLaunchKernelGGL(rope_attn_d128_kernel, dim3(n_heads), dim3(FAST_WAVES * 64), 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL(rope_attn_kernel, dim3(n_heads), dim3(ATTN_WAVES * 64), 0, (hipStream_t)stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }

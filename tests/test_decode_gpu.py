@@ -100,3 +100,60 @@ def test_graph_replay_equals_eager(cuda, impl):
         toks_g.append(int(graph.token))
         _ = torch.randn(64, 64, device=cuda) @ torch.randn(64, 64, device=cuda)    # unrelated eager work between replays
     assert toks_e == toks_g and int(graph.pos) == 16
+
+
+@pytest.mark.parametrize("d,nq,nkv", [(128, 8, 2), (128, 4, 4), (64, 8, 2), (32, 4, 1)])
+@pytest.mark.parametrize("pos", [0, 1, 3, 4, 5, 37, 255, 300])
+def test_rope_cache_attention_kernel(cuda, d, nq, nkv, pos):
+    """elutq_decode_rope_attn_f16 against the PyTorch restatement of the reference ops
+    (half-split RoPE, cache append, fp32-softmax GQA attention)."""
+    from elutq_amd import _lib
+    from elutq_amd.llama_decode import rope
+    g = torch.Generator(device=cuda).manual_seed(pos * 7 + d)
+    max_seq, base = 320, 10000.0
+    qkv = torch.randn(1, (nq + 2 * nkv) * d, generator=g, device=cuda).half()
+    kc = torch.randn(max_seq, nkv, d, generator=g, device=cuda).half()
+    vc = torch.randn(max_seq, nkv, d, generator=g, device=cuda).half()
+    kc0, vc0 = kc.clone(), vc.clone()
+    out = torch.zeros(1, nq * d, dtype=torch.float16, device=cuda)
+    pos_t = torch.tensor([pos], dtype=torch.long, device=cuda)
+    rc = _lib.lib().elutq_decode_rope_attn_f16(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), pos_t.data_ptr(),
+                                               out.data_ptr(), nq, nkv, d, max_seq, base,
+                                               torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    # reference
+    inv = base ** (-torch.arange(0, d, 2, device=cuda, dtype=torch.float32) / d)
+    ang = pos * inv
+    q, k, v = qkv[0].split([nq * d, nkv * d, nkv * d])
+    qr = rope(q.view(nq, d), ang.cos(), ang.sin())
+    kr = rope(k.view(nkv, d), ang.cos(), ang.sin())
+    kref, vref = kc0.clone(), vc0.clone()
+    kref[pos], vref[pos] = kr, v.view(nkv, d)
+    assert (kc[pos].float() - kref[pos].float()).abs().max() <= 4e-3 * kref[pos].float().abs().max()
+    assert torch.equal(vc[pos], vref[pos])
+    keep = torch.ones(max_seq, dtype=torch.bool, device=cuda)
+    keep[pos] = False
+    assert torch.equal(kc[keep], kc0[keep]) and torch.equal(vc[keep], vc0[keep])      # nothing else touched
+    qg = qr.view(nkv, nq // nkv, d).float()
+    sc = torch.matmul(qg, kref[:pos + 1].permute(1, 2, 0).float()) * d ** -0.5
+    ctx = torch.matmul(torch.softmax(sc, -1), vref[:pos + 1].permute(1, 0, 2).float()).reshape(1, nq * d)
+    assert (out.float() - ctx).abs().max() <= 5e-3 * max(1.0, float(ctx.abs().max()))
+
+
+def test_rope_attn_rejects_bad_arguments(cuda):
+    from elutq_amd import _lib
+    L = _lib.lib()
+    t = torch.zeros(4096, dtype=torch.float16, device=cuda)
+    p = torch.zeros(1, dtype=torch.long, device=cuda)
+    s = torch.cuda.current_stream().cuda_stream
+    args = lambda nq, nkv, d: (t.data_ptr(), t.data_ptr(), t.data_ptr(), p.data_ptr(), t.data_ptr(), nq, nkv, d, 8, 1e4, s)
+    assert L.elutq_decode_rope_attn_f16(*args(8, 3, 64)) == -2       # heads not a multiple of kv heads
+    assert L.elutq_decode_rope_attn_f16(*args(8, 2, 256)) == -2      # head_dim > 128
+    assert L.elutq_decode_rope_attn_f16(None, t.data_ptr(), t.data_ptr(), p.data_ptr(), t.data_ptr(), 8, 2, 64, 8, 1e4, s) == -1
+    # a position outside the cache leaves the output untouched
+    out = torch.full((1, 256), 7.0, dtype=torch.float16, device=cuda)
+    p.fill_(8)
+    assert L.elutq_decode_rope_attn_f16(t.data_ptr(), t.data_ptr(), t.data_ptr(), p.data_ptr(), out.data_ptr(), 4, 1, 64, 8, 1e4, s) == 0
+    torch.cuda.synchronize()
+    assert bool((out == 7).all())
