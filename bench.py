@@ -42,6 +42,7 @@ def parse():
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     p.add_argument("--no-decode", action="store_true", help="skip the decode tokens/s leg")
+    p.add_argument("--no-gemm", action="store_true", help="skip the small-batch GEMM leg")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
     p.add_argument("--mode", choices=["full", "kernel", "copy"], default="full",
                    help="kernel: only the dominant GEMV (4096x14336) over its weight ring, for counter runs; "
@@ -117,6 +118,40 @@ def cpu_baseline(budget_s):
         dt = (time.perf_counter() - t0) / reps
         out[threads] = {"GBps": nbytes / dt / 1e9, "ms_per_layer": dt * 1e3, "reps": reps}
     return out, ncpu
+
+
+MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
+
+
+def gemm_leg(torch, lib, dev, steps):
+    """BASELINE config 4: small-batch GEMM, HLQ w2g128, M in {16, 32, 64}, LLaMA-2-13B shapes;
+    each over a ring of weight sets > 400 MB.  Reports both roofline fractions (MFMA and HBM)."""
+    from elutq_amd.synth import LLAMA2_13B_PREFILL_SHAPES, algorithmic_bytes, make_device_layer
+    out = {}
+    for (k, n) in LLAMA2_13B_PREFILL_SHAPES:
+        nsets = -(-400 * 2 ** 20 // algorithmic_bytes(k, n, BITS, GROUP, 16))
+        mods = [make_device_layer(k, n, BITS, GROUP, seed=50_000 + i, device=dev) for i in range(nsets)]
+        for m in (16, 32, 64):
+            x = torch.randn(m, k, device=dev).to(torch.float16)
+            y = torch.empty(m, n, dtype=torch.float16, device=dev)
+            ws = torch.zeros(lib.elutq_hlq_workspace_bytes(k, n, BITS, GROUP, m), dtype=torch.uint8, device=dev)
+
+            def launch(stream):
+                for md in mods:
+                    rc = lib.elutq_hlq_gemm_f16(md.planes.data_ptr(), md.scales.data_ptr(), md.zeros.data_ptr(), None,
+                                                x.data_ptr(), y.data_ptr(), m, k, n, BITS, GROUP, ws.data_ptr(),
+                                                ws.numel(), stream)
+                    if rc:
+                        raise RuntimeError(f"elutq_hlq_gemm_f16 failed: {rc}")
+
+            sec = time_graph(torch, launch, max(3, min(steps, 10)), 1) / nsets
+            flops, nbytes = 2.0 * m * k * n, algorithmic_bytes(k, n, BITS, GROUP, m)
+            out[f"{k}x{n}_M{m}"] = {"us": sec * 1e6, "TFLOPs": flops / sec / 1e12,
+                                    "frac_mfma_peak": flops / sec / 1e12 / MFMA_PEAK_TFLOPS,
+                                    "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}
+        del mods
+        torch.cuda.empty_cache()
+    return out
 
 
 def counter_mode(a, torch, lib, dev):
@@ -238,6 +273,9 @@ def main():
         "per_shape": per_shape,
         "roofline": roofline,
     }
+
+    if not a.no_gemm:
+        out["gemm_w2g128_llama2_13b"] = gemm_leg(torch, lib, dev, a.steps)
 
     if not a.no_decode:
         try:

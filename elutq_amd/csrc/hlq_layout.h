@@ -58,7 +58,7 @@ static inline size_t hlq_zeros_bytes(const HlqGeo &g) { return (size_t)g.ncb * g
 // K slices the GEMM launcher uses for a shape: about one workgroup per CU, whole chunks.
 static inline void hlq_gemm_split(const HlqGeo &g, int &ksplit, int &ups)
 {
-    int ks = (HLQ_NUM_CU + g.ncb - 1) / g.ncb;
+    int ks = 2 * HLQ_NUM_CU / g.ncb;                     // at most two workgroups per CU, all resident at once
     const int most = (g.U + HLQ_GEMM_CH - 1) / HLQ_GEMM_CH;
     if (ks > most) ks = most;
     if (ks < 1) ks = 1;
