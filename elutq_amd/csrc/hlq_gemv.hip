@@ -10,16 +10,20 @@
 //    the same 4-activation chunk, so all 64 LDS reads fall in one 64-byte table and are
 //    conflict free (broadcast), and the per-column sums need no cross-lane reduction;
 //  * the activation tables hold the 16 subset sums of each chunk as int32 fixed point
-//    with a per-unit power-of-two scale chosen from max|x| of the unit: sums are exact
-//    integers (no LUT rounding unless |x_k| < 2^-13 max|x|, then <= 2^-24 max|x|), two
+//    with a power-of-two scale per 64-k half unit chosen from max|x| of that half: sums are
+//    exact integers (no LUT rounding unless |x_k| < 2^-13 max|x|, then <= 2^-24 max|x|), two
 //    lookups retire with one v_add3_u32;
 //  * the plane dwords are stored rotated so that `byte & 0x3C` is already the byte offset
 //    into the table; one SDWA v_and per lookup writes that offset into byte 0 of a
 //    register whose upper bytes keep the table base (dst_unused:UNUSED_PRESERVE), the
 //    chunk index rides in the ds_read immediate;
-//  * a workgroup owns one column block and a slice of K, builds only that slice's
-//    tables, its waves split the slice; slices are combined through a workspace by the
-//    last workgroup to arrive (fixed summation order, so results are deterministic).
+//  * a workgroup owns one column block and a slice of K; its (unit, plane) sub-tasks are
+//    dealt to the waves in contiguous runs, and each wave builds the tables of the units of
+//    its own run in its own LDS region, so no wave waits for another before its lookups;
+//  * loads are unconditional and ordered (activations, first sub-task, table build, rest of
+//    the run) so that the in-order vector-memory counter can be waited on precisely;
+//  * slices are combined through a workspace by the last workgroup to arrive (fixed
+//    summation order, so results are deterministic).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -43,6 +47,8 @@ struct GemvArgs {
     unsigned *counters;      // [ncb], zero between calls
     int N, U, NT, ncb;
     int ksplit, ups;         // slices per column block, units per slice
+    int spw;                 // sub-tasks per wave (contiguous run)
+    int nuw_max, wave_lds;   // units a wave's run can touch, bytes of its LDS region
     // optional fusion with the ops around the projection in a decoder layer
     int prologue;            // 0: x as is; 1: rmsnorm(x) * norm_w; 2: silu(x[0:K]) * x[K:2K]
     float eps;
@@ -124,8 +130,7 @@ __device__ __forceinline__ void load_sub(Sub &t, const GemvArgs &a, int cb, int 
     t.w = make_uint4(v.x, v.y, v.z, v.w);
     const size_t m = (size_t)cb * a.NT + (G64 ? u : (u >> 1));
     t.sc = a.scales[(m * BITS + b) * HLQ_CB + lane];
-    t.zz = 0;
-    if (b == 0) t.zz = a.zeros[m * HLQ_CB + lane];
+    t.zz = a.zeros[m * HLQ_CB + lane];       // used by plane 0 only; loaded always so that every sub-task is 3 loads
 }
 
 // The two 64-k halves of a unit have their own table scale (2^-p) and activation sum; at
@@ -188,120 +193,147 @@ __device__ __forceinline__ void chunk_values(int prologue, uint2 raw, uint2 raw2
     }
 }
 
+// Always two loads (without a prologue the second one re-reads the chunk): a fixed number
+// of loads lets the compiler wait for these with an exact vector-memory count while the
+// weight loads issued after them are still in flight.
 __device__ __forceinline__ void load_chunk(const GemvArgs &a, int K, size_t k, uint2 &raw, uint2 &raw2)
 {
     raw = *(const uint2 *)(a.x + k);
-    if (a.prologue == 1) raw2 = *(const uint2 *)(a.norm_w + k);
-    else if (a.prologue == 2) raw2 = *(const uint2 *)(a.x + (size_t)K + k);
+    const uint16_t *second = a.prologue == 1 ? a.norm_w + k : (a.prologue == 2 ? a.x + (size_t)K + k : a.x + k);
+    raw2 = *(const uint2 *)second;
 }
 
-// Subset-sum tables of the slice's units as int32 fixed point.  One thread per chunk of
-// 4 activations; the 16 threads of a DPP row cover one 64-k half unit, whose max|x| sets
-// the power-of-two table scale and whose sum feeds the zero-point fold.  `raw`/`raw2` hold
-// the chunk of the first pass (loaded by the caller ahead of the weight loads).
-__device__ __forceinline__ void build_luts(const GemvArgs &a, int K, size_t k0, uint2 raw, uint2 raw2, float rstd,
-                                           int nchunks, unsigned char *lut, float2 *xs_inv, int tid, int nthreads)
+// Subset-sum table of one chunk of 4 activations as int32 fixed point, 64 bytes at `tbl`.
+// The 16 lanes of a DPP row cover one 64-k half unit, whose max|x| sets the power-of-two
+// table scale and whose sum feeds the zero-point fold (row leader stores both in *half).
+__device__ __forceinline__ void build_chunk(int prologue, uint2 raw, uint2 raw2, float rstd, unsigned char *tbl,
+                                            float2 *half, bool leader)
 {
-    for (int ci = tid; ci < nchunks; ci += nthreads) {
-        if (ci != tid) load_chunk(a, K, k0 + (size_t)ci * 4, raw, raw2);
-        float v[4];
-        chunk_values(a.prologue, raw, raw2, rstd, v);
-        const float x0 = v[0], x1 = v[1], x2 = v[2], x3 = v[3];
-        float amax = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3)));
-        float s = (x0 + x1) + (x2 + x3);
-        HLQ_ROW_REDUCE(s, op_add);
-        HLQ_ROW_REDUCE(amax, op_max);
-        // amax < 2^(eb-126): scale by 2^(149-eb) so |x * scale| < 2^23, a 4-subset < 2^25 and
-        // the 16 lookups of a half unit < 2^29.
-        const uint32_t eb = (__float_as_uint(amax) >> 23) & 0xffu;
-        const float scale = eb ? __uint_as_float((276u - eb) << 23) : 1.0f;
-        const float inv = eb ? __uint_as_float((eb - 22u) << 23) : 1.0f;
-        const int i0 = __float2int_rn(x0 * scale), i1 = __float2int_rn(x1 * scale);
-        const int i2 = __float2int_rn(x2 * scale), i3 = __float2int_rn(x3 * scale);
-        const int e3 = i0 + i1, e5 = i0 + i2, e6 = i1 + i2, e7 = e3 + i2;
-        int4 *dst = (int4 *)(lut + (size_t)ci * TBL_BYTES);
-        dst[0] = make_int4(0, i0, i1, e3);
-        dst[1] = make_int4(i2, e5, e6, e7);
-        dst[2] = make_int4(i3, i3 + i0, i3 + i1, i3 + e3);
-        dst[3] = make_int4(i3 + i2, i3 + e5, i3 + e6, i3 + e7);
-        if ((ci & 15) == 0) xs_inv[ci >> 4] = make_float2(s, inv);
-    }
+    float v[4];
+    chunk_values(prologue, raw, raw2, rstd, v);
+    const float x0 = v[0], x1 = v[1], x2 = v[2], x3 = v[3];
+    float amax = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3)));
+    float s = (x0 + x1) + (x2 + x3);
+    HLQ_ROW_REDUCE(s, op_add);
+    HLQ_ROW_REDUCE(amax, op_max);
+    // amax < 2^(eb-126): scale by 2^(149-eb) so |x * scale| < 2^23, a 4-subset < 2^25 and
+    // the 16 lookups of a half unit < 2^29.
+    const uint32_t eb = (__float_as_uint(amax) >> 23) & 0xffu;
+    const float scale = eb ? __uint_as_float((276u - eb) << 23) : 1.0f;
+    const float inv = eb ? __uint_as_float((eb - 22u) << 23) : 1.0f;
+    const int i0 = __float2int_rn(x0 * scale), i1 = __float2int_rn(x1 * scale);
+    const int i2 = __float2int_rn(x2 * scale), i3 = __float2int_rn(x3 * scale);
+    const int e3 = i0 + i1, e5 = i0 + i2, e6 = i1 + i2, e7 = e3 + i2;
+    int4 *dst = (int4 *)tbl;
+    dst[0] = make_int4(0, i0, i1, e3);
+    dst[1] = make_int4(i2, e5, e6, e7);
+    dst[2] = make_int4(i3, i3 + i0, i3 + i1, i3 + e3);
+    dst[3] = make_int4(i3 + i2, i3 + e5, i3 + e6, i3 + e7);
+    if (leader) *half = make_float2(s, inv);
 }
 
-// 1 / rms of the whole activation vector (every workgroup computes it for itself: 2K bytes
-// from cache), for the fused RMSNorm prologue.  `red` is LDS scratch of >= 64 floats.
-__device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *red, int tid, int nthreads)
+// 1 / rms of the whole activation vector for the fused RMSNorm prologue; every wave
+// computes it for itself (2K bytes from cache, K/256 loads per lane), so no barrier.
+__device__ __forceinline__ float wave_rstd(const GemvArgs &a, int K, int lane)
 {
     float ssq = 0.f;
-    for (int i = tid; i < K / 4; i += nthreads) {
+    for (int i = lane; i < K / 4; i += 64) {
         const uint2 r = *(const uint2 *)(a.x + (size_t)i * 4);
         const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
         ssq += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
     }
     HLQ_ROW_REDUCE(ssq, op_add);
-    if ((tid & 15) == 0) red[tid >> 4] = ssq;
-    __syncthreads();
-    if (tid < 64) {
-        float v = tid < (nthreads >> 4) ? red[tid] : 0.f;
-        HLQ_ROW_REDUCE(v, op_add);
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
-        if (tid == 0) red[64] = v;
-    }
-    __syncthreads();
-    return rsqrtf(red[64] / (float)K + a.eps);
+    ssq += __shfl_xor(ssq, 16, 64);
+    ssq += __shfl_xor(ssq, 32, 64);
+    return rsqrtf(ssq / (float)K + a.eps);
 }
 
 constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 
-template <int BITS, bool G64>
+// One workgroup = one column block x one K slice.  Its (unit, plane) sub-tasks are dealt to
+// the waves in contiguous runs of `spw`; every wave builds the activation tables of the
+// (one or two) units its run touches in its own LDS region and goes on to its lookups
+// without waiting for the other waves -- the only workgroup barrier is the one in front of
+// the final cross-wave sum.
+template <int BITS, bool G64, int NSLOT>
 __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 {
     extern __shared__ __align__(256) unsigned char smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cb = blockIdx.x / a.ksplit, slice = blockIdx.x - cb * a.ksplit;
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
     const int nst = nU * BITS;                                             // sub-tasks of this workgroup
+    const int s_begin = min(wave * a.spw, nst), s_end = min(s_begin + a.spw, nst);
+    const int ub = s_begin / BITS;                                         // first unit (in the slice) of this wave
+    const int nuw = s_end > s_begin ? (s_end - 1) / BITS - ub + 1 : 0;     // units this wave touches
+    const int s_last = max(s_end - 1, 0);                                  // clamp target for loads past the run
 
-    unsigned char *lut = smem;
-    float2 *xs_inv = (float2 *)(smem + (size_t)a.ups * UNIT_LUT_BYTES);   // [2 * ups]
-    float *red = (float *)(xs_inv + 2 * a.ups);                            // [nw][64]
+    unsigned char *lut = smem + (size_t)wave * a.wave_lds;                 // this wave's tables [nuw][32][16] int32
+    float2 *xs_inv = (float2 *)(lut + (size_t)a.nuw_max * UNIT_LUT_BYTES); // [2 * nuw_max]
+    float *red = (float *)(smem + (size_t)nw * a.wave_lds);                // [nw][64]
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
     HLQ_STAMP(0);
-    // Activations first (they are needed first and come from cache), then the weight
-    // stream: its HBM latency overlaps the table build.
+    // Activations first, then the weight stream.  Every load below is unconditional (a wave
+    // whose run is shorter than NSLOT re-reads its last sub-task), so the number of loads
+    // behind the activations is a compile-time constant and the table build waits for the
+    // activations only (vmcnt(3 * NSLOT)), with the weights still in flight.
     const int K = a.U * HLQ_UNIT;
-    const size_t k0 = (size_t)u0 * HLQ_UNIT;
-    const int nchunks = nU * 32;
-    uint2 raw = make_uint2(0, 0), raw2 = make_uint2(0, 0);
-    if (tid < nchunks) load_chunk(a, K, k0 + (size_t)tid * 4, raw, raw2);
-
-    Sub slot[DEPTH];
-#pragma unroll
-    for (int d = 0; d < DEPTH; d++) {
-        const int st = wave + d * nw;
-        if (st < nst) load_sub<BITS, G64>(slot[d], a, cb, u0 + st / BITS, st % BITS, lane);
-    }
-
+    const size_t k0 = (size_t)(u0 + ub) * HLQ_UNIT;
+    const int nchunks = nuw * 32;
     float rstd = 1.f;
-    if (a.prologue == 1) rstd = block_rstd(a, K, red, tid, blockDim.x);
-    build_luts(a, K, k0, raw, raw2, rstd, nchunks, lut, xs_inv, tid, blockDim.x);
-    HLQ_STAMP(1);
-    __syncthreads();
-    HLQ_STAMP(2);
+    if (a.prologue == 1) rstd = wave_rstd(a, K, lane);
+    uint2 raw, raw2;
+    // lanes past the run (and waves without one, whose k0 is the end of the slice) re-read a valid chunk
+    load_chunk(a, K, nchunks ? k0 + (size_t)min(lane, nchunks - 1) * 4 : 0, raw, raw2);
+    asm volatile("" ::: "memory");      // keep both activation loads ahead of the weight loads
 
     const uint32_t mask = 0x3Cu;
     float acc = 0.f;
-    for (int base = wave; base < nst; base += DEPTH * nw) {
+    Sub slot[NSLOT];
+    {   // the first sub-task's loads start the weight stream ...
+        const int st = min(s_begin, s_last);
+        load_sub<BITS, G64>(slot[0], a, cb, u0 + st / BITS, st % BITS, lane);
+    }
+    asm volatile("" ::: "memory");
+
+    // ... the tables are built as soon as the activations are in (a wave that first queued all
+    // its weight loads would sit in the memory pipeline's back-pressure instead) ...
+    if (lane < nchunks)
+        build_chunk(a.prologue, raw, raw2, rstd, lut + (size_t)lane * TBL_BYTES, xs_inv + (lane >> 4), (lane & 15) == 0);
+    asm volatile("" ::: "memory");
+
+    // ... and the rest of the run's loads follow.
 #pragma unroll
-        for (int d = 0; d < DEPTH; d++) {
-            const int st = base + d * nw;
-            if (st < nst) {
-                const int lu = st / BITS, b = st % BITS;
-                acc = process_sub<G64>(slot[d], lu, b, (u0 + lu) & 1, lut_base, xs_inv, mask, acc);
-                const int sn = st + DEPTH * nw;
-                if (sn < nst) load_sub<BITS, G64>(slot[d], a, cb, u0 + sn / BITS, sn % BITS, lane);
+    for (int d = 1; d < NSLOT; d++) {
+        const int st = min(s_begin + d, s_last);
+        load_sub<BITS, G64>(slot[d], a, cb, u0 + st / BITS, st % BITS, lane);
+    }
+    for (int ci = lane + 64; ci < nchunks; ci += 64) {      // runs of more than two units (not the common case)
+        load_chunk(a, K, k0 + (size_t)ci * 4, raw, raw2);
+        build_chunk(a.prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0);
+    }
+    HLQ_STAMP(1);
+    // The tables were written by this wave and are read by this wave: LDS executes a wave's
+    // operations in order, so no barrier -- only keep the compiler from reordering.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+    HLQ_STAMP(2);
+
+    // Slot d holds sub-task base + d; it is refilled with sub-task base + d + NSLOT as soon as
+    // it has been consumed (past the end of the run: a reload nobody reads).
+    for (int base = s_begin; base < s_end; base += NSLOT) {
+#pragma unroll
+        for (int d = 0; d < NSLOT; d++) {
+            const int st = base + d;
+            if (st < s_end) {
+                const int u = st / BITS;
+                acc = process_sub<G64>(slot[d], u - ub, st % BITS, (u0 + u) & 1, lut_base, xs_inv, mask, acc);
+            }
+            if (base + NSLOT < s_end) {                     // wave-uniform: only runs longer than NSLOT refill
+                const int sn = min(st + NSLOT, s_last);
+                load_sub<BITS, G64>(slot[d], a, cb, u0 + sn / BITS, sn % BITS, lane);
             }
         }
     }
@@ -366,16 +398,34 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
     }
 }
 
-size_t gemv_lds_bytes(int ups, int waves)
+// Per-wave LDS region and run length for a slice of `ups` units handled by `waves` waves.
+struct WavePlan {
+    int spw, nuw_max, wave_lds;
+};
+
+WavePlan wave_plan(int ups, int bits, int waves)
 {
-    const int red = waves * HLQ_CB > 80 ? waves * HLQ_CB : 80;      // cross-wave sums; >= 65 floats for block_rstd
-    return (size_t)ups * UNIT_LUT_BYTES + (size_t)ups * 2 * sizeof(float2) + (size_t)red * sizeof(float) + 16;
+    WavePlan p;
+    const int nst = ups * bits;
+    p.spw = (nst + waves - 1) / waves;
+    if (p.spw > bits && p.spw % bits) p.spw += bits - p.spw % bits;     // whole units per wave when it has several
+    if (p.spw == 1) p.nuw_max = 1;
+    else if (p.spw % bits == 0) p.nuw_max = p.spw / bits;
+    else p.nuw_max = (p.spw + bits - 2) / bits + 1;
+    p.wave_lds = (p.nuw_max * (UNIT_LUT_BYTES + 2 * (int)sizeof(float2)) + 255) & ~255;
+    return p;
 }
 
-template <int BITS, bool G64>
-int launch_gemv(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
+size_t gemv_lds_bytes(int ups, int bits, int waves)
 {
-    auto kern = hlq_gemv_kernel<BITS, G64>;
+    const WavePlan p = wave_plan(ups, bits, waves);
+    return (size_t)waves * p.wave_lds + (size_t)waves * HLQ_CB * sizeof(float) + 16;
+}
+
+template <int BITS, bool G64, int NSLOT>
+int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
+{
+    auto kern = hlq_gemv_kernel<BITS, G64, NSLOT>;
     static bool big_lds_enabled = false;      // per template instance; the setting is sticky
     if (lds > 64 * 1024 && !big_lds_enabled) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS) != hipSuccess)
@@ -384,6 +434,18 @@ int launch_gemv(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
     }
     hipLaunchKernelGGL(kern, dim3(a.ncb * a.ksplit), dim3(waves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
+}
+
+// NSLOT = sub-tasks a wave keeps in flight: its whole run when that is at most DEPTH.
+template <int BITS, bool G64>
+int launch_gemv(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
+{
+    switch (a.spw < DEPTH ? a.spw : DEPTH) {
+    case 1: return launch_gemv_n<BITS, G64, 1>(a, waves, lds, stream);
+    case 2: return launch_gemv_n<BITS, G64, 2>(a, waves, lds, stream);
+    case 3: return launch_gemv_n<BITS, G64, 3>(a, waves, lds, stream);
+    default: return launch_gemv_n<BITS, G64, 4>(a, waves, lds, stream);
+    }
 }
 
 int dispatch_gemv(const GemvArgs &a, int bits, int group, int waves, size_t lds, hipStream_t stream)
@@ -409,18 +471,21 @@ int check_shape(int K, int N, int bits, int group)
 constexpr int WS_COUNTER_BYTES = HLQ_WS_COUNTER_BYTES;   // one arrival counter per column block, N <= 2^20
 constexpr int NUM_CU = HLQ_NUM_CU;
 
-// Launch shape (measured on MI355X): about one workgroup per CU, as few K slices as that
-// allows (every slice adds a trip through device memory to the tail of the kernel), and
-// 16 waves per workgroup so that every SIMD has several waves to hide LDS latency with.
+// Launch shape (measured on MI355X): 16 waves per workgroup so that every SIMD has several
+// waves to hide LDS latency with; K is sliced only where it has to be -- when the column
+// blocks alone leave most CUs idle (N < 4096), or when a slice longer than 32 units would
+// give a wave a run of more than four sub-tasks at w2 (every slice adds partial-sum
+// traffic and three dependent trips through device memory to the tail of the kernel).
 void choose_shape(const HlqGeo &g, int &ksplit, int &waves)
 {
     if (ksplit <= 0) {
-        ksplit = NUM_CU / g.ncb;
+        ksplit = g.ncb >= 64 ? 1 : NUM_CU / g.ncb;
         if (ksplit > 4) ksplit = 4;
-        if (ksplit < 1) ksplit = 1;
+        const int by_len = (g.U + 31) / 32;
+        if (ksplit < by_len) ksplit = by_len;
         if (ksplit > g.U) ksplit = g.U;
     }
-    if (waves <= 0) waves = g.ncb * ksplit > 300 ? 8 : 16;
+    if (waves <= 0) waves = 16;
 }
 
 }  // namespace
@@ -464,7 +529,7 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
     choose_shape(g, ksplit, waves);
     int ups = (g.U + ksplit - 1) / ksplit;
     // shrink the slice so its tables fit in LDS, then the slice count so that no slice is empty
-    while (gemv_lds_bytes(ups, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
+    while (gemv_lds_bytes(ups, bits, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
     ksplit = (g.U + ups - 1) / ups;
 
     GemvArgs a;
@@ -476,6 +541,8 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
     a.y = (uint16_t *)d_y;
     a.N = N; a.U = g.U; a.NT = g.NT; a.ncb = g.ncb;
     a.ksplit = ksplit; a.ups = ups;
+    const WavePlan wp = wave_plan(ups, bits, waves);
+    a.spw = wp.spw; a.nuw_max = wp.nuw_max; a.wave_lds = wp.wave_lds;
     a.partial = nullptr; a.counters = nullptr;
     a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr;
     if (fusion) {
@@ -494,7 +561,7 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
         a.counters = (unsigned *)d_workspace;
         a.partial = (float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
-    return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, waves), (hipStream_t)stream);
+    return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves), (hipStream_t)stream);
 }
 
 int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
