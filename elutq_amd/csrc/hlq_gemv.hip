@@ -232,20 +232,30 @@ __device__ __forceinline__ void build_chunk(int prologue, uint2 raw, uint2 raw2,
     if (leader) *half = make_float2(s, inv);
 }
 
-// 1 / rms of the whole activation vector for the fused RMSNorm prologue; every wave
-// computes it for itself (2K bytes from cache, K/256 loads per lane), so no barrier.
-__device__ __forceinline__ float wave_rstd(const GemvArgs &a, int K, int lane)
+// 1 / rms of the whole activation vector for the fused RMSNorm prologue: the workgroup sums
+// the squares together (one chunk per thread and pass), two barriers.  `scratch` is LDS of
+// RSTD_SCRATCH floats.  Every workgroup does this for itself (2K bytes from cache).
+constexpr int RSTD_SCRATCH = 80;
+__device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scratch, int tid, int nthreads)
 {
     float ssq = 0.f;
-    for (int i = lane; i < K / 4; i += 64) {
+    for (int i = tid; i < K / 4; i += nthreads) {
         const uint2 r = *(const uint2 *)(a.x + (size_t)i * 4);
         const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
         ssq += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
     }
     HLQ_ROW_REDUCE(ssq, op_add);
-    ssq += __shfl_xor(ssq, 16, 64);
-    ssq += __shfl_xor(ssq, 32, 64);
-    return rsqrtf(ssq / (float)K + a.eps);
+    if ((tid & 15) == 0) scratch[tid >> 4] = ssq;
+    __syncthreads();
+    if (tid < 64) {
+        float v = tid < (nthreads >> 4) ? scratch[tid] : 0.f;
+        HLQ_ROW_REDUCE(v, op_add);
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        if (tid == 0) scratch[64] = v;
+    }
+    __syncthreads();
+    return rsqrtf(scratch[64] / (float)K + a.eps);
 }
 
 constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
@@ -272,6 +282,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
     unsigned char *lut = smem + (size_t)wave * a.wave_lds;                 // this wave's tables [nuw][32][16] int32
     float2 *xs_inv = (float2 *)(lut + (size_t)a.nuw_max * UNIT_LUT_BYTES); // [2 * nuw_max]
     float *red = (float *)(smem + (size_t)nw * a.wave_lds);                // [nw][64]
+    float *rstd_scratch = red + nw * HLQ_CB;                               // [RSTD_SCRATCH]
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
     HLQ_STAMP(0);
@@ -283,7 +294,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
     const size_t k0 = (size_t)(u0 + ub) * HLQ_UNIT;
     const int nchunks = nuw * 32;
     float rstd = 1.f;
-    if (a.prologue == 1) rstd = wave_rstd(a, K, lane);
+    if (a.prologue == 1) rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x);
     uint2 raw, raw2;
     // lanes past the run (and waves without one, whose k0 is the end of the slice) re-read a valid chunk
     load_chunk(a, K, nchunks ? k0 + (size_t)min(lane, nchunks - 1) * 4 : 0, raw, raw2);
@@ -419,7 +430,7 @@ WavePlan wave_plan(int ups, int bits, int waves)
 size_t gemv_lds_bytes(int ups, int bits, int waves)
 {
     const WavePlan p = wave_plan(ups, bits, waves);
-    return (size_t)waves * p.wave_lds + (size_t)waves * HLQ_CB * sizeof(float) + 16;
+    return (size_t)waves * p.wave_lds + (size_t)waves * HLQ_CB * sizeof(float) + RSTD_SCRATCH * sizeof(float) + 16;
 }
 
 template <int BITS, bool G64, int NSLOT>
