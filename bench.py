@@ -44,9 +44,10 @@ def parse():
     p.add_argument("--no-decode", action="store_true", help="skip the decode tokens/s leg")
     p.add_argument("--no-gemm", action="store_true", help="skip the small-batch GEMM leg")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
-    p.add_argument("--mode", choices=["full", "kernel", "copy"], default="full",
+    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "gemm"], default="full",
                    help="kernel: only the dominant GEMV (4096x14336) over its weight ring, for counter runs; "
-                        "copy: a plain 64 MiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE")
+                        "copy: a plain 64 MiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE; "
+                        "decode / gemm: only that leg (for kernel traces)")
     p.add_argument("--launches", type=int, default=256, help="launches in --mode kernel / copy")
     return p.parse_args()
 
@@ -199,6 +200,13 @@ def main():
     lib = _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.mode == "decode":
+        from elutq_amd.llama_decode import bench_decode
+        print(json.dumps({"mode": "decode", "decode": bench_decode(dev)}))
+        return
+    if a.mode == "gemm":
+        print(json.dumps({"mode": "gemm", "gemm_w2g128_llama2_13b": gemm_leg(torch, lib, dev, a.steps)}))
+        return
     if a.mode != "full":
         counter_mode(a, torch, lib, dev)
         return
@@ -257,7 +265,7 @@ def main():
                 # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
                 # `bench.py --mode kernel`, each scaled by what the same counter reads for `--mode copy`
                 # (summary under profiles/); a property of the kernel's access pattern, not of this run.
-                "traffic": 17_648_000,
+                "traffic": 17_681_000,
                 "kernel": "hlq_gemv_kernel<2,false> K=4096 N=14336", "us_per_launch": dom["us"],
                 "bytes_per_launch": dom["bytes"]}
 
