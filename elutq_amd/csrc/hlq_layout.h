@@ -28,7 +28,7 @@
 #define HLQ_NUM_CU 256                 /* MI355X */
 #define HLQ_MAX_LDS (160 * 1024)       /* per workgroup on gfx950 */
 #define HLQ_WS_COUNTER_BYTES (64 * 1024) /* head of every workspace: one arrival counter per column block */
-#define HLQ_GEMM_CH 4                  /* units staged per chunk = waves per GEMM workgroup */
+#define HLQ_GEMM_WAVES 8               /* waves per GEMM workgroup */
 
 struct HlqGeo {
     int K, N, bits, group;
@@ -55,22 +55,27 @@ static inline size_t hlq_planes_bytes(const HlqGeo &g) { return (size_t)g.ncb * 
 static inline size_t hlq_scales_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * g.bits * HLQ_CB * 4; }
 static inline size_t hlq_zeros_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * HLQ_CB * 4; }
 
-// K slices the GEMM launcher uses for a shape: about one workgroup per CU, whole chunks.
-static inline void hlq_gemm_split(const HlqGeo &g, int &ksplit, int &ups)
+// Launch shape of the small-batch GEMM.  A workgroup has HLQ_GEMM_WAVES waves arranged as
+// (HLQ_GEMM_WAVES / kw) column blocks x kw K parts; a step consumes kw units (one per K part).
+// K is further cut into ksplit slices of ups units (whole steps) handled by different
+// workgroups, about one workgroup per CU in total.
+static inline void hlq_gemm_shape(const HlqGeo &g, int &kw, int &ksplit, int &ups)
 {
-    int ks = 2 * HLQ_NUM_CU / g.ncb;                     // at most two workgroups per CU, all resident at once
-    const int most = (g.U + HLQ_GEMM_CH - 1) / HLQ_GEMM_CH;
-    if (ks > most) ks = most;
+    if (kw != 2 && kw != 4) kw = 4;
+    const int cbw = HLQ_GEMM_WAVES / kw;
+    const int nsb = (g.ncb + cbw - 1) / cbw;                 // workgroups along N
+    const int steps = (g.U + kw - 1) / kw;                   // steps over all of K
+    int ks = ksplit > 0 ? ksplit : (HLQ_NUM_CU + nsb / 2) / nsb;
+    if (ks > steps) ks = steps;
     if (ks < 1) ks = 1;
-    ups = (g.U + ks - 1) / ks;
-    ups = (ups + HLQ_GEMM_CH - 1) / HLQ_GEMM_CH * HLQ_GEMM_CH;
+    ups = (steps + ks - 1) / ks * kw;
     ksplit = (g.U + ups - 1) / ups;
 }
 
 static inline size_t hlq_gemm_ws_bytes(const HlqGeo &g, int M)
 {
-    int ks, ups;
-    hlq_gemm_split(g, ks, ups);
+    int kw = 0, ks = 0, ups;
+    hlq_gemm_shape(g, kw, ks, ups);
     const int mpad = M <= 32 ? 32 : 64;
     return (size_t)HLQ_WS_COUNTER_BYTES + (ks > 1 ? (size_t)ks * mpad * g.ncb * HLQ_CB * sizeof(float) : 0);
 }

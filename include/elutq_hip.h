@@ -140,6 +140,20 @@ int elutq_hlq_gemm_f16(const void *d_planes, const void *d_scales, const void *d
                        void *d_workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Same computation with the launch shape chosen by the caller: `kparts` K parts inside a
+ * workgroup (2 or 4; the workgroup then covers 8 / kparts column blocks of 64) and
+ * `ksplit` K slices across workgroups (1..K/128); 0 = library default.  The workspace
+ * must hold 64 KiB + ksplit * (M <= 32 ? 32 : 64) * ceil(N/64)*64 * 4 bytes when the shape
+ * ends up with more than one slice.  For tuning and for tests that must reach every
+ * reduction path; results do not depend on these beyond fp32 summation order.
+ */
+int elutq_hlq_gemm_f16_tuned(const void *d_planes, const void *d_scales, const void *d_zeros,
+                             const void *d_bias, const void *d_x, void *d_y,
+                             int M, int K, int N, int bits, int group,
+                             void *d_workspace, size_t workspace_bytes, void *stream,
+                             int kparts, int ksplit);
+
+/*
  * Decode-step glue between the q|k|v projection and the o projection, one launch per layer:
  * half-split RoPE on q and k at position *d_pos, append of k and v to the caches at that
  * position, single-token grouped-query attention over positions 0..*d_pos, fp16 output

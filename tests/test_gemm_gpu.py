@@ -70,3 +70,50 @@ def test_llama2_13b_prefill_shapes(cuda, m, k, n):
     w = O.dequantize(L.w_quant, L.w_scale, L.w_zero, 128, np.float32)
     ref = L.x.astype(np.float64) @ w.astype(np.float64).T
     assert O.rel_err(y, ref) <= TOL
+
+
+@pytest.mark.parametrize("kparts", [2, 4])
+@pytest.mark.parametrize("ksplit", [1, 2, 3, 0])
+@pytest.mark.parametrize("m,k,n,bits,group", [(16, 1024, 100, 2, 128), (64, 1280, 320, 2, 128), (40, 1152, 576, 3, 64),
+                                               (7, 896, 64, 4, 128), (33, 640, 200, 1, 64)])
+def test_gemm_every_launch_shape(cuda, kparts, ksplit, m, k, n, bits, group):
+    """Every arrangement of a workgroup (K parts x column blocks) and of the K slices across
+    workgroups, including column blocks past N, slices of unequal length and steps only some
+    K parts take part in, against the float64 oracle; a second call on the same workspace
+    must give the same bits (arrival counters are left at zero)."""
+    from elutq_amd import _lib
+    L = make_layer(k, n, bits=bits, group=group, m=m, seed=k + n + kparts, bias=True)
+    mod = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, L.group, L.bias, cuda)
+    x = torch.from_numpy(L.x).to(cuda)
+    ncb = -(-n // 64)
+    ws = torch.zeros(64 * 1024 + (k // 128) * 64 * ncb * 64 * 4, dtype=torch.uint8, device=cuda)
+    ref = O.gemm_f64(L.x, L.w_quant, L.w_scale, L.w_zero, group, L.bias)
+    outs = []
+    for _ in range(2):
+        y = torch.full((m, n), float("nan"), dtype=torch.float16, device=cuda)
+        rc = _lib.lib().elutq_hlq_gemm_f16_tuned(mod.planes.data_ptr(), mod.scales.data_ptr(), mod.zeros.data_ptr(),
+                                                 mod.bias.data_ptr(), x.data_ptr(), y.data_ptr(), m, k, n, bits, group,
+                                                 ws.data_ptr(), ws.numel(), torch.cuda.current_stream().cuda_stream,
+                                                 kparts, ksplit)
+        assert rc == 0
+        torch.cuda.synchronize()
+        outs.append(y.cpu().numpy())
+    assert O.rel_err(outs[0], ref) <= TOL
+    assert np.array_equal(outs[0], outs[1])
+
+
+def test_gemm_tuned_rejects_bad_shapes(cuda):
+    from elutq_amd import _lib
+    L = make_layer(512, 64, bits=2, group=128, m=4, seed=1)
+    mod = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, L.group, None, cuda)
+    x = torch.from_numpy(L.x).to(cuda)
+    y = torch.empty(4, 64, dtype=torch.float16, device=cuda)
+    ws = torch.zeros(64 * 1024, dtype=torch.uint8, device=cuda)
+    call = lambda kp, ks, wsb: _lib.lib().elutq_hlq_gemm_f16_tuned(
+        mod.planes.data_ptr(), mod.scales.data_ptr(), mod.zeros.data_ptr(), None, x.data_ptr(), y.data_ptr(), 4, 512, 64,
+        2, 128, ws.data_ptr(), wsb, torch.cuda.current_stream().cuda_stream, kp, ks)
+    assert call(3, 0, ws.numel()) == -7          # K parts must be 2 or 4
+    assert call(4, 5, ws.numel()) == -7          # more slices than units
+    assert call(2, 2, ws.numel()) == -5          # two slices need room for partial sums
+    assert call(4, 1, 0) == 0                    # one slice needs no workspace
+    torch.cuda.synchronize()
