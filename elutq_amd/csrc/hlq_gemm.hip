@@ -224,11 +224,15 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
                 split_tiles(cur.w[b].z, cur.w[b].w, tw[b][0][1], tw[b][1][1]);
             }
             split_tiles(cur.zz, cur.zz, zzj[0], zzj[1]);
-            // A operands are read one MFMA step ahead of their use
+            // A operands are read two MFMA steps ahead of their use (three rotating registers sets);
+            // scheduling barriers between the steps keep the compiler from sinking the reads
             const _Float16 *arow = xl + (size_t)col * ROW_HALFS + kp * HLQ_UNIT + h * 32;
-            half8 aop[2][MT];
+            half8 aop[3][MT];
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) aop[0][mt] = *(const half8 *)(arow + (size_t)mt * 32 * ROW_HALFS);
+            for (int st = 0; st < 2; st++)
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++)
+                    aop[st][mt] = *(const half8 *)(arow + (size_t)mt * 32 * ROW_HALFS + (st >> 2) * 64 + (st & 3) * 8);
 #pragma unroll
             for (int pr = 0; pr < 2; pr++) {          // 64-k pair of dwords: k = 64pr + 32h + ...
                 const bool hi = G64 ? pr == 1 : (u & 1) != 0;       // fp16 of the meta dwords this pair belongs to
@@ -250,16 +254,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
 #pragma unroll
                 for (int s = 0; s < 4; s++) {
                     const int st = pr * 4 + s;        // step 0..7 of the unit
-                    if (st < 7) {
-                        const int nx = st + 1;
+                    if (st < 6) {
+                        const int nx = st + 2;
 #pragma unroll
                         for (int mt = 0; mt < MT; mt++)
-                            aop[nx & 1][mt] = *(const half8 *)(arow + (size_t)mt * 32 * ROW_HALFS + (nx >> 2) * 64 + (nx & 3) * 8);
+                            aop[nx % 3][mt] = *(const half8 *)(arow + (size_t)mt * 32 * ROW_HALFS + (nx >> 2) * 64 + (nx & 3) * 8);
                     }
+                    // planes outermost: consecutive MFMAs then go to different accumulators
 #pragma unroll
-                    for (int j = 0; j < 2; j++)
+                    for (int b = 0; b < BITS; b++)
 #pragma unroll
-                        for (int b = 0; b < BITS; b++) {
+                        for (int j = 0; j < 2; j++) {
                             uint32_t o[4];
 #pragma unroll
                             for (int q = 0; q < 4; q++) {
@@ -272,8 +277,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
                             const half8 bop = __builtin_bit_cast(half8, make_uint4(o[0], o[1], o[2], o[3]));
 #pragma unroll
                             for (int mt = 0; mt < MT; mt++)
-                                acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[st & 1][mt], bop, acc[mt][j], 0, 0, 0);
+                                acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[st % 3][mt], bop, acc[mt][j], 0, 0, 0);
                         }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 // centre term: c[n, g] * sum_{k in g} x[m, k]; C rows of register i: 8*(i/4) + 4h + i%4
                 if (G64 || pr == 1) {
