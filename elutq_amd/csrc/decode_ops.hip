@@ -9,6 +9,7 @@
 #include <stdint.h>
 
 #include "../../include/elutq_hip.h"
+#include "hlq_layout.h"
 
 namespace {
 
@@ -19,7 +20,12 @@ struct AttnArgs {
     uint16_t *out;           // fp16 [nq*d]
     int nq, nkv, d, max_seq;
     float log2_base;
+    int splits;              // workgroups per query head (head_dim 128 only)
+    float *partial;          // [nq][splits][d + 2] unnormalised output, running max, running sum
+    unsigned *counters;      // [nq] arrival counters, zero between launches
 };
+
+constexpr int ATTN_MAX_SPLITS = 8;
 
 __device__ __forceinline__ float h2f(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
 __device__ __forceinline__ uint16_t f2h(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
@@ -40,6 +46,17 @@ __device__ __forceinline__ float wave_sum(float v)
     v += __shfl_xor(v, 32, 64);
     return v;
 }
+
+#ifdef HLQ_TIMING
+// Profiling builds only: wall-clock stamps (100 MHz) of thread 0 of every workgroup.
+__device__ unsigned long long *g_attn_stamps = nullptr;
+#define ATTN_STAMP(i)                                                                                  \
+    do {                                                                                               \
+        if (g_attn_stamps && threadIdx.x == 0 && (i) < 16) g_attn_stamps[(size_t)blockIdx.x * 16 + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define ATTN_STAMP(i) do { } while (0)
+#endif
 
 constexpr int ATTN_WAVES = 4;
 constexpr int ATTN_UNROLL = 4;
@@ -135,11 +152,12 @@ __global__ __launch_bounds__(ATTN_WAVES * 64) void rope_attn_kernel(const AttnAr
 // 8 dims (one dwordx4 per lane, 1 KiB contiguous per kv head row group); the 16 lanes of a
 // DPP row reduce their partial dot products among themselves, so no LDS permutes are
 // needed, and every (wave, row) pair runs its own running-max softmax stream over the
-// positions it sees.  Batches of FAST_BATCH row groups are loaded before any is used.
+// positions it sees (one running-max update per batch); the four streams of a wave are
+// merged with wave shuffles, the waves through LDS.  Batches of FAST_BATCH row groups are
+// loaded before any is used, the first one before the position is even known (4 * FAST_WAVES *
+// FAST_BATCH = 256 rows).
 // ---------------------------------------------------------------------------------------
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-constexpr int FAST_WAVES = 8;
-constexpr int FAST_BATCH = 8;
 constexpr int FAST_D = 128;
 
 __device__ __forceinline__ float dot8(const uint4 &q, const uint4 &k)
@@ -171,99 +189,227 @@ __device__ __forceinline__ void stream_update(float s, bool valid, const uint4 &
     m = mx;
 }
 
-__global__ __launch_bounds__(FAST_WAVES * 64) void rope_attn_d128_kernel(const AttnArgs a)
+// WAVES x BATCH x 4 rows form a block; split sp of S takes blocks sp, sp + S, ... of the cached
+// positions.  S > 1: the splits of a head meet in device memory (unnormalised fp32 output,
+// running max and sum per split; agent-scope stores, arrival ticket, the last workgroup of the
+// head merges the splits in order), as the K slices of the GEMV do.
+template <int WAVES, int BATCH>
+__global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnArgs a)
 {
-    constexpr int D = FAST_D, HALF = D / 2, STREAMS = FAST_WAVES * 4;
+    constexpr int D = FAST_D, HALF = D / 2, BLOCK_ROWS = WAVES * BATCH * 4;
     __shared__ __align__(16) uint16_t sq[D], sk[D], sv[D];
-    __shared__ float sm_m[STREAMS], sm_l[STREAMS];
-    __shared__ float sm_o[STREAMS][D];
+    __shared__ float sm_m[WAVES], sm_l[WAVES];
+    __shared__ float sm_o[WAVES][D];
+    __shared__ unsigned s_ticket;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int h = blockIdx.x, grp = a.nq / a.nkv, g = h / grp;
-    const int pos = (int)*a.pos;
-    if (pos < 0 || pos >= a.max_seq) return;
+    const int S = a.splits;
+    const int h = blockIdx.x / S, sp = blockIdx.x - h * S, grp = a.nq / a.nkv, g = h / grp;
+    const int seg = lane & 15, r = lane >> 4;
+
+    // Everything the kernel needs from memory first is requested before anything is waited for:
+    // the first block of cache rows (row numbers clamped by the cache size, not by the position,
+    // so the addresses do not depend on *pos; rows at or beyond it are masked later), q and the
+    // new k / v, and the position itself.  One memory round trip instead of three dependent ones.
+    ATTN_STAMP(0);
+    const long long pos64 = *a.pos;
+    uint4 kk[BATCH], vv[BATCH];
+#pragma unroll
+    for (int b = 0; b < BATCH; b++) {
+        const int p = min(sp * BLOCK_ROWS + (wave + WAVES * b) * 4 + r, a.max_seq - 1);
+        const size_t row = ((size_t)p * a.nkv + g) * D;
+        kk[b] = ((const uint4 *)(a.kc + row))[seg];
+        vv[b] = ((const uint4 *)(a.vc + row))[seg];
+    }
+    // every wave loads the rotary pair (lane, lane + 64) of q, k and v (only wave 0 uses it):
+    // unconditional, so that nothing is converted -- and therefore waited for -- in between
+    const uint16_t *qp = a.qkv + (size_t)h * D, *kp = a.qkv + (size_t)a.nq * D + (size_t)g * D;
+    const uint16_t *vp = a.qkv + (size_t)(a.nq + a.nkv) * D + (size_t)g * D;
+    const uint16_t qa16 = qp[lane], qb16 = qp[lane + HALF], ka16 = kp[lane], kb16 = kp[lane + HALF];
+    const uint16_t va16 = vp[lane], vb16 = vp[lane + HALF];
+    asm volatile("" ::: "memory");
+    const int pos = (int)pos64;
+    if (pos64 < 0 || pos64 >= a.max_seq) return;
+    ATTN_STAMP(1);
 
     if (tid < HALF) {                                    // rotary pair (tid, tid + 64) of q and of the new k
         const int j = tid;
         const float inv_freq = exp2f(-(float)(2 * j) / (float)D * a.log2_base);
         float sn, cs;
         __sincosf((float)pos * inv_freq, &sn, &cs);
-        const uint16_t *qp = a.qkv + (size_t)h * D, *kp = a.qkv + (size_t)a.nq * D + (size_t)g * D;
-        const uint16_t *vp = a.qkv + (size_t)(a.nq + a.nkv) * D + (size_t)g * D;
-        const float qa = h2f(qp[j]), qb = h2f(qp[j + HALF]), ka = h2f(kp[j]), kb = h2f(kp[j + HALF]);
+        const float qa = h2f(qa16), qb = h2f(qb16), ka = h2f(ka16), kb = h2f(kb16);
         sq[j] = f2h(qa * cs - qb * sn); sq[j + HALF] = f2h(qb * cs + qa * sn);
         sk[j] = f2h(ka * cs - kb * sn); sk[j + HALF] = f2h(kb * cs + ka * sn);
-        sv[j] = vp[j]; sv[j + HALF] = vp[j + HALF];
+        sv[j] = va16; sv[j + HALF] = vb16;
     }
     __syncthreads();
-    if (h % grp == 0 && tid < D / 8) {                   // one workgroup per kv head appends the new row
+    if (h % grp == 0 && sp == 0 && tid < D / 8) {        // one workgroup per kv head appends the new row
         const size_t row = ((size_t)pos * a.nkv + g) * D;
         ((uint4 *)(a.kc + row))[tid] = ((const uint4 *)sk)[tid];
         ((uint4 *)(a.vc + row))[tid] = ((const uint4 *)sv)[tid];
     }
 
-    const int seg = lane & 15, r = lane >> 4;
+    ATTN_STAMP(2);
     const uint4 qv = ((const uint4 *)sq)[seg];
     const float scale = rsqrtf((float)D);
-    const int ngroups = (pos + 3) >> 2;                  // row groups of the cached positions 0..pos-1
+    int stamp_i = 3;
+    (void)stamp_i;
     float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.f;
 
-    for (int gb = wave; gb < ngroups; gb += FAST_WAVES * FAST_BATCH) {
-        uint4 kk[FAST_BATCH], vv[FAST_BATCH];
-        bool ok[FAST_BATCH];
+    for (int blk = sp; blk * BLOCK_ROWS < pos; blk += S) {
+        const int base = blk * BLOCK_ROWS;
+        if (blk != sp) {                                 // later blocks of a long context
 #pragma unroll
-        for (int b = 0; b < FAST_BATCH; b++) {
-            const int p = (gb + FAST_WAVES * b) * 4 + r;
-            ok[b] = p < pos;
-            const size_t row = ((size_t)(ok[b] ? p : 0) * a.nkv + g) * D;
-            kk[b] = ((const uint4 *)(a.kc + row))[seg];
-            vv[b] = ((const uint4 *)(a.vc + row))[seg];
+            for (int b = 0; b < BATCH; b++) {
+                const int p = min(base + (wave + WAVES * b) * 4 + r, a.max_seq - 1);
+                const size_t row = ((size_t)p * a.nkv + g) * D;
+                kk[b] = ((const uint4 *)(a.kc + row))[seg];
+                vv[b] = ((const uint4 *)(a.vc + row))[seg];
+            }
+            // keep the whole batch of loads ahead of the first use (the scheduler would otherwise
+            // sink each load to its consumer and serialise the memory round trips)
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
         }
-        // keep the whole batch of loads ahead of the first use (the scheduler would otherwise
-        // sink each load to its consumer and serialise the memory round trips)
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
+        // one running-max update per batch: scores first, then a single rescale of the stream
+        float sc[BATCH], mx = m;
 #pragma unroll
-        for (int b = 0; b < FAST_BATCH; b++) {
-            const float s = dot8(qv, kk[b]) * scale;
-            stream_update(s, ok[b], vv[b], m, l, acc);
+        for (int b = 0; b < BATCH; b++) {
+            const bool ok = base + (wave + WAVES * b) * 4 + r < pos;
+            sc[b] = ok ? dot8(qv, kk[b]) * scale : -INFINITY;
+            mx = fmaxf(mx, sc[b]);
         }
+        if (mx > -INFINITY) {                            // uniform per 16-lane stream; false only if no row was valid yet
+            const float corr = __expf(m - mx);
+            l *= corr;
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[i] *= corr;
+#pragma unroll
+            for (int b = 0; b < BATCH; b++) {
+                const float e = __expf(sc[b] - mx);
+                const uint32_t w[4] = {vv[b].x, vv[b].y, vv[b].z, vv[b].w};
+                l += e;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    acc[2 * i] = fmaf(e, h2f((uint16_t)(w[i] & 0xffffu)), acc[2 * i]);
+                    acc[2 * i + 1] = fmaf(e, h2f((uint16_t)(w[i] >> 16)), acc[2 * i + 1]);
+                }
+            }
+            m = mx;
+        }
+        ATTN_STAMP(stamp_i); stamp_i++;
     }
-    if (wave == 0) {                                     // the token being decoded, from LDS (row 0 only)
+    if (wave == 0 && sp == 0) {                          // the token being decoded, from LDS (row 0 only)
         const float s = dot8(qv, ((const uint4 *)sk)[seg]) * scale;
         stream_update(s, r == 0, ((const uint4 *)sv)[seg], m, l, acc);
     }
-    const int stream = wave * 4 + r;
-    if (seg == 0) { sm_m[stream] = m; sm_l[stream] = l; }
+    // merge the four row streams of the wave (lanes 16 and 32 apart), then the waves through LDS
 #pragma unroll
-    for (int i = 0; i < 8; i++) sm_o[stream][seg * 8 + i] = acc[i];
+    for (int sh = 16; sh <= 32; sh <<= 1) {
+        const float m2 = __shfl_xor(m, sh, 64), l2 = __shfl_xor(l, sh, 64);
+        const float mx = fmaxf(m, m2);
+        const float f1 = (m == mx) ? 1.f : __expf(m - mx), f2 = (m2 == mx) ? 1.f : __expf(m2 - mx);
+        l = l * f1 + l2 * f2;
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = acc[i] * f1 + __shfl_xor(acc[i], sh, 64) * f2;
+        m = mx;
+    }
+    if (lane == 0) { sm_m[wave] = m; sm_l[wave] = l; }
+    if (r == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) sm_o[wave][seg * 8 + i] = acc[i];
+    }
+    ATTN_STAMP(12);
     __syncthreads();
+    ATTN_STAMP(13);
+    float M = -INFINITY, L = 0.f, o = 0.f;               // this split's result for dimension tid
     if (tid < D) {
-        float M = -INFINITY;
 #pragma unroll
-        for (int s = 0; s < STREAMS; s++) M = fmaxf(M, sm_m[s]);
-        float L = 0.f, o = 0.f;
+        for (int s = 0; s < WAVES; s++) M = fmaxf(M, sm_m[s]);
 #pragma unroll
-        for (int s = 0; s < STREAMS; s++) {
-            const float f = __expf(sm_m[s] - M);
+        for (int s = 0; s < WAVES; s++) {
+            const float f = (sm_m[s] == M) ? 1.f : __expf(sm_m[s] - M);
             L = fmaf(sm_l[s], f, L);
             o = fmaf(sm_o[s][tid], f, o);
         }
-        a.out[(size_t)h * D + tid] = f2h(o / L);
     }
+    if (S == 1) {
+        if (tid < D) a.out[(size_t)h * D + tid] = f2h(o / L);
+        ATTN_STAMP(14);
+        return;
+    }
+    float *po = a.partial + ((size_t)h * S + sp) * (D + 2);
+    if (tid < D) __hip_atomic_store(&po[tid], o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) {
+        __hip_atomic_store(&po[D], M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&po[D + 1], L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) s_ticket = __hip_atomic_fetch_add(&a.counters[h], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != (unsigned)S - 1u) return;
+    if (tid < D) {
+        // all loads of the merge are issued before the first is used
+        float pm[ATTN_MAX_SPLITS], pl[ATTN_MAX_SPLITS], pv[ATTN_MAX_SPLITS];
+#pragma unroll
+        for (int s = 0; s < ATTN_MAX_SPLITS; s++) {
+            const float *ps = a.partial + ((size_t)h * S + min(s, S - 1)) * (D + 2);
+            pv[s] = __hip_atomic_load(&ps[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            pm[s] = __hip_atomic_load(&ps[D], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            pl[s] = __hip_atomic_load(&ps[D + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        float MM = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < ATTN_MAX_SPLITS; s++)
+            if (s < S) MM = fmaxf(MM, pm[s]);
+        float LL = 0.f, oo = 0.f;
+#pragma unroll
+        for (int s = 0; s < ATTN_MAX_SPLITS; s++)
+            if (s < S) {
+                const float f = (pm[s] == MM) ? 1.f : __expf(pm[s] - MM);
+                LL = fmaf(pl[s], f, LL);
+                oo = fmaf(pv[s], f, oo);
+            }
+        a.out[(size_t)h * D + tid] = f2h(oo / LL);
+    }
+    if (tid == 0) __hip_atomic_store(&a.counters[h], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ATTN_STAMP(14);
 }
 
 }  // namespace
 
-extern "C" int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,
-                                          void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,
-                                          float rope_base, void *stream)
+extern "C" size_t elutq_decode_attn_workspace_bytes(int n_heads, int head_dim, int splits)
+{
+    if (n_heads < 1 || head_dim < 2 || splits < 0 || splits > ATTN_MAX_SPLITS) return 0;
+    const int s = splits == 0 ? ATTN_MAX_SPLITS : splits;
+    return (size_t)HLQ_WS_COUNTER_BYTES + (size_t)n_heads * s * (head_dim + 2) * sizeof(float);
+}
+
+#ifdef HLQ_TIMING
+extern "C" int elutq_debug_set_attn_stamps(void *d_buf)
+{
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_attn_stamps), &d_buf, sizeof(d_buf)) == hipSuccess ? 0 : -1;
+}
+#endif
+
+extern "C" int elutq_decode_rope_attn_split_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,
+                                                void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                                                float rope_base, int splits, void *d_workspace, size_t workspace_bytes,
+                                                void *stream)
 {
     if (!d_qkv || !d_k_cache || !d_v_cache || !d_pos || !d_out) return ELUTQ_ERR_NULL;
     if (n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads != 0 || head_dim < 2 || head_dim > 128 ||
         head_dim % 2 != 0 || max_seq < 1 || !(rope_base > 1.f))
         return ELUTQ_ERR_SHAPE;
+    if (splits < 0 || splits > ATTN_MAX_SPLITS) return ELUTQ_ERR_TUNING;
+    if (splits == 0) {                                   // default: about one workgroup per CU, if there is a workspace
+        splits = d_workspace ? HLQ_NUM_CU / n_heads : 1;
+        if (splits > ATTN_MAX_SPLITS) splits = ATTN_MAX_SPLITS;
+        if (splits < 1) splits = 1;
+    }
+    if (head_dim != FAST_D) splits = 1;
     AttnArgs a;
     a.qkv = (const uint16_t *)d_qkv;
     a.kc = (uint16_t *)d_k_cache;
@@ -272,9 +418,27 @@ extern "C" int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, vo
     a.out = (uint16_t *)d_out;
     a.nq = n_heads; a.nkv = n_kv_heads; a.d = head_dim; a.max_seq = max_seq;
     a.log2_base = log2f(rope_base);
-    if (head_dim == FAST_D)
-        hipLaunchKernelGGL(rope_attn_d128_kernel, dim3(n_heads), dim3(FAST_WAVES * 64), 0, (hipStream_t)stream, a);
-    else
+    a.splits = splits; a.partial = nullptr; a.counters = nullptr;
+    if (splits > 1) {
+        if (!d_workspace) return ELUTQ_ERR_NULL;
+        if ((size_t)n_heads * sizeof(unsigned) > (size_t)HLQ_WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
+        if (workspace_bytes < elutq_decode_attn_workspace_bytes(n_heads, head_dim, splits)) return ELUTQ_ERR_WORKSPACE;
+        a.counters = (unsigned *)d_workspace;
+        a.partial = (float *)((unsigned char *)d_workspace + HLQ_WS_COUNTER_BYTES);
+    }
+    if (head_dim != FAST_D)
         hipLaunchKernelGGL(rope_attn_kernel, dim3(n_heads), dim3(ATTN_WAVES * 64), 0, (hipStream_t)stream, a);
+    else if (splits == 1)
+        hipLaunchKernelGGL((rope_attn_d128_kernel<8, 8>), dim3(n_heads), dim3(8 * 64), 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL((rope_attn_d128_kernel<4, 4>), dim3(n_heads * splits), dim3(4 * 64), 0, (hipStream_t)stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
+}
+
+extern "C" int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,
+                                          void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                                          float rope_base, void *stream)
+{
+    return elutq_decode_rope_attn_split_f16(d_qkv, d_k_cache, d_v_cache, d_pos, d_out, n_heads, n_kv_heads, head_dim,
+                                            max_seq, rope_base, 1, nullptr, 0, stream);
 }

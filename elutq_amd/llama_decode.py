@@ -140,10 +140,11 @@ def fused_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tensor) 
     rmsnorm+gate|up | silu*up+down+residual.  The residual stream enters and leaves in b.xa."""
     s = layer.s
     layer.qkv.gemv_fused(b.xa, b.qkv, b.ws, prologue=1, norm_weight=layer.ln1, eps=s.rms_eps)
-    rc = _lib.lib().elutq_decode_rope_attn_f16(
+    rc = _lib.lib().elutq_decode_rope_attn_split_f16(
         b.qkv.data_ptr(), layer.k_cache.data_ptr(), layer.v_cache.data_ptr(), pos.data_ptr(), b.attn.data_ptr(),
-        s.n_heads, s.n_kv_heads, s.head_dim, s.max_seq, s.rope_base, torch.cuda.current_stream().cuda_stream)
-    _lib.check(rc, "elutq_decode_rope_attn_f16")
+        s.n_heads, s.n_kv_heads, s.head_dim, s.max_seq, s.rope_base, 0, b.ws.data_ptr(), b.ws.numel(),
+        torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "elutq_decode_rope_attn_split_f16")
     layer.o_proj.gemv_fused(b.attn, b.xb, b.ws, residual=b.xa)
     layer.gate_up.gemv_fused(b.xb, b.gu, b.ws, prologue=1, norm_weight=layer.ln2, eps=s.rms_eps)
     layer.down_proj.gemv_fused(b.gu, b.xa, b.ws, prologue=2, residual=b.xb)
@@ -197,6 +198,7 @@ class LlamaDecoder(nn.Module):
         self._buf = None
         if impl == "hip":
             ws = max(m.workspace_bytes for m in self.modules() if isinstance(m, HLQLinear))
+            ws = max(ws, _lib.lib().elutq_decode_attn_workspace_bytes(s.n_heads, s.head_dim, 0))
             self._buf = FusedBuffers(s, ws, dev)
 
     @torch.no_grad()

@@ -167,6 +167,21 @@ int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, void *d_v_cac
                                void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,
                                float rope_base, void *stream);
 
+/*
+ * The same operator with the cached positions of every head divided among `splits`
+ * workgroups (1..8; 0 = about one workgroup per CU), which meet in `d_workspace`
+ * (elutq_decode_attn_workspace_bytes(n_heads, head_dim, splits) bytes, zero-filled once like the
+ * GEMV workspace, which it may share: calls on one stream leave its counters at zero).  One
+ * compute unit takes in a cache of a few hundred rows no faster than the whole chip takes in
+ * all heads', so long contexts want the split.  head_dim other than 128 runs unsplit.
+ * No counterpart in the reference beyond the operators elutq_decode_rope_attn_f16 replaces.
+ */
+size_t elutq_decode_attn_workspace_bytes(int n_heads, int head_dim, int splits);
+int elutq_decode_rope_attn_split_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,
+                                     void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                                     float rope_base, int splits, void *d_workspace, size_t workspace_bytes,
+                                     void *stream);
+
 /* W[N][K] fp16 row-major from the repacked buffers (dequantize_with_scales). */
 int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
                           void *d_w_out, int K, int N, int bits, int group, void *stream);

@@ -102,26 +102,42 @@ def test_graph_replay_equals_eager(cuda, impl):
     assert toks_e == toks_g and int(graph.pos) == 16
 
 
-@pytest.mark.parametrize("d,nq,nkv", [(128, 8, 2), (128, 4, 4), (64, 8, 2), (32, 4, 1)])
-@pytest.mark.parametrize("pos", [0, 1, 3, 4, 5, 37, 255, 300])
-def test_rope_cache_attention_kernel(cuda, d, nq, nkv, pos):
-    """elutq_decode_rope_attn_f16 against the PyTorch restatement of the reference ops
-    (half-split RoPE, cache append, fp32-softmax GQA attention)."""
+@pytest.mark.parametrize("d,nq,nkv,splits", [(128, 8, 2, 1), (128, 4, 4, 1), (64, 8, 2, 1), (32, 4, 1, 1),
+                                             (128, 8, 2, 2), (128, 8, 2, 8), (128, 32, 8, 0), (128, 4, 4, 3), (64, 8, 2, 4)])
+@pytest.mark.parametrize("pos", [0, 1, 3, 4, 5, 37, 63, 64, 65, 255, 300, 513, 1030])
+def test_rope_cache_attention_kernel(cuda, d, nq, nkv, splits, pos):
+    """elutq_decode_rope_attn_f16 / _split_f16 (cached positions divided among `splits`
+    workgroups per head, 0 = default) against the PyTorch restatement of the reference ops
+    (half-split RoPE, cache append, fp32-softmax GQA attention); two calls in a row on one
+    workspace (the second must find the arrival counters at zero)."""
     from elutq_amd import _lib
     from elutq_amd.llama_decode import rope
     g = torch.Generator(device=cuda).manual_seed(pos * 7 + d)
-    max_seq, base = 320, 10000.0
+    max_seq, base = 1100, 10000.0
+    L = _lib.lib()
     qkv = torch.randn(1, (nq + 2 * nkv) * d, generator=g, device=cuda).half()
     kc = torch.randn(max_seq, nkv, d, generator=g, device=cuda).half()
     vc = torch.randn(max_seq, nkv, d, generator=g, device=cuda).half()
     kc0, vc0 = kc.clone(), vc.clone()
-    out = torch.zeros(1, nq * d, dtype=torch.float16, device=cuda)
     pos_t = torch.tensor([pos], dtype=torch.long, device=cuda)
-    rc = _lib.lib().elutq_decode_rope_attn_f16(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), pos_t.data_ptr(),
-                                               out.data_ptr(), nq, nkv, d, max_seq, base,
-                                               torch.cuda.current_stream().cuda_stream)
-    assert rc == 0
-    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream().cuda_stream
+    ws = torch.zeros(L.elutq_decode_attn_workspace_bytes(nq, d, 0), dtype=torch.uint8, device=cuda)
+    outs = []
+    for _ in range(2):
+        out = torch.zeros(1, nq * d, dtype=torch.float16, device=cuda)
+        if splits == 1:
+            rc = L.elutq_decode_rope_attn_f16(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), pos_t.data_ptr(),
+                                              out.data_ptr(), nq, nkv, d, max_seq, base, stream)
+        else:
+            rc = L.elutq_decode_rope_attn_split_f16(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), pos_t.data_ptr(),
+                                                    out.data_ptr(), nq, nkv, d, max_seq, base, splits, ws.data_ptr(),
+                                                    ws.numel(), stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    assert not ws[:64 * 1024].any()
+    out = outs[0]
     # reference
     inv = base ** (-torch.arange(0, d, 2, device=cuda, dtype=torch.float32) / d)
     ang = pos * inv
