@@ -30,6 +30,8 @@ SIGNATURES = {
     "elutq_decode_rope_attn_f16": (_ci, [_vp] * 5 + [_ci] * 4 + [ctypes.c_float, _vp]),
     "elutq_decode_rope_attn_split_f16": (_ci, [_vp] * 5 + [_ci] * 4 + [ctypes.c_float, _ci, _vp, _sz, _vp]),
     "elutq_decode_attn_workspace_bytes": (_sz, [_ci] * 3),
+    "elutq_decode_rmsnorm_f16": (_ci, [_vp] * 3 + [_ci, ctypes.c_float, _vp]),
+    "elutq_decode_argmax_f16": (_ci, [_vp, _ci, _vp, _vp, _vp]),
     "elutq_hlq_gemm_f16": (_ci, [_vp] * 6 + [_ci] * 5 + [_vp, _sz, _vp]),
     "elutq_hlq_gemm_f16_tuned": (_ci, [_vp] * 6 + [_ci] * 5 + [_vp, _sz, _vp, _ci, _ci]),
     "elutq_hlq_dequant_f16": (_ci, [_vp] * 4 + [_ci] * 4 + [_vp]),

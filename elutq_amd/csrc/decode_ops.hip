@@ -378,6 +378,75 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     ATTN_STAMP(14);
 }
 
+// ---------------------------------------------------------------------------------------
+// Tail of the decode step: final RMSNorm in front of the lm_head and the greedy pick behind
+// it (launch_pre_rms_norm, C++/ops/src/arm/arm_rmsnorm.cpp:25-84: fp32 statistics, fp16
+// output; arm_argmax_last, C++/ops/src/arm/arm_argmax.cpp:3-30: first index of the strict
+// maximum).  One workgroup each: the vectors are a few KiB to a few hundred KiB.
+// ---------------------------------------------------------------------------------------
+constexpr int TAIL_THREADS = 1024;
+
+__global__ __launch_bounds__(TAIL_THREADS) void rmsnorm_kernel(const uint16_t *x, const uint16_t *w, uint16_t *out, int n,
+                                                               float eps)
+{
+    __shared__ float part[TAIL_THREADS / 64];
+    const int tid = threadIdx.x;
+    float ssq = 0.f;
+    for (int i = tid; i < n; i += TAIL_THREADS) {
+        const float v = h2f(x[i]);
+        ssq = fmaf(v, v, ssq);
+    }
+    ssq = wave_sum(ssq);
+    if ((tid & 63) == 0) part[tid >> 6] = ssq;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int i = 0; i < TAIL_THREADS / 64; i++) tot += part[i];
+    const float rstd = rsqrtf(tot / (float)n + eps);
+    for (int i = tid; i < n; i += TAIL_THREADS) out[i] = f2h(h2f(x[i]) * rstd * h2f(w[i]));
+}
+
+// (value, index) order of the greedy pick: larger value first, lower index among equals.
+__device__ __forceinline__ void pick(float &v, int &i, float v2, int i2)
+{
+    if (v2 > v || (v2 == v && i2 < i)) { v = v2; i = i2; }
+}
+
+__global__ __launch_bounds__(TAIL_THREADS) void argmax_kernel(const uint16_t *logits, int n, long long *token, long long *pos)
+{
+    __shared__ float sv[TAIL_THREADS / 64];
+    __shared__ int si[TAIL_THREADS / 64];
+    const int tid = threadIdx.x;
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    const bool aligned = ((uintptr_t)logits & 15) == 0;
+    const int nvec = aligned ? n / 8 : 0;
+    for (int c = tid; c < nvec; c += TAIL_THREADS) {     // 8 values per load; indices rise within a thread
+        const uint4 q = ((const uint4 *)logits)[c];
+        const uint32_t wd[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float lo = h2f((uint16_t)(wd[j] & 0xffffu)), hi = h2f((uint16_t)(wd[j] >> 16));
+            if (lo > best) { best = lo; idx = c * 8 + 2 * j; }
+            if (hi > best) { best = hi; idx = c * 8 + 2 * j + 1; }
+        }
+    }
+    for (int i = nvec * 8 + tid; i < n; i += TAIL_THREADS) {
+        const float v = h2f(logits[i]);
+        if (v > best) { best = v; idx = i; }
+    }
+#pragma unroll
+    for (int sh = 1; sh < 64; sh <<= 1) pick(best, idx, __shfl_xor(best, sh, 64), __shfl_xor(idx, sh, 64));
+    if ((tid & 63) == 0) { sv[tid >> 6] = best; si[tid >> 6] = idx; }
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+        for (int i = 1; i < TAIL_THREADS / 64; i++) pick(best, idx, sv[i], si[i]);
+        *token = idx == 0x7fffffff ? 0 : idx;            // nothing compared greater than -inf: the reference's initial 0
+        if (pos) *pos += 1;
+    }
+}
+
 }  // namespace
 
 extern "C" size_t elutq_decode_attn_workspace_bytes(int n_heads, int head_dim, int splits)
@@ -441,4 +510,22 @@ extern "C" int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, vo
 {
     return elutq_decode_rope_attn_split_f16(d_qkv, d_k_cache, d_v_cache, d_pos, d_out, n_heads, n_kv_heads, head_dim,
                                             max_seq, rope_base, 1, nullptr, 0, stream);
+}
+
+extern "C" int elutq_decode_rmsnorm_f16(const void *d_x, const void *d_weight, void *d_out, int n, float eps, void *stream)
+{
+    if (!d_x || !d_weight || !d_out) return ELUTQ_ERR_NULL;
+    if (n < 1) return ELUTQ_ERR_SHAPE;
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(TAIL_THREADS), 0, (hipStream_t)stream, (const uint16_t *)d_x,
+                       (const uint16_t *)d_weight, (uint16_t *)d_out, n, eps);
+    return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
+}
+
+extern "C" int elutq_decode_argmax_f16(const void *d_logits, int n, void *d_token, void *d_pos, void *stream)
+{
+    if (!d_logits || !d_token) return ELUTQ_ERR_NULL;
+    if (n < 1) return ELUTQ_ERR_SHAPE;
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(TAIL_THREADS), 0, (hipStream_t)stream, (const uint16_t *)d_logits, n,
+                       (long long *)d_token, (long long *)d_pos);
+    return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }

@@ -10,10 +10,12 @@ pairs (j, j + d/2) with theta = pos * base^(-2j/d) and no frequency rescaling
 (arm_rotary.cpp:31-46), fp32 softmax, GQA map h_kv = h * n_kv / n_q
 (arm_attention.cpp:199-274), SiLU*up in fp32 (arm_activation.cpp:36-49).
 
-Everything except the HLQ projections is plain PyTorch-ROCm glue; the step is captured in a
-HIP graph (token id and position live in device tensors), so one replay = one token.
-q|k|v and gate|up are fused along N, which in the kernel layout is a concatenation of the
-packed buffers.
+impl="hip": five fused launches per layer, final norm and greedy pick as kernels of the
+library, embedding gather and the fp16 lm_head (hipBLASLt) through PyTorch; impl="torch": the
+same model with PyTorch-ROCm ops around the HLQ projections (the parity partner).  The step
+is captured in a HIP graph (token id and position live in device tensors), so one replay =
+one token.  q|k|v and gate|up are fused along N, which in the kernel layout is a
+concatenation of the packed buffers.
 """
 from __future__ import annotations
 
@@ -133,6 +135,7 @@ class FusedBuffers:
         self.attn = torch.zeros(1, s.n_heads * d, **f16)
         self.gu = torch.zeros(1, 2 * s.ffn, **f16)
         self.ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=device)
+        self.logits = torch.zeros(1, s.vocab, **f16)
 
 
 def fused_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tensor) -> None:
@@ -229,6 +232,14 @@ class LlamaDecoder(nn.Module):
             mask = torch.where(self.arange <= self.pos, 0.0, float("-inf")).view(1, 1, -1)
             for layer in self.layers:
                 x = layer(x, self.pos, cos, sin, mask)
+        if self.impl == "hip":
+            L, stream = _lib.lib(), torch.cuda.current_stream().cuda_stream
+            _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), b.xb.data_ptr(), self.s.hidden,
+                                                  self.s.rms_eps, stream), "elutq_decode_rmsnorm_f16")
+            logits = torch.mm(b.xb, self.lm_head.t(), out=b.logits)
+            _lib.check(L.elutq_decode_argmax_f16(logits.data_ptr(), self.s.vocab, self.token.data_ptr(),
+                                                 self.pos.data_ptr(), stream), "elutq_decode_argmax_f16")
+            return logits
         logits = F.linear(rms_norm(x, self.norm, self.s.rms_eps), self.lm_head)
         self.token.copy_(logits.argmax(-1))
         self.pos.add_(1)
@@ -285,4 +296,6 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
             "model": f"LLaMA-3-8B-shaped random init, {s.n_layers} layers, HLQ w{s.bits}g{s.group}, fp16 lm_head",
             "glue": ("5 launches per layer (rmsnorm+qkv | rope+cache+attention | o+residual | rmsnorm+gate|up | "
                      "silu*up+down+residual), " if impl == "hip" else "PyTorch-ROCm ops around the HLQ GEMVs, ")
-                    + "torch embedding / final norm / hipBLASLt fp16 lm_head / argmax, one HIP graph per token"}
+                    + ("own final norm and argmax kernels, torch embedding gather, hipBLASLt fp16 lm_head, "
+                       if impl == "hip" else "torch embedding / final norm / hipBLASLt fp16 lm_head / argmax, ")
+                    + "one HIP graph per token"}

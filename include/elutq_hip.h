@@ -182,6 +182,16 @@ int elutq_decode_rope_attn_split_f16(const void *d_qkv, void *d_k_cache, void *d
                                      float rope_base, int splits, void *d_workspace, size_t workspace_bytes,
                                      void *stream);
 
+/*
+ * Tail of a decode step.  elutq_decode_rmsnorm_f16: out[i] = fp16(x[i] * rsqrt(mean(x^2) + eps)
+ * * weight[i]), statistics in fp32 (launch_pre_rms_norm, C++/ops/src/arm/arm_rmsnorm.cpp:25-84).
+ * elutq_decode_argmax_f16: *d_token (DEVICE int64) = first index of the strict maximum of the
+ * fp16 logits (arm_argmax_last, C++/ops/src/arm/arm_argmax.cpp:3-30; NaNs never win), and, if
+ * d_pos is not NULL, *d_pos (DEVICE int64) += 1 -- so a captured graph advances its own state.
+ */
+int elutq_decode_rmsnorm_f16(const void *d_x, const void *d_weight, void *d_out, int n, float eps, void *stream);
+int elutq_decode_argmax_f16(const void *d_logits, int n, void *d_token, void *d_pos, void *stream);
+
 /* W[N][K] fp16 row-major from the repacked buffers (dequantize_with_scales). */
 int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
                           void *d_w_out, int K, int N, int bits, int group, void *stream);

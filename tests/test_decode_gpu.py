@@ -173,3 +173,59 @@ def test_rope_attn_rejects_bad_arguments(cuda):
     assert L.elutq_decode_rope_attn_f16(t.data_ptr(), t.data_ptr(), t.data_ptr(), p.data_ptr(), out.data_ptr(), 4, 1, 64, 8, 1e4, s) == 0
     torch.cuda.synchronize()
     assert bool((out == 7).all())
+
+
+@pytest.mark.parametrize("n", [1, 7, 8, 4096, 128256, 128259])
+def test_argmax_kernel(cuda, n):
+    """elutq_decode_argmax_f16: first index of the strict maximum (arm_argmax.cpp:3-30), also
+    with the maximum repeated, at either end, in the unaligned tail, and with NaNs present;
+    the position counter is advanced by one."""
+    from elutq_amd import _lib
+    L = _lib.lib()
+    g = torch.Generator(device=cuda).manual_seed(n)
+    stream = torch.cuda.current_stream().cuda_stream
+    tok = torch.full((1,), -5, dtype=torch.long, device=cuda)
+    pos = torch.tensor([41], dtype=torch.long, device=cuda)
+    cases = [torch.randn(n, generator=g, device=cuda).half() for _ in range(3)]
+    t = cases[0].clone(); t[n - 1] = 60000.0; cases.append(t)                    # last element
+    t = cases[1].clone(); t[0] = 60000.0; cases.append(t)                        # first element
+    t = cases[2].clone(); t[n // 2:] = t.max(); cases.append(t)                  # a run of equal maxima
+    t = cases[0].clone(); t[::3] = float("nan"); cases.append(t)                 # NaNs never win
+    cases.append(torch.full((n,), float("-inf"), dtype=torch.float16, device=cuda))
+    for i, c in enumerate(cases):
+        assert L.elutq_decode_argmax_f16(c.data_ptr(), n, tok.data_ptr(), pos.data_ptr(), stream) == 0
+        torch.cuda.synchronize()
+        v = c.float().cpu().numpy()
+        best, want = float("-inf"), 0
+        for j in range(n):                                                       # the reference's loop
+            if v[j] > best:
+                best, want = v[j], j
+        assert int(tok) == want, (i, n)
+        assert int(pos) == 42 + i
+    # unaligned pointer: same answer through the scalar path
+    if n > 9:
+        c = cases[0]
+        assert L.elutq_decode_argmax_f16(c.data_ptr() + 2, n - 1, tok.data_ptr(), None, stream) == 0
+        torch.cuda.synchronize()
+        assert int(tok) == int(c[1:].float().argmax())
+    assert L.elutq_decode_argmax_f16(None, n, tok.data_ptr(), None, stream) == -1
+    assert L.elutq_decode_argmax_f16(cases[0].data_ptr(), 0, tok.data_ptr(), None, stream) == -2
+
+
+@pytest.mark.parametrize("n", [64, 4096, 5120, 1000])
+def test_final_rmsnorm_kernel(cuda, n):
+    """elutq_decode_rmsnorm_f16 against the fp32 restatement of arm_rmsnorm.cpp:25-84."""
+    from elutq_amd import _lib
+    from elutq_amd.llama_decode import rms_norm
+    g = torch.Generator(device=cuda).manual_seed(n)
+    x = (torch.randn(1, n, generator=g, device=cuda) * 3).half()
+    w = (1 + 0.1 * torch.randn(n, generator=g, device=cuda)).half()
+    out = torch.zeros(1, n, dtype=torch.float16, device=cuda)
+    rc = _lib.lib().elutq_decode_rmsnorm_f16(x.data_ptr(), w.data_ptr(), out.data_ptr(), n, 1e-5,
+                                             torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    ref = rms_norm(x, w, 1e-5)
+    # same formula, different fp32 summation order: at most one fp16 ulp apart
+    assert (out.float() - ref.float()).abs().max() <= 2.0 ** -10 * ref.float().abs().max()
+    assert (out != ref).float().mean() < 0.02
