@@ -96,3 +96,80 @@ def read_export_dir(path: str, groupsize: int | None = None) -> ExportedLinear:
                           w_quant=w_quant.reshape(bits, n, k // 8),
                           w_scale=w_scale.reshape(bits, n, k // group),
                           w_zero=w_zero.reshape(n, k // group), bias=bias)
+
+
+# ---------------------------------------------------------------------------------------
+# Whole-model export tree (GPTQ/llama.py:285-343 writes it, C++/examples/models/llama.cpp:59-115
+# reads it): fp16 raw binaries next to the per-layer linear directories.
+#
+#   <root>/embed_tokens.bin               fp16 [vocab][hidden]   (shared_embed_lm_head.bin when the
+#                                                                 exporter found tied embeddings)
+#   <root>/lm_head.bin                    fp16 [vocab][hidden]   or <root>/lm_head/lm_head/ (HLQ)
+#   <root>/final_rmsnorm_weight.bin       fp16 [hidden]
+#   <root>/<i>/input_layernorm_weight.bin, post_attention_layernorm_weight.bin   fp16 [hidden]
+#   <root>/<i>/self_attn.{q,k,v,o}_proj/, mlp.{gate,up,down}_proj/               linear directories
+# ---------------------------------------------------------------------------------------
+LAYER_LINEARS = ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj",
+                 "mlp.gate_proj", "mlp.up_proj", "mlp.down_proj")
+LAYER_NORMS = ("input_layernorm_weight.bin", "post_attention_layernorm_weight.bin")
+REPACKED_JSON = "repacked.json"
+REPACK_LAYOUT_VERSION = 1
+
+
+def write_fp16_bin(path: str, a) -> None:
+    os.makedirs(os.path.dirname(path) or ".", exist_ok=True)
+    with open(path, "wb") as f:
+        f.write(np.ascontiguousarray(a, dtype=np.float16).tobytes())
+
+
+def read_fp16_bin(path: str, count: int | None = None) -> np.ndarray:
+    a = np.fromfile(path, dtype=np.float16)
+    if count is not None and a.size != count:
+        raise ValueError(f"{path}: {a.size} fp16 values, expected {count}")
+    return a
+
+
+def embedding_file(root: str) -> str:
+    """embed_tokens.bin, or the name the exporter uses for tied embeddings."""
+    for name in ("embed_tokens.bin", "shared_embed_lm_head.bin"):
+        if os.path.exists(os.path.join(root, name)):
+            return os.path.join(root, name)
+    raise FileNotFoundError(f"{root}: neither embed_tokens.bin nor shared_embed_lm_head.bin")
+
+
+def lm_head_kind(root: str) -> str:
+    """'hlq' (lm_head/lm_head directory), 'fp16' (lm_head.bin) or 'tied' (llama.cpp:70-80)."""
+    if os.path.isdir(os.path.join(root, "lm_head", "lm_head")):
+        return "hlq"
+    if os.path.exists(os.path.join(root, "lm_head.bin")):
+        return "fp16"
+    return "tied"
+
+
+def is_repacked_dir(path: str) -> bool:
+    return os.path.exists(os.path.join(path, REPACKED_JSON))
+
+
+def write_repacked_dir(path: str, k: int, n: int, bits: int, group: int, planes, scales, zeros, bias=None) -> None:
+    """Kernel-layout buffers of one linear layer as files that load with a plain copy."""
+    os.makedirs(path, exist_ok=True)
+    for name, a in (("planes.bin", planes), ("scales.bin", scales), ("zeros.bin", zeros)):
+        with open(os.path.join(path, name), "wb") as f:
+            f.write(np.ascontiguousarray(a, dtype=np.uint8).tobytes())
+    if bias is not None:
+        write_fp16_bin(os.path.join(path, "bias.bin"), bias)
+    with open(os.path.join(path, REPACKED_JSON), "w") as f:
+        json.dump({"layout_version": REPACK_LAYOUT_VERSION, "in_channel": int(k), "out_channel": int(n),
+                   "base_bit": int(bits), "groupsize": int(group), "has_bias": bias is not None}, f, indent=4)
+
+
+def read_repacked_dir(path: str):
+    """-> (k, n, bits, group, planes, scales, zeros, bias) with uint8 buffers (bias fp16 or None)."""
+    with open(os.path.join(path, REPACKED_JSON)) as f:
+        cfg = json.load(f)
+    if cfg.get("layout_version") != REPACK_LAYOUT_VERSION:
+        raise ValueError(f"{path}: layout version {cfg.get('layout_version')}, this build reads {REPACK_LAYOUT_VERSION}")
+    k, n, bits, group = int(cfg["in_channel"]), int(cfg["out_channel"]), int(cfg["base_bit"]), int(cfg["groupsize"])
+    bufs = [np.fromfile(os.path.join(path, name), dtype=np.uint8) for name in ("planes.bin", "scales.bin", "zeros.bin")]
+    bias = read_fp16_bin(os.path.join(path, "bias.bin"), n) if cfg.get("has_bias") else None
+    return (k, n, bits, group, *bufs, bias)

@@ -18,7 +18,7 @@ import torch
 from torch import nn
 
 from . import _lib
-from .export_io import ExportedLinear, read_export_dir
+from .export_io import ExportedLinear, is_repacked_dir, read_export_dir, read_repacked_dir
 
 _workspaces: dict = {}
 
@@ -121,7 +121,24 @@ class HLQLinear(nn.Module):
 
     @classmethod
     def from_export_dir(cls, path: str, device="cuda", group_size: int | None = None) -> "HLQLinear":
+        """A linear directory of the reference's export, or the same after `python -m elutq_amd.repack`."""
+        if is_repacked_dir(path):
+            return cls.from_repacked_dir(path, device)
         return cls.from_export(read_export_dir(path, group_size), device)
+
+    @classmethod
+    def from_repacked_dir(cls, path: str, device="cuda") -> "HLQLinear":
+        k, n, bits, group, planes, scales, zeros, bias = read_repacked_dir(path)
+        L = _lib.lib()
+        want = (L.elutq_hlq_planes_bytes(k, n, bits), L.elutq_hlq_scales_bytes(k, n, bits, group),
+                L.elutq_hlq_zeros_bytes(k, n, group))
+        if 0 in want or (planes.size, scales.size, zeros.size) != want:
+            raise ValueError(f"{path}: buffer sizes {(planes.size, scales.size, zeros.size)} do not match "
+                             f"K={k} N={n} bits={bits} group={group} (expected {want})")
+        dev = torch.device(device)
+        b = None if bias is None else torch.from_numpy(bias).to(dev)
+        return cls(k, n, bits, group, torch.from_numpy(planes).to(dev), torch.from_numpy(scales).to(dev),
+                   torch.from_numpy(zeros).to(dev), b)
 
     # -- compute -----------------------------------------------------------------------
     def forward(self, x: torch.Tensor) -> torch.Tensor:

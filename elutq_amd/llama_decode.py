@@ -160,10 +160,76 @@ def rope(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
     return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1).to(torch.float16)
 
 
+PROJ_DIRS = {"q_proj": "self_attn.q_proj", "k_proj": "self_attn.k_proj", "v_proj": "self_attn.v_proj",
+             "o_proj": "self_attn.o_proj", "gate_proj": "mlp.gate_proj", "up_proj": "mlp.up_proj",
+             "down_proj": "mlp.down_proj"}
+
+
+def proj_shapes(s: LlamaShape) -> dict:
+    d = s.head_dim
+    return {"q_proj": (s.hidden, s.n_heads * d), "k_proj": (s.hidden, s.n_kv_heads * d),
+            "v_proj": (s.hidden, s.n_kv_heads * d), "o_proj": (s.n_heads * d, s.hidden),
+            "gate_proj": (s.hidden, s.ffn), "up_proj": (s.hidden, s.ffn), "down_proj": (s.ffn, s.hidden)}
+
+
+def random_parts(s: LlamaShape, dev, seed: int) -> dict:
+    """Random-init weights of the shape (generated on the device)."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    layers = []
+    sd = seed * 100_003
+    for _ in range(s.n_layers):
+        lin = {}
+        for name, (k, n) in proj_shapes(s).items():
+            lin[name] = make_device_layer(k, n, s.bits, s.group, seed=sd, device=dev)
+            sd += 1
+        norms = tuple((1.0 + 0.1 * torch.randn(s.hidden, generator=g, device=dev)).to(torch.float16) for _ in range(2))
+        layers.append((lin, norms))
+    embed = (torch.randn(s.vocab, s.hidden, generator=g, device=dev) * 0.5).to(torch.float16)
+    lm_head = (torch.randn(s.vocab, s.hidden, generator=g, device=dev) * 0.02).to(torch.float16)
+    norm = (1.0 + 0.1 * torch.randn(s.hidden, generator=g, device=dev)).to(torch.float16)
+    return {"layers": layers, "embed": embed, "lm_head": lm_head, "norm": norm}
+
+
+def parts_from_export(root: str, s: LlamaShape, dev) -> dict:
+    """Reads the reference's model export tree (written by GPTQ/llama.py:285-343, read by
+    C++/examples/models/llama.cpp:59-115), or the same tree after `python -m elutq_amd.repack`.
+    The lm_head is the HLQ layer in lm_head/lm_head if that directory exists, else lm_head.bin,
+    else the (tied) embedding, in the order of llama.cpp:68-80."""
+    import os
+    from . import export_io as io
+
+    def vec(path, n):
+        return torch.from_numpy(io.read_fp16_bin(path, n)).to(dev)
+
+    layers = []
+    for i in range(s.n_layers):
+        base = os.path.join(root, str(i))
+        lin = {}
+        for name, (k, n) in proj_shapes(s).items():
+            m = HLQLinear.from_export_dir(os.path.join(base, PROJ_DIRS[name]), dev)
+            if (m.in_features, m.out_features) != (k, n):
+                raise ValueError(f"{base}/{PROJ_DIRS[name]}: {m.in_features}x{m.out_features}, the shape needs {k}x{n}")
+            lin[name] = m
+        layers.append((lin, tuple(vec(os.path.join(base, f), s.hidden) for f in io.LAYER_NORMS)))
+    embed = vec(io.embedding_file(root), s.vocab * s.hidden).view(s.vocab, s.hidden)
+    kind = io.lm_head_kind(root)
+    if kind == "hlq":
+        lm_head = HLQLinear.from_export_dir(os.path.join(root, "lm_head", "lm_head"), dev)
+        if (lm_head.in_features, lm_head.out_features) != (s.hidden, s.vocab):
+            raise ValueError("lm_head/lm_head does not match hidden x vocab")
+    elif kind == "fp16":
+        lm_head = vec(os.path.join(root, "lm_head.bin"), s.vocab * s.hidden).view(s.vocab, s.hidden)
+    else:
+        lm_head = None
+    return {"layers": layers, "embed": embed, "lm_head": lm_head,
+            "norm": vec(os.path.join(root, "final_rmsnorm_weight.bin"), s.hidden)}
+
+
 class LlamaDecoder(nn.Module):
     """Random-init LLaMA-shaped decoder for the decode benchmark and its parity test."""
 
-    def __init__(self, s: LlamaShape, device="cuda", seed: int = 0, fuse: bool = True, impl: str = "hip"):
+    def __init__(self, s: LlamaShape, device="cuda", seed: int = 0, fuse: bool = True, impl: str = "hip",
+                 parts: dict | None = None):
         """impl "hip": five fused launches per layer through the C ABI (needs fuse=True);
         impl "torch": the same step with PyTorch ops around plain HLQLinear calls."""
         super().__init__()
@@ -171,24 +237,16 @@ class LlamaDecoder(nn.Module):
         self.s = s
         self.impl = impl
         dev = torch.device(device)
-        g = torch.Generator(device=dev).manual_seed(seed)
         d = s.head_dim
-        shapes = {"q_proj": (s.hidden, s.n_heads * d), "k_proj": (s.hidden, s.n_kv_heads * d),
-                  "v_proj": (s.hidden, s.n_kv_heads * d), "o_proj": (s.n_heads * d, s.hidden),
-                  "gate_proj": (s.hidden, s.ffn), "up_proj": (s.hidden, s.ffn), "down_proj": (s.ffn, s.hidden)}
-        layers = []
-        sd = seed * 100_003
-        for _ in range(s.n_layers):
-            lin = {}
-            for name, (k, n) in shapes.items():
-                lin[name] = make_device_layer(k, n, s.bits, s.group, seed=sd, device=dev)
-                sd += 1
-            norms = tuple((1.0 + 0.1 * torch.randn(s.hidden, generator=g, device=dev)).to(torch.float16) for _ in range(2))
-            layers.append(DecoderLayer(s, lin, norms, fuse))
-        self.layers = nn.ModuleList(layers)
-        self.register_buffer("embed", (torch.randn(s.vocab, s.hidden, generator=g, device=dev) * 0.5).to(torch.float16))
-        self.register_buffer("lm_head", (torch.randn(s.vocab, s.hidden, generator=g, device=dev) * 0.02).to(torch.float16))
-        self.register_buffer("norm", (1.0 + 0.1 * torch.randn(s.hidden, generator=g, device=dev)).to(torch.float16))
+        if parts is None:
+            parts = random_parts(s, dev, seed)
+        self.layers = nn.ModuleList([DecoderLayer(s, lin, norms, fuse) for lin, norms in parts["layers"]])
+        self.register_buffer("embed", parts["embed"])
+        self.register_buffer("norm", parts["norm"])
+        # lm_head: fp16 [vocab, hidden] (lm_head.bin, or the embedding when tied) or an HLQ layer
+        head = parts["lm_head"] if parts["lm_head"] is not None else parts["embed"]
+        self.lm_head_q = head if isinstance(head, HLQLinear) else None
+        self.register_buffer("lm_head", None if isinstance(head, HLQLinear) else head)
         inv = s.rope_base ** (-torch.arange(0, d, 2, device=dev, dtype=torch.float32) / d)
         ang = torch.arange(s.max_seq, device=dev, dtype=torch.float32)[:, None] * inv[None, :]
         self.register_buffer("cos_t", ang.cos())
@@ -203,6 +261,11 @@ class LlamaDecoder(nn.Module):
             ws = max(m.workspace_bytes for m in self.modules() if isinstance(m, HLQLinear))
             ws = max(ws, _lib.lib().elutq_decode_attn_workspace_bytes(s.n_heads, s.head_dim, 0))
             self._buf = FusedBuffers(s, ws, dev)
+
+    @classmethod
+    def from_export(cls, root: str, s: LlamaShape, device="cuda", fuse: bool = True, impl: str = "hip") -> "LlamaDecoder":
+        """A decoder over a genuinely exported model (bits and group size come from the files)."""
+        return cls(s, device=device, fuse=fuse, impl=impl, parts=parts_from_export(root, s, torch.device(device)))
 
     @torch.no_grad()
     def fill_cache(self, n_tokens: int, seed: int = 1) -> None:
@@ -236,11 +299,15 @@ class LlamaDecoder(nn.Module):
             L, stream = _lib.lib(), torch.cuda.current_stream().cuda_stream
             _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), b.xb.data_ptr(), self.s.hidden,
                                                   self.s.rms_eps, stream), "elutq_decode_rmsnorm_f16")
-            logits = torch.mm(b.xb, self.lm_head.t(), out=b.logits)
+            if self.lm_head_q is not None:
+                logits = self.lm_head_q.gemv_fused(b.xb, b.logits, b.ws)
+            else:
+                logits = torch.mm(b.xb, self.lm_head.t(), out=b.logits)
             _lib.check(L.elutq_decode_argmax_f16(logits.data_ptr(), self.s.vocab, self.token.data_ptr(),
                                                  self.pos.data_ptr(), stream), "elutq_decode_argmax_f16")
             return logits
-        logits = F.linear(rms_norm(x, self.norm, self.s.rms_eps), self.lm_head)
+        xn = rms_norm(x, self.norm, self.s.rms_eps)
+        logits = self.lm_head_q(xn) if self.lm_head_q is not None else F.linear(xn, self.lm_head)
         self.token.copy_(logits.argmax(-1))
         self.pos.add_(1)
         return logits
@@ -287,7 +354,7 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
     dt = time.perf_counter() - t0
     hlq_bytes = sum(m.planes.numel() + m.scales.numel() + m.zeros.numel()
                     for m in model.modules() if isinstance(m, HLQLinear))
-    lm_bytes = model.lm_head.numel() * 2
+    lm_bytes = model.lm_head.numel() * 2 if model.lm_head is not None else 0
     kv_bytes = 2 * s.n_layers * n_ctx * s.n_kv_heads * s.head_dim * 2
     ms = dt / (n_gen - 1) * 1e3
     return {"tokens_per_s": (n_gen - 1) / dt, "ms_per_token": ms, "n_ctx": n_ctx, "n_gen": n_gen,

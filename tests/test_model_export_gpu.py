@@ -1,0 +1,64 @@
+"""LlamaDecoder over an exported model tree: the reference's layout, the same tree after the
+offline repack, and the in-memory construction must decode the same tokens."""
+import numpy as np
+import pytest
+import torch
+
+from elutq_amd.hlq_linear import HLQLinear
+from elutq_amd.llama_decode import LlamaDecoder
+from elutq_amd.repack import repack_tree
+
+from model_export_fixture import TINY, write_tiny_export
+
+pytestmark = pytest.mark.gpu
+
+
+def in_memory_parts(arrays, dev):
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+    layers = []
+    for lay in arrays["layers"]:
+        lin = {name: HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, L.group, L.bias, dev)
+               for name, L in lay.items() if not name.endswith(".bin")}
+        layers.append((lin, (t(lay["input_layernorm_weight.bin"]), t(lay["post_attention_layernorm_weight.bin"]))))
+    head = arrays.get("lm_head")
+    if head is not None and not isinstance(head, np.ndarray):
+        head = HLQLinear.from_export_arrays(head.w_quant, head.w_scale, head.w_zero, head.group, None, dev)
+    elif head is not None:
+        head = t(head)
+    return {"layers": layers, "embed": t(arrays["embed"]), "lm_head": head, "norm": t(arrays["norm"])}
+
+
+@pytest.mark.parametrize("kind", ["fp16", "hlq", "tied"])
+@pytest.mark.parametrize("impl", ["hip", "torch"])
+def test_decoder_from_export_tree(cuda, tmp_path, kind, impl):
+    src, dst = str(tmp_path / "export"), str(tmp_path / "repacked")
+    arrays = write_tiny_export(src, lm_head=kind)
+    repack_tree(src, dst)
+    models = [LlamaDecoder.from_export(src, TINY, device=cuda, impl=impl),
+              LlamaDecoder.from_export(dst, TINY, device=cuda, impl=impl),
+              LlamaDecoder(TINY, device=cuda, impl=impl, parts=in_memory_parts(arrays, cuda))]
+    assert (models[0].lm_head_q is not None) == (kind == "hlq")
+    if kind == "tied":
+        assert torch.equal(models[0].lm_head, models[0].embed)
+    outs = []
+    for m in models:
+        m.fill_cache(9, seed=3)
+        m.token.fill_(5)
+        toks, logits = [], []
+        for _ in range(4):
+            logits.append(m.step().clone())
+            toks.append(int(m.token))
+        outs.append((toks, torch.cat(logits)))
+    for toks, logits in outs[1:]:
+        assert toks == outs[0][0] and torch.equal(logits, outs[0][1])
+    assert all(0 <= t < TINY.vocab for t in outs[0][0]) and int(models[0].pos) == 13
+
+
+def test_from_export_rejects_wrong_shape(cuda, tmp_path):
+    import dataclasses
+    src = str(tmp_path / "export")
+    write_tiny_export(src)
+    with pytest.raises(ValueError, match="the shape needs"):
+        LlamaDecoder.from_export(src, dataclasses.replace(TINY, ffn=512), device=cuda)
+    with pytest.raises(ValueError, match="fp16 values"):
+        LlamaDecoder.from_export(src, dataclasses.replace(TINY, vocab=301), device=cuda)
