@@ -32,6 +32,10 @@ SIGNATURES = {
     "elutq_decode_attn_workspace_bytes": (_sz, [_ci] * 3),
     "elutq_decode_rmsnorm_f16": (_ci, [_vp] * 3 + [_ci, ctypes.c_float, _vp]),
     "elutq_decode_argmax_f16": (_ci, [_vp, _ci, _vp, _vp, _vp]),
+    "elutq_hlq_gemv_group_workspace_bytes": (_sz, [_vp, _ci, _ci, _ci]),
+    "elutq_hlq_gemv_group_create": (_ci, [_vp, _ci, _ci, _ci, _vp, _sz, _vp]),
+    "elutq_hlq_gemv_group_run": (_ci, [_vp, _vp]),
+    "elutq_hlq_gemv_group_destroy": (_ci, [_vp]),
     "elutq_hlq_gemm_f16": (_ci, [_vp] * 6 + [_ci] * 5 + [_vp, _sz, _vp]),
     "elutq_hlq_gemm_f16_tuned": (_ci, [_vp] * 6 + [_ci] * 5 + [_vp, _sz, _vp, _ci, _ci]),
     "elutq_hlq_dequant_f16": (_ci, [_vp] * 4 + [_ci] * 4 + [_vp]),
@@ -43,6 +47,13 @@ class GemvFusion(ctypes.Structure):
     """struct elutq_gemv_fusion of include/elutq_hip.h."""
     _fields_ = [("prologue", ctypes.c_int), ("eps", ctypes.c_float),
                 ("d_norm_weight", ctypes.c_void_p), ("d_residual", ctypes.c_void_p)]
+
+
+class GemvProblem(ctypes.Structure):
+    """struct elutq_gemv_problem of include/elutq_hip.h."""
+    _fields_ = [("d_planes", ctypes.c_void_p), ("d_scales", ctypes.c_void_p), ("d_zeros", ctypes.c_void_p),
+                ("d_bias", ctypes.c_void_p), ("d_x", ctypes.c_void_p), ("d_y", ctypes.c_void_p),
+                ("K", ctypes.c_int), ("N", ctypes.c_int)]
 
 
 _lib = None

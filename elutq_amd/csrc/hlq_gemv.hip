@@ -25,6 +25,7 @@
 //  * slices are combined through a workspace by the last workgroup to arrive (fixed
 //    summation order, so results are deterministic).
 #include <hip/hip_runtime.h>
+#include <vector>
 #include <stdint.h>
 
 #include "../../include/elutq_hip.h"
@@ -265,13 +266,17 @@ constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 // (one or two) units its run touches in its own LDS region and goes on to its lookups
 // without waiting for the other waves -- the only workgroup barrier is the one in front of
 // the final cross-wave sum.
+//
+// `vblock` = column block * ksplit + slice (the block index of a launch that runs one
+// GEMV); `red_sel` picks one of two cross-wave buffers so that a caller that runs tiles
+// back to back needs no barrier between them: waves other than wave 0 may start the next
+// tile while wave 0 still sums and stores this one.
 template <int BITS, bool G64, int NSLOT>
-__global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
+__device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, unsigned char *smem, int red_sel)
 {
-    extern __shared__ __align__(256) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int cb = blockIdx.x / a.ksplit, slice = blockIdx.x - cb * a.ksplit;
+    const int cb = vblock / a.ksplit, slice = vblock - cb * a.ksplit;
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
     const int nst = nU * BITS;                                             // sub-tasks of this workgroup
     const int s_begin = min(wave * a.spw, nst), s_end = min(s_begin + a.spw, nst);
@@ -281,8 +286,9 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 
     unsigned char *lut = smem + (size_t)wave * a.wave_lds;                 // this wave's tables [nuw][32][16] int32
     float2 *xs_inv = (float2 *)(lut + (size_t)a.nuw_max * UNIT_LUT_BYTES); // [2 * nuw_max]
-    float *red = (float *)(smem + (size_t)nw * a.wave_lds);                // [nw][64]
-    float *rstd_scratch = red + nw * HLQ_CB;                               // [RSTD_SCRATCH]
+    float *red0 = (float *)(smem + (size_t)nw * a.wave_lds);               // [2][nw][64]
+    float *red = red0 + red_sel * nw * HLQ_CB;
+    float *rstd_scratch = red0 + 2 * nw * HLQ_CB;                          // [RSTD_SCRATCH]
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
     HLQ_STAMP(0);
@@ -409,6 +415,36 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
     }
 }
 
+template <int BITS, bool G64, int NSLOT>
+__global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
+{
+    extern __shared__ __align__(256) unsigned char smem[];
+    gemv_tile<BITS, G64, NSLOT>(a, blockIdx.x, smem, 0);
+}
+
+// Many independent GEMVs in one launch: the tiles of all of them form one list that the
+// workgroups walk with stride gridDim.x (tiles of one GEMV are neighbours in the list, so its
+// activations stay in cache and the slices of a column block run at about the same time).
+// Nothing waits for another workgroup -- slices still meet through tickets -- so the launch,
+// the first memory round trips and the tail of a GEMV are paid once per list instead of once
+// per GEMV, and with two workgroups per CU the sum-and-store of one tile hides under the
+// lookups of another.
+struct GroupItem {
+    int problem, vblock;
+};
+
+template <int BITS, bool G64, int NSLOT>
+__global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *problems, const GroupItem *items, int n_items)
+{
+    extern __shared__ __align__(256) unsigned char smem[];
+    int sel = 0;
+    for (int i = blockIdx.x; i < n_items; i += gridDim.x, sel ^= 1) {
+        const GroupItem it = items[i];
+        const GemvArgs a = problems[it.problem];
+        gemv_tile<BITS, G64, NSLOT>(a, it.vblock, smem, sel);
+    }
+}
+
 // Per-wave LDS region and run length for a slice of `ups` units handled by `waves` waves.
 struct WavePlan {
     int spw, nuw_max, wave_lds;
@@ -430,7 +466,7 @@ WavePlan wave_plan(int ups, int bits, int waves)
 size_t gemv_lds_bytes(int ups, int bits, int waves)
 {
     const WavePlan p = wave_plan(ups, bits, waves);
-    return (size_t)waves * p.wave_lds + (size_t)waves * HLQ_CB * sizeof(float) + RSTD_SCRATCH * sizeof(float) + 16;
+    return (size_t)waves * p.wave_lds + 2 * (size_t)waves * HLQ_CB * sizeof(float) + RSTD_SCRATCH * sizeof(float) + 16;
 }
 
 template <int BITS, bool G64, int NSLOT>
@@ -467,6 +503,44 @@ int dispatch_gemv(const GemvArgs &a, int bits, int group, int waves, size_t lds,
     case 2: return g64 ? launch_gemv<2, true>(a, waves, lds, stream) : launch_gemv<2, false>(a, waves, lds, stream);
     case 3: return g64 ? launch_gemv<3, true>(a, waves, lds, stream) : launch_gemv<3, false>(a, waves, lds, stream);
     case 4: return g64 ? launch_gemv<4, true>(a, waves, lds, stream) : launch_gemv<4, false>(a, waves, lds, stream);
+    }
+    return ELUTQ_ERR_BITS;
+}
+
+template <int BITS, bool G64, int NSLOT>
+int launch_group_n(const GemvArgs *d_problems, const GroupItem *d_items, int n_items, int grid, int waves, size_t lds,
+                   hipStream_t stream)
+{
+    auto kern = hlq_gemv_group_kernel<BITS, G64, NSLOT>;
+    static bool big_lds_enabled = false;
+    if (lds > 64 * 1024 && !big_lds_enabled) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS) != hipSuccess)
+            return ELUTQ_ERR_HIP;
+        big_lds_enabled = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * 64), lds, stream, d_problems, d_items, n_items);
+    return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
+}
+
+template <int BITS, bool G64>
+int launch_group(int nslot, const GemvArgs *p, const GroupItem *it, int n, int grid, int waves, size_t lds, hipStream_t st)
+{
+    switch (nslot) {
+    case 1: return launch_group_n<BITS, G64, 1>(p, it, n, grid, waves, lds, st);
+    case 2: return launch_group_n<BITS, G64, 2>(p, it, n, grid, waves, lds, st);
+    case 3: return launch_group_n<BITS, G64, 3>(p, it, n, grid, waves, lds, st);
+    default: return launch_group_n<BITS, G64, 4>(p, it, n, grid, waves, lds, st);
+    }
+}
+
+int dispatch_group(int bits, bool g64, int nslot, const GemvArgs *p, const GroupItem *it, int n, int grid, int waves,
+                   size_t lds, hipStream_t st)
+{
+    switch (bits) {
+    case 1: return g64 ? launch_group<1, true>(nslot, p, it, n, grid, waves, lds, st) : launch_group<1, false>(nslot, p, it, n, grid, waves, lds, st);
+    case 2: return g64 ? launch_group<2, true>(nslot, p, it, n, grid, waves, lds, st) : launch_group<2, false>(nslot, p, it, n, grid, waves, lds, st);
+    case 3: return g64 ? launch_group<3, true>(nslot, p, it, n, grid, waves, lds, st) : launch_group<3, false>(nslot, p, it, n, grid, waves, lds, st);
+    case 4: return g64 ? launch_group<4, true>(nslot, p, it, n, grid, waves, lds, st) : launch_group<4, false>(nslot, p, it, n, grid, waves, lds, st);
     }
     return ELUTQ_ERR_BITS;
 }
@@ -573,6 +647,148 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
         a.partial = (float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves), (hipStream_t)stream);
+}
+
+// ---- grouped launch of independent GEMVs --------------------------------------------------
+struct GroupShape {                      // tile shape of one problem inside a group
+    HlqGeo g;
+    int ksplit, ups;
+    WavePlan wp;
+};
+
+static int group_shape(const elutq_gemv_problem &p, int bits, int group, GroupShape &sh)
+{
+    int rc = check_shape(p.K, p.N, bits, group);
+    if (rc != ELUTQ_OK) return rc;
+    if (!p.d_planes || !p.d_scales || !p.d_zeros || !p.d_x || !p.d_y) return ELUTQ_ERR_NULL;
+    sh.g = hlq_geo(p.K, p.N, bits, group);
+    // the list supplies the parallelism: slice K only as far as run length and LDS ask for
+    int ksplit = (sh.g.U + 31) / 32;
+    int ups = (sh.g.U + ksplit - 1) / ksplit;
+    while (gemv_lds_bytes(ups, bits, 16) > (size_t)MAX_LDS / 2) ups = (ups + 1) / 2;     // two workgroups per CU
+    sh.ups = ups;
+    sh.ksplit = (sh.g.U + ups - 1) / ups;
+    sh.wp = wave_plan(ups, bits, 16);
+    return ELUTQ_OK;
+}
+
+struct GemvGroupPlan {
+    int bits, group, nslot, n_items, grid;
+    size_t lds;
+    GemvArgs *d_problems;
+    GroupItem *d_items;
+};
+
+static size_t group_layout(const elutq_gemv_problem *problems, int count, int bits, int group,
+                           std::vector<GroupShape> *shapes, std::vector<size_t> *counter_off, std::vector<size_t> *partial_off,
+                           int *rc_out)
+{
+    size_t counters = 0, partials = 0;
+    *rc_out = ELUTQ_OK;
+    for (int i = 0; i < count; i++) {
+        GroupShape sh;
+        const int rc = group_shape(problems[i], bits, group, sh);
+        if (rc != ELUTQ_OK) { *rc_out = rc; return 0; }
+        if (shapes) shapes->push_back(sh);
+        if (counter_off) counter_off->push_back(counters);
+        if (partial_off) partial_off->push_back(partials);
+        if (sh.ksplit > 1) {
+            counters += (size_t)sh.g.ncb * sizeof(unsigned);
+            partials += (size_t)sh.ksplit * sh.g.ncb * HLQ_CB * sizeof(float);
+        }
+    }
+    counters = (counters + 255) & ~(size_t)255;
+    if (partial_off)
+        for (auto &o : *partial_off) o += counters;
+    return counters + partials + 256;
+}
+
+size_t elutq_hlq_gemv_group_workspace_bytes(const elutq_gemv_problem *problems, int count, int bits, int group)
+{
+    if (!problems || count < 1) return 0;
+    int rc;
+    const size_t n = group_layout(problems, count, bits, group, nullptr, nullptr, nullptr, &rc);
+    return rc == ELUTQ_OK ? n : 0;
+}
+
+int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, int bits, int group, void *d_workspace,
+                                size_t workspace_bytes, void **plan_out)
+{
+    if (!problems || !plan_out) return ELUTQ_ERR_NULL;
+    if (count < 1) return ELUTQ_ERR_SHAPE;
+    *plan_out = nullptr;
+    std::vector<GroupShape> shapes;
+    std::vector<size_t> coff, poff;
+    int rc;
+    const size_t need = group_layout(problems, count, bits, group, &shapes, &coff, &poff, &rc);
+    if (rc != ELUTQ_OK) return rc;
+    bool any_split = false;
+    for (auto &sh : shapes) any_split |= sh.ksplit > 1;
+    if (any_split) {
+        if (!d_workspace) return ELUTQ_ERR_NULL;
+        if (workspace_bytes < need) return ELUTQ_ERR_WORKSPACE;
+    }
+    std::vector<GemvArgs> args(count);
+    std::vector<GroupItem> items;
+    int nslot = 1;
+    size_t lds = 0;
+    for (int i = 0; i < count; i++) {
+        const GroupShape &sh = shapes[i];
+        GemvArgs &a = args[i];
+        a.planes = (const uint4 *)problems[i].d_planes;
+        a.scales = (const uint32_t *)problems[i].d_scales;
+        a.zeros = (const uint32_t *)problems[i].d_zeros;
+        a.bias = (const uint16_t *)problems[i].d_bias;
+        a.x = (const uint16_t *)problems[i].d_x;
+        a.y = (uint16_t *)problems[i].d_y;
+        a.N = problems[i].N; a.U = sh.g.U; a.NT = sh.g.NT; a.ncb = sh.g.ncb;
+        a.ksplit = sh.ksplit; a.ups = sh.ups;
+        a.spw = sh.wp.spw; a.nuw_max = sh.wp.nuw_max; a.wave_lds = sh.wp.wave_lds;
+        a.partial = nullptr; a.counters = nullptr;
+        if (sh.ksplit > 1) {
+            a.counters = (unsigned *)((unsigned char *)d_workspace + coff[i]);
+            a.partial = (float *)((unsigned char *)d_workspace + poff[i]);
+        }
+        a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr;
+        const int ns = a.spw < DEPTH ? a.spw : DEPTH;
+        if (ns > nslot) nslot = ns;
+        const size_t l = gemv_lds_bytes(sh.ups, bits, 16);
+        if (l > lds) lds = l;
+        for (int vb = 0; vb < sh.g.ncb * sh.ksplit; vb++) items.push_back(GroupItem{i, vb});
+    }
+    GemvGroupPlan *pl = new GemvGroupPlan();
+    pl->bits = bits; pl->group = group; pl->nslot = nslot; pl->n_items = (int)items.size(); pl->lds = lds;
+    const int slots = NUM_CU * (lds <= (size_t)MAX_LDS / 2 ? 2 : 1);
+    pl->grid = pl->n_items < slots ? pl->n_items : slots;
+    pl->d_problems = nullptr; pl->d_items = nullptr;
+    if (hipMalloc((void **)&pl->d_problems, args.size() * sizeof(GemvArgs)) != hipSuccess ||
+        hipMalloc((void **)&pl->d_items, items.size() * sizeof(GroupItem)) != hipSuccess ||
+        hipMemcpy(pl->d_problems, args.data(), args.size() * sizeof(GemvArgs), hipMemcpyHostToDevice) != hipSuccess ||
+        hipMemcpy(pl->d_items, items.data(), items.size() * sizeof(GroupItem), hipMemcpyHostToDevice) != hipSuccess) {
+        if (pl->d_problems) (void)hipFree(pl->d_problems);
+        if (pl->d_items) (void)hipFree(pl->d_items);
+        delete pl;
+        return ELUTQ_ERR_HIP;
+    }
+    *plan_out = pl;
+    return ELUTQ_OK;
+}
+
+int elutq_hlq_gemv_group_run(void *plan, void *stream)
+{
+    if (!plan) return ELUTQ_ERR_NULL;
+    const GemvGroupPlan *pl = (const GemvGroupPlan *)plan;
+    return dispatch_group(pl->bits, pl->group == 64, pl->nslot, pl->d_problems, pl->d_items, pl->n_items, pl->grid, 16,
+                          pl->lds, (hipStream_t)stream);
+}
+
+int elutq_hlq_gemv_group_destroy(void *plan)
+{
+    if (!plan) return ELUTQ_ERR_NULL;
+    GemvGroupPlan *pl = (GemvGroupPlan *)plan;
+    const bool ok = hipFree(pl->d_problems) == hipSuccess && hipFree(pl->d_items) == hipSuccess;
+    delete pl;
+    return ok ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
 
 int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,

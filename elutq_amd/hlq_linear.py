@@ -210,6 +210,56 @@ class HLQLinear(nn.Module):
                 f"group_size={self.group_size}, bias={self.bias is not None}")
 
 
+class GemvGroup:
+    """Independent batch-1 GEMVs that share one launch (elutq_hlq_gemv_group_* of the C ABI).
+
+    `mods`, `xs`, `ys`: equally long lists of HLQLinear layers (same bits and group size), their
+    fp16 inputs [1, K] and caller-owned fp16 outputs [1, N].  Creation allocates the device-side
+    problem list and a workspace; `run()` is one kernel launch on the current stream and can be
+    captured in a HIP graph.  Inputs and outputs are referenced, not copied: refill them in place."""
+
+    def __init__(self, mods, xs, ys):
+        if not mods or not (len(mods) == len(xs) == len(ys)):
+            raise ValueError("need equally long, non-empty lists of layers, inputs and outputs")
+        bits, group = mods[0].bits, mods[0].group_size
+        arr = (_lib.GemvProblem * len(mods))()
+        for p, m, x, y in zip(arr, mods, xs, ys):
+            if (m.bits, m.group_size) != (bits, group):
+                raise ValueError("all layers of a group must share bits and group size")
+            if x.dtype != torch.float16 or y.dtype != torch.float16 or x.numel() != m.in_features or y.numel() != m.out_features:
+                raise ValueError("inputs must be fp16 [K], outputs fp16 [N]")
+            p.d_planes, p.d_scales, p.d_zeros = m.planes.data_ptr(), m.scales.data_ptr(), m.zeros.data_ptr()
+            p.d_bias = m.bias.data_ptr() if m.bias is not None else None
+            p.d_x, p.d_y, p.K, p.N = x.data_ptr(), y.data_ptr(), m.in_features, m.out_features
+        L = _lib.lib()
+        self._keep = (list(mods), list(xs), list(ys))
+        self._device = mods[0].planes.device
+        nbytes = L.elutq_hlq_gemv_group_workspace_bytes(ctypes.byref(arr), len(mods), bits, group)
+        if nbytes == 0:
+            raise ValueError("unsupported shape in the group")
+        self.ws = torch.zeros(nbytes, dtype=torch.uint8, device=self._device)
+        plan = ctypes.c_void_p()
+        _lib.check(L.elutq_hlq_gemv_group_create(ctypes.byref(arr), len(mods), bits, group, self.ws.data_ptr(),
+                                                 self.ws.numel(), ctypes.byref(plan)), "elutq_hlq_gemv_group_create")
+        self._plan = plan
+
+    def run(self) -> None:
+        _lib.check(_lib.lib().elutq_hlq_gemv_group_run(self._plan, torch.cuda.current_stream(self._device).cuda_stream),
+                   "elutq_hlq_gemv_group_run")
+
+    def close(self) -> None:
+        if self._plan is not None:
+            torch.cuda.synchronize(self._device)
+            _lib.lib().elutq_hlq_gemv_group_destroy(self._plan)
+            self._plan = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 def replace_linear(model: nn.Module, export_root: str, device="cuda", group_size: int | None = None) -> int:
     """Swaps every ``nn.Linear`` that has an export directory for an HLQLinear.
 

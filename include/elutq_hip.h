@@ -131,6 +131,31 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
                              const elutq_gemv_fusion *fusion, int ksplit, int waves);
 
 /*
+ * Many independent batch-1 GEMVs in one launch (same bits and group size; any shapes).  The
+ * reference issues arm_gemm once per projection (llama::forward, C++/examples/models/llama.cpp:
+ * 244-739); projections that do not depend on each other -- q, k and v of a layer, gate and up,
+ * the layers of a benchmark sweep -- can instead share one launch, which pays the launch, the
+ * first memory round trips and the tail once and keeps HBM streaming across GEMV boundaries.
+ * A plan holds the device-side problem list: create it once (allocates and copies; not
+ * capturable), run it any number of times (one kernel launch, capturable), destroy it.
+ * The workspace (elutq_hlq_gemv_group_workspace_bytes, zero-filled once) is bound at creation
+ * and must not be shared with calls that may run concurrently.  Results equal those of
+ * elutq_hlq_gemv_f16_tuned with the same K slicing, which the group chooses itself.
+ */
+typedef struct elutq_gemv_problem {
+    const void *d_planes, *d_scales, *d_zeros, *d_bias;  /* as for elutq_hlq_gemv_f16; bias may be NULL */
+    const void *d_x;                                      /* fp16 [K] */
+    void *d_y;                                            /* fp16 [N] */
+    int K, N;
+} elutq_gemv_problem;
+
+size_t elutq_hlq_gemv_group_workspace_bytes(const elutq_gemv_problem *problems, int count, int bits, int group);
+int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, int bits, int group,
+                                void *d_workspace, size_t workspace_bytes, void **plan);
+int elutq_hlq_gemv_group_run(void *plan, void *stream);
+int elutq_hlq_gemv_group_destroy(void *plan);
+
+/*
  * y[M][N] = x[M][K] W^T + bias, row-major fp16, 1 <= M.  Replaces arm_gemm(m > 1, ...),
  * which the reference defines as one GEMV per row.
  */
