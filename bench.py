@@ -44,7 +44,7 @@ def parse():
     p.add_argument("--no-decode", action="store_true", help="skip the decode tokens/s leg")
     p.add_argument("--no-gemm", action="store_true", help="skip the small-batch GEMM leg")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
-    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "gemm"], default="full",
+    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "gemm", "group"], default="full",
                    help="kernel: only the dominant GEMV (4096x14336) over its weight ring, for counter runs; "
                         "copy: a plain 64 MiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE; "
                         "decode / gemm: only that leg (for kernel traces)")
@@ -207,6 +207,22 @@ def main():
     if a.mode == "gemm":
         print(json.dumps({"mode": "gemm", "gemm_w2g128_llama2_13b": gemm_leg(torch, lib, dev, a.steps)}))
         return
+    if a.mode == "group":
+        # the whole sweep as one grouped launch, `steps` times (for rocprofv3 --kernel-trace)
+        from elutq_amd.hlq_linear import GemvGroup
+        mods, nbytes = [], 0
+        for i in range(N_LAYERS):
+            for (k, n) in LLAMA3_8B_SHAPES.values():
+                mods.append(make_device_layer(k, n, BITS, GROUP, seed=len(mods), device=dev))
+                nbytes += algorithmic_bytes(k, n, BITS, GROUP)
+        xk = {k: torch.randn(1, k, device=dev).to(torch.float16) for k in {m.in_features for m in mods}}
+        grp = GemvGroup(mods, [xk[m.in_features] for m in mods],
+                        [torch.empty(1, m.out_features, dtype=torch.float16, device=dev) for m in mods])
+        sec = time_graph(torch, lambda s: grp.run(), a.steps, a.warmup)
+        print(json.dumps({"mode": "group", "gemvs_per_launch": len(mods), "bytes_per_launch": nbytes, "us_per_launch": sec * 1e6,
+                          "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}))
+        grp.close()
+        return
     if a.mode != "full":
         counter_mode(a, torch, lib, dev)
         return
@@ -233,6 +249,28 @@ def main():
 
     sec_step = time_graph(torch, launch_step, a.steps, a.warmup)
     value = step_bytes / sec_step / 1e9
+
+    # ---- the same sweep through the grouped entry point: one launch for all 224 GEMVs, and one
+    # launch per layer (7 GEMVs); every GEMV writes its own output ---------------------------------
+    from elutq_amd.hlq_linear import GemvGroup
+    g_mods = [c.mod for c in calls]
+    g_xs = [xs[m.in_features] for m in g_mods]
+    g_ys = [torch.empty(1, m.out_features, dtype=torch.float16, device=dev) for m in g_mods]
+    grouped = {}
+    for label, per in (("one_launch", len(g_mods)), ("launch_per_layer", len(LLAMA3_8B_SHAPES))):
+        groups = [GemvGroup(g_mods[i:i + per], g_xs[i:i + per], g_ys[i:i + per]) for i in range(0, len(g_mods), per)]
+
+        def launch_groups(stream, groups=groups):
+            for g in groups:
+                g.run()
+
+        sec = time_graph(torch, launch_groups, a.steps, a.warmup)
+        grouped[label] = {"launches": len(groups), "ms_per_step": sec * 1e3, "GBps": step_bytes / sec / 1e9,
+                          "frac_hbm_peak": step_bytes / sec / 1e9 / HBM_PEAK_GBPS}
+        for g in groups:
+            g.close()
+    del g_ys
+    torch.cuda.empty_cache()
 
     # ---- per shape, each over a ring of weight sets > 512 MB ------------------------------
     per_shape = {}
@@ -280,6 +318,9 @@ def main():
         "frac_hbm_peak": value / HBM_PEAK_GBPS,
         "per_shape": per_shape,
         "roofline": roofline,
+        # supplementary: the same 224 GEMVs handed to elutq_hlq_gemv_group_* (they are independent in this
+        # sweep); `value` above stays the one-call-per-GEMV figure of the drop-in entry point
+        "grouped_sweep": grouped,
     }
 
     if not a.no_gemm:

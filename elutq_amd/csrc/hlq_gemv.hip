@@ -197,10 +197,10 @@ __device__ __forceinline__ void chunk_values(int prologue, uint2 raw, uint2 raw2
 // Always two loads (without a prologue the second one re-reads the chunk): a fixed number
 // of loads lets the compiler wait for these with an exact vector-memory count while the
 // weight loads issued after them are still in flight.
-__device__ __forceinline__ void load_chunk(const GemvArgs &a, int K, size_t k, uint2 &raw, uint2 &raw2)
+__device__ __forceinline__ void load_chunk(const GemvArgs &a, int prologue, int K, size_t k, uint2 &raw, uint2 &raw2)
 {
     raw = *(const uint2 *)(a.x + k);
-    const uint16_t *second = a.prologue == 1 ? a.norm_w + k : (a.prologue == 2 ? a.x + (size_t)K + k : a.x + k);
+    const uint16_t *second = prologue == 1 ? a.norm_w + k : (prologue == 2 ? a.x + (size_t)K + k : a.x + k);
     raw2 = *(const uint2 *)second;
 }
 
@@ -271,9 +271,17 @@ constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 // GEMV); `red_sel` picks one of two cross-wave buffers so that a caller that runs tiles
 // back to back needs no barrier between them: waves other than wave 0 may start the next
 // tile while wave 0 still sums and stores this one.
-template <int BITS, bool G64, int NSLOT>
-__device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, unsigned char *smem, int red_sel)
+//
+// MULTI: the tile covers `ncb_run` consecutive column blocks of the same slice.  The tables are
+// built once; while a wave looks up its sub-tasks of one column block, each slot it has
+// consumed is refilled with the same sub-task of the next block, so the weight stream never
+// stops between blocks.  Needs runs of at most NSLOT sub-tasks per wave.
+// PLAIN: no prologue and no residual (their fields of `a` are not read).
+template <int BITS, bool G64, int NSLOT, bool MULTI, bool PLAIN>
+__device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb_run, unsigned char *smem, int &red_sel)
 {
+    const int prologue = PLAIN ? 0 : a.prologue;
+    const uint16_t *residual = PLAIN ? nullptr : a.residual;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cb = vblock / a.ksplit, slice = vblock - cb * a.ksplit;
@@ -287,7 +295,6 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, unsigne
     unsigned char *lut = smem + (size_t)wave * a.wave_lds;                 // this wave's tables [nuw][32][16] int32
     float2 *xs_inv = (float2 *)(lut + (size_t)a.nuw_max * UNIT_LUT_BYTES); // [2 * nuw_max]
     float *red0 = (float *)(smem + (size_t)nw * a.wave_lds);               // [2][nw][64]
-    float *red = red0 + red_sel * nw * HLQ_CB;
     float *rstd_scratch = red0 + 2 * nw * HLQ_CB;                          // [RSTD_SCRATCH]
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
@@ -300,10 +307,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, unsigne
     const size_t k0 = (size_t)(u0 + ub) * HLQ_UNIT;
     const int nchunks = nuw * 32;
     float rstd = 1.f;
-    if (a.prologue == 1) rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x);
+    if (prologue == 1) rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x);
     uint2 raw, raw2;
     // lanes past the run (and waves without one, whose k0 is the end of the slice) re-read a valid chunk
-    load_chunk(a, K, nchunks ? k0 + (size_t)min(lane, nchunks - 1) * 4 : 0, raw, raw2);
+    load_chunk(a, prologue, K, nchunks ? k0 + (size_t)min(lane, nchunks - 1) * 4 : 0, raw, raw2);
     asm volatile("" ::: "memory");      // keep both activation loads ahead of the weight loads
 
     const uint32_t mask = 0x3Cu;
@@ -318,7 +325,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, unsigne
     // ... the tables are built as soon as the activations are in (a wave that first queued all
     // its weight loads would sit in the memory pipeline's back-pressure instead) ...
     if (lane < nchunks)
-        build_chunk(a.prologue, raw, raw2, rstd, lut + (size_t)lane * TBL_BYTES, xs_inv + (lane >> 4), (lane & 15) == 0);
+        build_chunk(prologue, raw, raw2, rstd, lut + (size_t)lane * TBL_BYTES, xs_inv + (lane >> 4), (lane & 15) == 0);
     asm volatile("" ::: "memory");
 
     // ... and the rest of the run's loads follow.
@@ -328,8 +335,8 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, unsigne
         load_sub<BITS, G64>(slot[d], a, cb, u0 + st / BITS, st % BITS, lane);
     }
     for (int ci = lane + 64; ci < nchunks; ci += 64) {      // runs of more than two units (not the common case)
-        load_chunk(a, K, k0 + (size_t)ci * 4, raw, raw2);
-        build_chunk(a.prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0);
+        load_chunk(a, prologue, K, k0 + (size_t)ci * 4, raw, raw2);
+        build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0);
     }
     HLQ_STAMP(1);
     // The tables were written by this wave and are read by this wave: LDS executes a wave's
@@ -337,6 +344,87 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, unsigne
     asm volatile("" ::: "memory");
     __builtin_amdgcn_wave_barrier();
     HLQ_STAMP(2);
+
+    // Combine the waves of this workgroup, then the slices of this column block.
+    auto finish = [&](int cbf, float accf) __attribute__((always_inline)) {
+        float *red = red0 + red_sel * nw * HLQ_CB;
+        red_sel ^= 1;
+        const int n = cbf * HLQ_CB + lane;
+        float total = accf;
+        if (nw > 1) {
+            red[wave * HLQ_CB + lane] = accf;
+            __syncthreads();
+            if (wave == 0) {
+                total = 0.f;
+                for (int w = 0; w < nw; w++) total += red[w * HLQ_CB + lane];
+            }
+        }
+        HLQ_STAMP(4);
+        if (a.ksplit == 1) {
+            if (wave == 0 && n < a.N) {
+                if (a.bias) total += (float)__builtin_bit_cast(_Float16, a.bias[n]);
+                if (residual) total += (float)__builtin_bit_cast(_Float16, residual[n]);
+                a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)total);
+            }
+            return;
+        }
+        // Slices meet through device memory.  Partial sums are written and read with
+        // agent-scope atomics (they bypass the per-XCD L2s' non-coherent lines), the writer
+        // waits for its stores to be acknowledged before it takes a ticket, and the reader's
+        // loads depend on the ticket it drew -- so no cache write-back / invalidate is needed.
+        const size_t npad = (size_t)a.ncb * HLQ_CB;
+        if (wave == 0) {
+            __hip_atomic_store(&a.partial[(size_t)slice * npad + n], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            HLQ_STAMP(5);
+            unsigned ticket = 0;
+            if (lane == 0)
+                ticket = __hip_atomic_fetch_add(&a.counters[cbf], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            ticket = __builtin_amdgcn_readfirstlane(ticket);
+            HLQ_STAMP(6);
+            if (ticket == (unsigned)a.ksplit - 1u) {
+                // eight independent loads in flight at a time, summed in slice order
+                float sum = 0.f;
+                for (int s0 = 0; s0 < a.ksplit; s0 += 8) {
+                    float v[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) {
+                        const int sl = min(s0 + j, a.ksplit - 1);
+                        v[j] = __hip_atomic_load(&a.partial[(size_t)sl * npad + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 8; j++)
+                        if (s0 + j < a.ksplit) sum += v[j];
+                }
+                if (n < a.N) {
+                    if (a.bias) sum += (float)__builtin_bit_cast(_Float16, a.bias[n]);
+                    if (residual) sum += (float)__builtin_bit_cast(_Float16, residual[n]);
+                    a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
+                }
+                if (lane == 0) __hip_atomic_store(&a.counters[cbf], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                HLQ_STAMP(7);
+            }
+        }
+    };
+
+    if (MULTI) {
+        for (int c = 0; c < ncb_run; c++) {
+            const int cbn = min(cb + c + 1, cb + ncb_run - 1);        // past the run: a reload nobody reads
+            float accc = 0.f;
+#pragma unroll
+            for (int d = 0; d < NSLOT; d++) {
+                const int st = s_begin + d;
+                if (st < s_end) {
+                    const int u = st / BITS;
+                    accc = process_sub<G64>(slot[d], u - ub, st % BITS, (u0 + u) & 1, lut_base, xs_inv, mask, accc);
+                }
+                const int sn = min(st, s_last);
+                load_sub<BITS, G64>(slot[d], a, cbn, u0 + sn / BITS, sn % BITS, lane);
+            }
+            finish(cb + c, accc);
+        }
+        return;
+    }
 
     // Slot d holds sub-task base + d; it is refilled with sub-task base + d + NSLOT as soon as
     // it has been consumed (past the end of the run: a reload nobody reads).
@@ -354,72 +442,16 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, unsigne
             }
         }
     }
-
     HLQ_STAMP(3);
-    // Combine the waves of this workgroup, then the slices of this column block.
-    const int n = cb * HLQ_CB + lane;
-    float total = acc;
-    if (nw > 1) {
-        red[wave * HLQ_CB + lane] = acc;
-        __syncthreads();
-        if (wave == 0) {
-            total = 0.f;
-            for (int w = 0; w < nw; w++) total += red[w * HLQ_CB + lane];
-        }
-    }
-    HLQ_STAMP(4);
-    if (a.ksplit == 1) {
-        if (wave == 0 && n < a.N) {
-            if (a.bias) total += (float)__builtin_bit_cast(_Float16, a.bias[n]);
-            if (a.residual) total += (float)__builtin_bit_cast(_Float16, a.residual[n]);
-            a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)total);
-        }
-        return;
-    }
-    // Slices meet through device memory.  Partial sums are written and read with
-    // agent-scope atomics (they bypass the per-XCD L2s' non-coherent lines), the writer
-    // waits for its stores to be acknowledged before it takes a ticket, and the reader's
-    // loads depend on the ticket it drew -- so no cache write-back / invalidate is needed.
-    const size_t npad = (size_t)a.ncb * HLQ_CB;
-    if (wave == 0) {
-        __hip_atomic_store(&a.partial[(size_t)slice * npad + n], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        HLQ_STAMP(5);
-        unsigned ticket = 0;
-        if (lane == 0)
-            ticket = __hip_atomic_fetch_add(&a.counters[cb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ticket = __builtin_amdgcn_readfirstlane(ticket);
-        HLQ_STAMP(6);
-        if (ticket == (unsigned)a.ksplit - 1u) {
-            // eight independent loads in flight at a time, summed in slice order
-            float sum = 0.f;
-            for (int s0 = 0; s0 < a.ksplit; s0 += 8) {
-                float v[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const int s = min(s0 + j, a.ksplit - 1);
-                    v[j] = __hip_atomic_load(&a.partial[(size_t)s * npad + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-#pragma unroll
-                for (int j = 0; j < 8; j++)
-                    if (s0 + j < a.ksplit) sum += v[j];
-            }
-            if (n < a.N) {
-                if (a.bias) sum += (float)__builtin_bit_cast(_Float16, a.bias[n]);
-                if (a.residual) sum += (float)__builtin_bit_cast(_Float16, a.residual[n]);
-                a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
-            }
-            if (lane == 0) __hip_atomic_store(&a.counters[cb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            HLQ_STAMP(7);
-        }
-    }
+    finish(cb, acc);
 }
 
 template <int BITS, bool G64, int NSLOT>
 __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 {
     extern __shared__ __align__(256) unsigned char smem[];
-    gemv_tile<BITS, G64, NSLOT>(a, blockIdx.x, smem, 0);
+    int sel = 0;
+    gemv_tile<BITS, G64, NSLOT, false, false>(a, blockIdx.x, 1, smem, sel);
 }
 
 // Many independent GEMVs in one launch: the tiles of all of them form one list that the
@@ -430,7 +462,8 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 // per GEMV, and with two workgroups per CU the sum-and-store of one tile hides under the
 // lookups of another.
 struct GroupItem {
-    int problem, vblock;
+    int problem, vblock;     // vblock = first column block * ksplit + slice
+    int ncb_run;             // consecutive column blocks of that slice
 };
 
 template <int BITS, bool G64, int NSLOT>
@@ -438,10 +471,10 @@ __global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *pr
 {
     extern __shared__ __align__(256) unsigned char smem[];
     int sel = 0;
-    for (int i = blockIdx.x; i < n_items; i += gridDim.x, sel ^= 1) {
+    for (int i = blockIdx.x; i < n_items; i += gridDim.x) {
         const GroupItem it = items[i];
         const GemvArgs a = problems[it.problem];
-        gemv_tile<BITS, G64, NSLOT>(a, it.vblock, smem, sel);
+        gemv_tile<BITS, G64, NSLOT, true, true>(a, it.vblock, it.ncb_run, smem, sel);
     }
 }
 
@@ -507,6 +540,7 @@ int dispatch_gemv(const GemvArgs &a, int bits, int group, int waves, size_t lds,
     return ELUTQ_ERR_BITS;
 }
 
+// grid < 0: no launch, returns the number of workgroups of this shape a CU holds at once
 template <int BITS, bool G64, int NSLOT>
 int launch_group_n(const GemvArgs *d_problems, const GroupItem *d_items, int n_items, int grid, int waves, size_t lds,
                    hipStream_t stream)
@@ -517,6 +551,12 @@ int launch_group_n(const GemvArgs *d_problems, const GroupItem *d_items, int n_i
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS) != hipSuccess)
             return ELUTQ_ERR_HIP;
         big_lds_enabled = true;
+    }
+    if (grid < 0) {
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)kern, waves * 64, lds) != hipSuccess || per_cu < 1)
+            return 1;
+        return per_cu;
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(waves * 64), lds, stream, d_problems, d_items, n_items);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
@@ -662,10 +702,13 @@ static int group_shape(const elutq_gemv_problem &p, int bits, int group, GroupSh
     if (rc != ELUTQ_OK) return rc;
     if (!p.d_planes || !p.d_scales || !p.d_zeros || !p.d_x || !p.d_y) return ELUTQ_ERR_NULL;
     sh.g = hlq_geo(p.K, p.N, bits, group);
-    // the list supplies the parallelism: slice K only as far as run length and LDS ask for
-    int ksplit = (sh.g.U + 31) / 32;
+    // the list supplies the parallelism: slice K only as far as LDS and the run length ask for
+    // (a wave's run must fit its DEPTH slots: at most 16 * DEPTH sub-tasks per slice)
+    int ksplit = (sh.g.U * bits + 16 * DEPTH - 1) / (16 * DEPTH);
     int ups = (sh.g.U + ksplit - 1) / ksplit;
-    while (gemv_lds_bytes(ups, bits, 16) > (size_t)MAX_LDS / 2) ups = (ups + 1) / 2;     // two workgroups per CU
+    while (ups > 1 && (gemv_lds_bytes(ups, bits, 16) > (size_t)MAX_LDS / 2 ||            // two workgroups per CU
+                       wave_plan(ups, bits, 16).spw > DEPTH))                            // whole units per wave may round the run up
+        ups--;
     sh.ups = ups;
     sh.ksplit = (sh.g.U + ups - 1) / ups;
     sh.wp = wave_plan(ups, bits, 16);
@@ -730,6 +773,12 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
     }
     std::vector<GemvArgs> args(count);
     std::vector<GroupItem> items;
+    // column blocks per tile: long runs amortise the table build, as long as every CU still gets a tile
+    long total_cbs = 0;
+    for (auto &sh : shapes) total_cbs += (long)sh.g.ncb * sh.ksplit;
+    int cbs_per_item = (int)((total_cbs + NUM_CU - 1) / NUM_CU);
+    if (cbs_per_item > 16) cbs_per_item = 16;
+    if (cbs_per_item < 1) cbs_per_item = 1;
     int nslot = 1;
     size_t lds = 0;
     for (int i = 0; i < count; i++) {
@@ -754,11 +803,20 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
         if (ns > nslot) nslot = ns;
         const size_t l = gemv_lds_bytes(sh.ups, bits, 16);
         if (l > lds) lds = l;
-        for (int vb = 0; vb < sh.g.ncb * sh.ksplit; vb++) items.push_back(GroupItem{i, vb});
+        // runs of column blocks share one table build
+        for (int sl = 0; sl < sh.ksplit; sl++)
+            for (int cb0 = 0; cb0 < sh.g.ncb; cb0 += cbs_per_item) {
+                const int len = sh.g.ncb - cb0 < cbs_per_item ? sh.g.ncb - cb0 : cbs_per_item;
+                items.push_back(GroupItem{i, cb0 * sh.ksplit + sl, len});
+            }
     }
     GemvGroupPlan *pl = new GemvGroupPlan();
     pl->bits = bits; pl->group = group; pl->nslot = nslot; pl->n_items = (int)items.size(); pl->lds = lds;
-    const int slots = NUM_CU * (lds <= (size_t)MAX_LDS / 2 ? 2 : 1);
+    // as many workgroups as the chip holds at once: each walks the list with that stride
+    int per_cu = dispatch_group(bits, group == 64, nslot, nullptr, nullptr, 0, -1, 16, lds, nullptr);
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 2) per_cu = 2;
+    const int slots = NUM_CU * per_cu;
     pl->grid = pl->n_items < slots ? pl->n_items : slots;
     pl->d_problems = nullptr; pl->d_items = nullptr;
     if (hipMalloc((void **)&pl->d_problems, args.size() * sizeof(GemvArgs)) != hipSuccess ||
