@@ -270,6 +270,12 @@ def main():
         for g in groups:
             g.close()
     del g_ys
+    # what a plain device-to-device copy reaches on this GPU (read + write bytes), as a yardstick
+    cp_a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    cp_b = torch.empty_like(cp_a)
+    sec = time_graph(torch, lambda s: cp_b.copy_(cp_a), 10, 2)
+    grouped["device_copy_1GiB_GBps"] = 2 * cp_a.numel() / sec / 1e9
+    del cp_a, cp_b
     torch.cuda.empty_cache()
 
     # ---- per shape, each over a ring of weight sets > 512 MB ------------------------------

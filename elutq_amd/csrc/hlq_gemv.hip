@@ -37,15 +37,24 @@ constexpr int MAX_LDS = HLQ_MAX_LDS;
 constexpr int TBL_BYTES = 64;                    // 16 int32 entries
 constexpr int UNIT_LUT_BYTES = 32 * TBL_BYTES;   // 32 chunks per unit
 
+// Device pointers are declared in the global address space for the device pass: a pointer that a
+// kernel reads out of a struct in memory (the grouped launch) would otherwise be generic, and
+// generic loads count on the LDS counter too, which serialises them with the table lookups.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define HLQ_GLOBAL __attribute__((address_space(1)))
+#else
+#define HLQ_GLOBAL
+#endif
+
 struct GemvArgs {
-    const uint4 *planes;
-    const uint32_t *scales;
-    const uint32_t *zeros;
-    const uint16_t *bias;    // fp16 or null
-    const uint16_t *x;       // fp16 [K]
-    uint16_t *y;             // fp16 [N]
-    float *partial;          // [ksplit][ncb*64]   (ksplit > 1)
-    unsigned *counters;      // [ncb], zero between calls
+    const HLQ_GLOBAL uint4 *planes;
+    const HLQ_GLOBAL uint32_t *scales;
+    const HLQ_GLOBAL uint32_t *zeros;
+    const HLQ_GLOBAL uint16_t *bias;    // fp16 or null
+    const HLQ_GLOBAL uint16_t *x;       // fp16 [K]
+    HLQ_GLOBAL uint16_t *y;             // fp16 [N]
+    HLQ_GLOBAL float *partial;          // [ksplit][ncb*64]   (ksplit > 1)
+    HLQ_GLOBAL unsigned *counters;      // [ncb], zero between calls
     int N, U, NT, ncb;
     int ksplit, ups;         // slices per column block, units per slice
     int spw;                 // sub-tasks per wave (contiguous run)
@@ -53,8 +62,8 @@ struct GemvArgs {
     // optional fusion with the ops around the projection in a decoder layer
     int prologue;            // 0: x as is; 1: rmsnorm(x) * norm_w; 2: silu(x[0:K]) * x[K:2K]
     float eps;
-    const uint16_t *norm_w;  // fp16 [K]      (prologue 1)
-    const uint16_t *residual;  // fp16 [N] added to the output, or null
+    const HLQ_GLOBAL uint16_t *norm_w;  // fp16 [K]      (prologue 1)
+    const HLQ_GLOBAL uint16_t *residual;  // fp16 [N] added to the output, or null
 };
 
 #ifdef HLQ_TIMING
@@ -127,7 +136,7 @@ struct Sub {
 template <int BITS, bool G64>
 __device__ __forceinline__ void load_sub(Sub &t, const GemvArgs &a, int cb, int u, int b, int lane)
 {
-    const u32x4 v = __builtin_nontemporal_load((const u32x4 *)(a.planes + (((size_t)cb * a.U + u) * BITS + b) * HLQ_CB + lane));
+    const u32x4 v = __builtin_nontemporal_load((const HLQ_GLOBAL u32x4 *)(a.planes + (((size_t)cb * a.U + u) * BITS + b) * HLQ_CB + lane));
     t.w = make_uint4(v.x, v.y, v.z, v.w);
     const size_t m = (size_t)cb * a.NT + (G64 ? u : (u >> 1));
     t.sc = a.scales[(m * BITS + b) * HLQ_CB + lane];
@@ -199,9 +208,9 @@ __device__ __forceinline__ void chunk_values(int prologue, uint2 raw, uint2 raw2
 // weight loads issued after them are still in flight.
 __device__ __forceinline__ void load_chunk(const GemvArgs &a, int prologue, int K, size_t k, uint2 &raw, uint2 &raw2)
 {
-    raw = *(const uint2 *)(a.x + k);
-    const uint16_t *second = prologue == 1 ? a.norm_w + k : (prologue == 2 ? a.x + (size_t)K + k : a.x + k);
-    raw2 = *(const uint2 *)second;
+    raw = *(const HLQ_GLOBAL uint2 *)(a.x + k);
+    const HLQ_GLOBAL uint16_t *second = prologue == 1 ? a.norm_w + k : (prologue == 2 ? a.x + (size_t)K + k : a.x + k);
+    raw2 = *(const HLQ_GLOBAL uint2 *)second;
 }
 
 // Subset-sum table of one chunk of 4 activations as int32 fixed point, 64 bytes at `tbl`.
@@ -241,7 +250,7 @@ __device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scr
 {
     float ssq = 0.f;
     for (int i = tid; i < K / 4; i += nthreads) {
-        const uint2 r = *(const uint2 *)(a.x + (size_t)i * 4);
+        const uint2 r = *(const HLQ_GLOBAL uint2 *)(a.x + (size_t)i * 4);
         const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
         ssq += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
     }
@@ -281,7 +290,7 @@ template <int BITS, bool G64, int NSLOT, bool MULTI, bool PLAIN>
 __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb_run, unsigned char *smem, int &red_sel)
 {
     const int prologue = PLAIN ? 0 : a.prologue;
-    const uint16_t *residual = PLAIN ? nullptr : a.residual;
+    const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int cb = vblock / a.ksplit, slice = vblock - cb * a.ksplit;
@@ -411,6 +420,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb
         for (int c = 0; c < ncb_run; c++) {
             const int cbn = min(cb + c + 1, cb + ncb_run - 1);        // past the run: a reload nobody reads
             float accc = 0.f;
+            HLQ_STAMP(2);
 #pragma unroll
             for (int d = 0; d < NSLOT; d++) {
                 const int st = s_begin + d;
@@ -421,7 +431,9 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb
                 const int sn = min(st, s_last);
                 load_sub<BITS, G64>(slot[d], a, cbn, u0 + sn / BITS, sn % BITS, lane);
             }
+            HLQ_STAMP(3);
             finish(cb + c, accc);
+            HLQ_STAMP(6);
         }
         return;
     }
@@ -467,7 +479,8 @@ struct GroupItem {
 };
 
 template <int BITS, bool G64, int NSLOT>
-__global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *problems, const GroupItem *items, int n_items)
+__global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *__restrict__ problems,
+                                                              const GroupItem *__restrict__ items, int n_items)
 {
     extern __shared__ __align__(256) unsigned char smem[];
     int sel = 0;
@@ -658,12 +671,12 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
     ksplit = (g.U + ups - 1) / ups;
 
     GemvArgs a;
-    a.planes = (const uint4 *)d_planes;
-    a.scales = (const uint32_t *)d_scales;
-    a.zeros = (const uint32_t *)d_zeros;
-    a.bias = (const uint16_t *)d_bias;
-    a.x = (const uint16_t *)d_x;
-    a.y = (uint16_t *)d_y;
+    a.planes = (const HLQ_GLOBAL uint4 *)d_planes;
+    a.scales = (const HLQ_GLOBAL uint32_t *)d_scales;
+    a.zeros = (const HLQ_GLOBAL uint32_t *)d_zeros;
+    a.bias = (const HLQ_GLOBAL uint16_t *)d_bias;
+    a.x = (const HLQ_GLOBAL uint16_t *)d_x;
+    a.y = (HLQ_GLOBAL uint16_t *)d_y;
     a.N = N; a.U = g.U; a.NT = g.NT; a.ncb = g.ncb;
     a.ksplit = ksplit; a.ups = ups;
     const WavePlan wp = wave_plan(ups, bits, waves);
@@ -675,16 +688,16 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
         if (fusion->prologue == 1 && !fusion->d_norm_weight) return ELUTQ_ERR_NULL;
         a.prologue = fusion->prologue;
         a.eps = fusion->eps;
-        a.norm_w = (const uint16_t *)fusion->d_norm_weight;
-        a.residual = (const uint16_t *)fusion->d_residual;
+        a.norm_w = (const HLQ_GLOBAL uint16_t *)fusion->d_norm_weight;
+        a.residual = (const HLQ_GLOBAL uint16_t *)fusion->d_residual;
     }
     if (ksplit > 1) {
         if (!d_workspace) return ELUTQ_ERR_NULL;
         if ((size_t)g.ncb * sizeof(unsigned) > (size_t)WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
         if (workspace_bytes < (size_t)WS_COUNTER_BYTES + (size_t)ksplit * g.ncb * HLQ_CB * sizeof(float))
             return ELUTQ_ERR_WORKSPACE;
-        a.counters = (unsigned *)d_workspace;
-        a.partial = (float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
+        a.counters = (HLQ_GLOBAL unsigned *)d_workspace;
+        a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves), (hipStream_t)stream);
 }
@@ -784,19 +797,19 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
     for (int i = 0; i < count; i++) {
         const GroupShape &sh = shapes[i];
         GemvArgs &a = args[i];
-        a.planes = (const uint4 *)problems[i].d_planes;
-        a.scales = (const uint32_t *)problems[i].d_scales;
-        a.zeros = (const uint32_t *)problems[i].d_zeros;
-        a.bias = (const uint16_t *)problems[i].d_bias;
-        a.x = (const uint16_t *)problems[i].d_x;
-        a.y = (uint16_t *)problems[i].d_y;
+        a.planes = (const HLQ_GLOBAL uint4 *)problems[i].d_planes;
+        a.scales = (const HLQ_GLOBAL uint32_t *)problems[i].d_scales;
+        a.zeros = (const HLQ_GLOBAL uint32_t *)problems[i].d_zeros;
+        a.bias = (const HLQ_GLOBAL uint16_t *)problems[i].d_bias;
+        a.x = (const HLQ_GLOBAL uint16_t *)problems[i].d_x;
+        a.y = (HLQ_GLOBAL uint16_t *)problems[i].d_y;
         a.N = problems[i].N; a.U = sh.g.U; a.NT = sh.g.NT; a.ncb = sh.g.ncb;
         a.ksplit = sh.ksplit; a.ups = sh.ups;
         a.spw = sh.wp.spw; a.nuw_max = sh.wp.nuw_max; a.wave_lds = sh.wp.wave_lds;
         a.partial = nullptr; a.counters = nullptr;
         if (sh.ksplit > 1) {
-            a.counters = (unsigned *)((unsigned char *)d_workspace + coff[i]);
-            a.partial = (float *)((unsigned char *)d_workspace + poff[i]);
+            a.counters = (HLQ_GLOBAL unsigned *)((unsigned char *)d_workspace + coff[i]);
+            a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + poff[i]);
         }
         a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr;
         const int ns = a.spw < DEPTH ? a.spw : DEPTH;
