@@ -466,6 +466,18 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
     gemv_tile<BITS, G64, NSLOT, false, false>(a, blockIdx.x, 1, smem, sel);
 }
 
+// One GEMV with more column blocks than the chip has CUs: every workgroup takes a run of
+// consecutive column blocks (tables built once, weights prefetched across the blocks) instead
+// of the launch holding two workgroups per CU that each build the same tables.
+template <int BITS, bool G64, int NSLOT>
+__global__ __launch_bounds__(1024) void hlq_gemv_run_kernel(const GemvArgs a, int run)
+{
+    extern __shared__ __align__(256) unsigned char smem[];
+    const int cb0 = (blockIdx.x / a.ksplit) * run, slice = blockIdx.x % a.ksplit;
+    int sel = 0;
+    gemv_tile<BITS, G64, NSLOT, true, false>(a, cb0 * a.ksplit + slice, min(run, a.ncb - cb0), smem, sel);
+}
+
 // Many independent GEMVs in one launch: the tiles of all of them form one list that the
 // workgroups walk with stride gridDim.x (tiles of one GEMV are neighbours in the list, so its
 // activations stay in cache and the slices of a column block run at about the same time).
@@ -515,6 +527,8 @@ size_t gemv_lds_bytes(int ups, int bits, int waves)
     return (size_t)waves * p.wave_lds + 2 * (size_t)waves * HLQ_CB * sizeof(float) + RSTD_SCRATCH * sizeof(float) + 16;
 }
 
+constexpr int NUM_CU_RUN = HLQ_NUM_CU;
+
 template <int BITS, bool G64, int NSLOT>
 int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
@@ -524,6 +538,20 @@ int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS) != hipSuccess)
             return ELUTQ_ERR_HIP;
         big_lds_enabled = true;
+    }
+    // more tiles than CUs and runs that fit the slots: runs of column blocks, one workgroup per CU
+    const int run = (a.ncb * a.ksplit + NUM_CU_RUN - 1) / NUM_CU_RUN;
+    if (run > 1 && a.spw <= NSLOT && waves == 16) {
+        auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT>;
+        static bool big_lds_run = false;
+        if (lds > 64 * 1024 && !big_lds_run) {
+            if (hipFuncSetAttribute((const void *)kern_run, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS) != hipSuccess)
+                return ELUTQ_ERR_HIP;
+            big_lds_run = true;
+        }
+        const int groups = (a.ncb + run - 1) / run;
+        hipLaunchKernelGGL(kern_run, dim3(groups * a.ksplit), dim3(waves * 64), lds, stream, a, run);
+        return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
     }
     hipLaunchKernelGGL(kern, dim3(a.ncb * a.ksplit), dim3(waves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
