@@ -303,6 +303,29 @@ def main():
         del extra, ring
         torch.cuda.empty_cache()
 
+    # ---- the same four shapes at w3g128 and w2g64 (plane count and group size in the fold) ---
+    other_formats = {}
+    for bits, group in ((3, 128), (2, 64)):
+        res = {}
+        for (k, n) in sorted(set(LLAMA3_8B_SHAPES.values())):
+            nbytes = algorithmic_bytes(k, n, bits, group)
+            ring = []
+            for i in range(-(-512 * 2 ** 20 // nbytes)):
+                mod = make_device_layer(k, n, bits, group, seed=20_000 + i + k, device=dev)
+                ring.append(Gemv(lib, mod, xs[k], ys[n], ws))
+
+            def launch_ring(stream, ring=ring):
+                for c in ring:
+                    c(stream)
+
+            reps = max(3, min(a.steps, int(20000 / len(ring)) + 1))
+            sec = time_graph(torch, launch_ring, reps, 2) / len(ring)
+            res[f"{k}x{n}"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                               "bytes": nbytes}
+            del ring
+            torch.cuda.empty_cache()
+        other_formats[f"w{bits}g{group}"] = res
+
     dom = per_shape["4096x14336"]
     roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": dom["GBps"] / HBM_PEAK_GBPS,
@@ -323,6 +346,7 @@ def main():
                    "bits": BITS, "group": GROUP, "bytes_per_step": step_bytes, "gemvs_per_step": len(calls)},
         "frac_hbm_peak": value / HBM_PEAK_GBPS,
         "per_shape": per_shape,
+        "per_shape_other_formats": other_formats,
         "roofline": roofline,
         # supplementary: the same 224 GEMVs handed to elutq_hlq_gemv_group_* (they are independent in this
         # sweep); `value` above stays the one-call-per-GEMV figure of the drop-in entry point
