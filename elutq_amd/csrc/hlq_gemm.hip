@@ -417,6 +417,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
     GEMM_STAMP(15);
 }
 
+// Kernels that need more than 64 KiB of dynamic LDS must be told so once per device (the
+// setting is sticky); `done` is the caller's per-kernel table of devices already set.
+inline bool allow_big_lds(const void *kern, size_t lds, int limit, bool (&done)[64])
+{
+    if (lds <= 64 * 1024) return true;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    if (!done[dev]) {
+        if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, limit) != hipSuccess) return false;
+        done[dev] = true;
+    }
+    return true;
+}
+
 template <int MT, int KW>
 size_t gemm_lds_bytes()
 {
@@ -430,12 +444,8 @@ int launch_gemm(const GemmArgs &a, hipStream_t stream)
 {
     auto kern = hlq_gemm_kernel<BITS, G64, MT, KW>;
     const size_t lds = gemm_lds_bytes<MT, KW>();
-    static bool big_lds_enabled = false;
-    if (lds > 64 * 1024 && !big_lds_enabled) {
-        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-            return ELUTQ_ERR_HIP;
-        big_lds_enabled = true;
-    }
+    static bool big_lds_done[64] = {};        // per template instance
+    if (!allow_big_lds((const void *)kern, lds, (int)lds, big_lds_done)) return ELUTQ_ERR_HIP;
     const int cbw = GW / KW, nsb = (a.ncb + cbw - 1) / cbw;
     hipLaunchKernelGGL(kern, dim3(nsb * a.ksplit), dim3(GEMM_THREADS), lds, stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;

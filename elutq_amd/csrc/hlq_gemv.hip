@@ -529,26 +529,33 @@ size_t gemv_lds_bytes(int ups, int bits, int waves)
 
 constexpr int NUM_CU_RUN = HLQ_NUM_CU;
 
+// Kernels that need more than 64 KiB of dynamic LDS must be told so once per device (the
+// setting is sticky); `done` is the caller's per-kernel table of devices already set.
+inline bool allow_big_lds(const void *kern, size_t lds, int limit, bool (&done)[64])
+{
+    if (lds <= 64 * 1024) return true;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    if (!done[dev]) {
+        if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, limit) != hipSuccess) return false;
+        done[dev] = true;
+    }
+    return true;
+}
+
+
 template <int BITS, bool G64, int NSLOT>
 int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
     auto kern = hlq_gemv_kernel<BITS, G64, NSLOT>;
-    static bool big_lds_enabled = false;      // per template instance; the setting is sticky
-    if (lds > 64 * 1024 && !big_lds_enabled) {
-        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS) != hipSuccess)
-            return ELUTQ_ERR_HIP;
-        big_lds_enabled = true;
-    }
+    static bool big_lds_done[64] = {};        // per template instance
+    if (!allow_big_lds((const void *)kern, lds, MAX_LDS, big_lds_done)) return ELUTQ_ERR_HIP;
     // more tiles than CUs and runs that fit the slots: runs of column blocks, one workgroup per CU
     const int run = (a.ncb * a.ksplit + NUM_CU_RUN - 1) / NUM_CU_RUN;
     if (run > 1 && a.spw <= NSLOT && waves == 16) {
         auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT>;
-        static bool big_lds_run = false;
-        if (lds > 64 * 1024 && !big_lds_run) {
-            if (hipFuncSetAttribute((const void *)kern_run, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS) != hipSuccess)
-                return ELUTQ_ERR_HIP;
-            big_lds_run = true;
-        }
+        static bool big_lds_run_done[64] = {};
+        if (!allow_big_lds((const void *)kern_run, lds, MAX_LDS, big_lds_run_done)) return ELUTQ_ERR_HIP;
         const int groups = (a.ncb + run - 1) / run;
         hipLaunchKernelGGL(kern_run, dim3(groups * a.ksplit), dim3(waves * 64), lds, stream, a, run);
         return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
@@ -587,12 +594,8 @@ int launch_group_n(const GemvArgs *d_problems, const GroupItem *d_items, int n_i
                    hipStream_t stream)
 {
     auto kern = hlq_gemv_group_kernel<BITS, G64, NSLOT>;
-    static bool big_lds_enabled = false;
-    if (lds > 64 * 1024 && !big_lds_enabled) {
-        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_LDS) != hipSuccess)
-            return ELUTQ_ERR_HIP;
-        big_lds_enabled = true;
-    }
+    static bool big_lds_done[64] = {};
+    if (!allow_big_lds((const void *)kern, lds, MAX_LDS, big_lds_done)) return ELUTQ_ERR_HIP;
     if (grid < 0) {
         int per_cu = 0;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)kern, waves * 64, lds) != hipSuccess || per_cu < 1)
