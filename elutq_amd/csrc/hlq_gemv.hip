@@ -67,14 +67,21 @@ struct GemvArgs {
 };
 
 #ifdef HLQ_TIMING
-// Profiling builds only: per-stage wall-clock stamps (100 MHz) of wave 0 of every workgroup.
+// Profiling builds only: per-stage wall-clock stamps (100 MHz) of every wave (up to 16) of every
+// workgroup, kept in registers and written once when the tile is done.
 __device__ unsigned long long *g_hlq_stamps = nullptr;
-#define HLQ_STAMP(i)                                                                              \
+#define HLQ_STAMP_DECL unsigned long long hlq_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}
+#define HLQ_STAMP(i) hlq_t[i] = wall_clock64()
+#define HLQ_STAMP_FLUSH                                                                           \
     do {                                                                                          \
-        if (g_hlq_stamps && threadIdx.x == 0) g_hlq_stamps[(size_t)blockIdx.x * 8 + (i)] = wall_clock64(); \
+        if (g_hlq_stamps && (threadIdx.x & 63) == 0)                                              \
+            for (int hlq_i = 0; hlq_i < 8; hlq_i++)                                               \
+                g_hlq_stamps[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 8 + hlq_i] = hlq_t[hlq_i]; \
     } while (0)
 #else
+#define HLQ_STAMP_DECL do { } while (0)
 #define HLQ_STAMP(i) do { } while (0)
+#define HLQ_STAMP_FLUSH do { } while (0)
 #endif
 
 typedef __attribute__((address_space(3))) const int lds_cint;
@@ -94,9 +101,11 @@ __device__ __forceinline__ float h2f_hi(uint32_t v) { return (float)__builtin_bi
         : "+v"(a)                                                                              \
         : "v"(mask), "v"(src))
 
-// Eight lookups for one plane dword (32 k): chunks 8*D .. 8*D+7 of the unit.
+// Eight lookups for one plane dword (32 k): chunks 8*D .. 8*D+7 of the unit.  Issue and sum are
+// separate so that the lookups of the next dword are on their way to LDS before the wave waits
+// for the results of this one (LDS returns a wave's reads in order).
 template <int D>
-__device__ __forceinline__ int lookup_dword(uint32_t w, uint32_t (&a)[8], uint32_t mask, int acc)
+__device__ __forceinline__ void lookup_issue(uint32_t w, uint32_t (&a)[8], uint32_t mask, int (&v)[8])
 {
     const uint32_t r = __builtin_amdgcn_alignbit(w, w, 4);
     HLQ_SDWA_AND(a[0], mask, w, 0);
@@ -108,18 +117,16 @@ __device__ __forceinline__ int lookup_dword(uint32_t w, uint32_t (&a)[8], uint32
     HLQ_SDWA_AND(a[6], mask, w, 3);
     HLQ_SDWA_AND(a[7], mask, r, 3);
     constexpr int base = D * 8 * TBL_BYTES;
-    const int v0 = lds_ld(a[0], base + 0 * TBL_BYTES);
-    const int v1 = lds_ld(a[1], base + 1 * TBL_BYTES);
-    const int v2 = lds_ld(a[2], base + 2 * TBL_BYTES);
-    const int v3 = lds_ld(a[3], base + 3 * TBL_BYTES);
-    const int v4 = lds_ld(a[4], base + 4 * TBL_BYTES);
-    const int v5 = lds_ld(a[5], base + 5 * TBL_BYTES);
-    const int v6 = lds_ld(a[6], base + 6 * TBL_BYTES);
-    const int v7 = lds_ld(a[7], base + 7 * TBL_BYTES);
-    acc = acc + v0 + v1;
-    acc = acc + v2 + v3;
-    acc = acc + v4 + v5;
-    acc = acc + v6 + v7;
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = lds_ld(a[j], base + j * TBL_BYTES);
+}
+
+__device__ __forceinline__ int lookup_sum(const int (&v)[8], int acc)
+{
+    acc = acc + v[0] + v[1];
+    acc = acc + v[2] + v[3];
+    acc = acc + v[4] + v[5];
+    acc = acc + v[6] + v[7];
     return acc;
 }
 
@@ -133,14 +140,39 @@ struct Sub {
     uint32_t zz;   // fp16 zeros of the pair; loaded for plane 0 only, which folds the zero point
 };
 
-template <int BITS, bool G64>
-__device__ __forceinline__ void load_sub(Sub &t, const GemvArgs &a, int cb, int u, int b, int lane)
+// Byte addresses of one column block's data, uniform over the wave: every load of a sub-task
+// is one of these (scalar registers) plus a 32-bit offset, so the per-load address arithmetic
+// stays short -- the scalar unit is shared by the four SIMDs of a CU and the index arithmetic
+// of sixteen waves would otherwise hold up the start of the weight stream.
+struct CbBase {
+    const HLQ_GLOBAL unsigned char *planes;   // sub-task 0 of the slice
+    const HLQ_GLOBAL unsigned char *scales;   // meta row 0 of the column block
+    const HLQ_GLOBAL unsigned char *zeros;    // meta row 0 of the column block
+};
+
+template <int BITS>
+__device__ __forceinline__ CbBase cb_base(const GemvArgs &a, int cb, int u0)
 {
-    const u32x4 v = __builtin_nontemporal_load((const HLQ_GLOBAL u32x4 *)(a.planes + (((size_t)cb * a.U + u) * BITS + b) * HLQ_CB + lane));
+    CbBase p;
+    p.planes = (const HLQ_GLOBAL unsigned char *)a.planes + ((size_t)cb * a.U + u0) * (size_t)(BITS * HLQ_CB * 16);
+    p.scales = (const HLQ_GLOBAL unsigned char *)a.scales + (size_t)cb * a.NT * (size_t)(BITS * HLQ_CB * 4);
+    p.zeros = (const HLQ_GLOBAL unsigned char *)a.zeros + (size_t)cb * a.NT * (size_t)(HLQ_CB * 4);
+    return p;
+}
+
+// st = sub-task index inside the slice (unit u0 + st / BITS, plane st % BITS); planes of a
+// slice are contiguous in st.
+template <int BITS, bool G64>
+__device__ __forceinline__ void load_sub(Sub &t, const CbBase &p, int u0, int st, int lane)
+{
+    const uint32_t u = (uint32_t)(u0 + st / BITS), b = (uint32_t)(st % BITS);
+    const uint32_t row = G64 ? u : (u >> 1);
+    const u32x4 v = __builtin_nontemporal_load(
+        (const HLQ_GLOBAL u32x4 *)(p.planes + ((uint32_t)st * (uint32_t)(HLQ_CB * 16) + (uint32_t)lane * 16u)));
     t.w = make_uint4(v.x, v.y, v.z, v.w);
-    const size_t m = (size_t)cb * a.NT + (G64 ? u : (u >> 1));
-    t.sc = a.scales[(m * BITS + b) * HLQ_CB + lane];
-    t.zz = a.zeros[m * HLQ_CB + lane];       // used by plane 0 only; loaded always so that every sub-task is 3 loads
+    t.sc = *(const HLQ_GLOBAL uint32_t *)(p.scales + ((row * BITS + b) * (uint32_t)(HLQ_CB * 4) + (uint32_t)lane * 4u));
+    // used by plane 0 only; loaded always so that every sub-task is 3 loads
+    t.zz = *(const HLQ_GLOBAL uint32_t *)(p.zeros + (row * (uint32_t)(HLQ_CB * 4) + (uint32_t)lane * 4u));
 }
 
 // The two 64-k halves of a unit have their own table scale (2^-p) and activation sum; at
@@ -150,15 +182,24 @@ template <bool G64>
 __device__ __forceinline__ float process_sub(const Sub &t, int lu, int b, int odd, uint32_t lut_base,
                                              const float2 *xs_inv, uint32_t mask, float acc)
 {
-    uint32_t a[8];
+    // two sets of address registers (table base in the upper bytes) alternate between the dwords
+    uint32_t a0[8], a1[8];
+    int v0[8], v1[8];
     const uint32_t ub = lut_base + (uint32_t)lu * UNIT_LUT_BYTES;
 #pragma unroll
-    for (int j = 0; j < 8; j++) a[j] = ub;
+    for (int j = 0; j < 8; j++) a0[j] = a1[j] = ub;
     const float2 h0 = xs_inv[2 * lu], h1 = xs_inv[2 * lu + 1];      // .x = sum of x, .y = 2^-p
-    int i0 = lookup_dword<0>(t.w.x, a, mask, 0);
-    i0 = lookup_dword<1>(t.w.y, a, mask, i0);
-    int i1 = lookup_dword<2>(t.w.z, a, mask, 0);
-    i1 = lookup_dword<3>(t.w.w, a, mask, i1);
+    lookup_issue<0>(t.w.x, a0, mask, v0);
+    lookup_issue<1>(t.w.y, a1, mask, v1);
+    __builtin_amdgcn_sched_barrier(0);
+    int i0 = lookup_sum(v0, 0);
+    lookup_issue<2>(t.w.z, a0, mask, v0);
+    __builtin_amdgcn_sched_barrier(0);
+    i0 = lookup_sum(v1, i0);
+    lookup_issue<3>(t.w.w, a1, mask, v1);
+    __builtin_amdgcn_sched_barrier(0);
+    int i1 = lookup_sum(v0, 0);
+    i1 = lookup_sum(v1, i1);
     const uint32_t sc = G64 ? t.sc : (odd ? (t.sc >> 16) * 0x10001u : (t.sc & 0xffffu) * 0x10001u);
     acc = fmaf((float)i0 * h0.y, h2f_lo(sc), acc);
     acc = fmaf((float)i1 * h1.y, h2f_hi(sc), acc);
@@ -268,6 +309,16 @@ __device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scr
     return rsqrtf(scratch[64] / (float)K + a.eps);
 }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load of the wave (its fence covers all address spaces), which here would
+// be the weight loads that are meant to stay in flight across the barrier.
+__device__ __forceinline__ void lds_barrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 
 // One workgroup = one column block x one K slice.  Its (unit, plane) sub-tasks are dealt to
@@ -276,8 +327,7 @@ constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 // without waiting for the other waves -- the only workgroup barrier is the one in front of
 // the final cross-wave sum.
 //
-// `vblock` = column block * ksplit + slice (the block index of a launch that runs one
-// GEMV); `red_sel` picks one of two cross-wave buffers so that a caller that runs tiles
+// `red_sel` picks one of two cross-wave buffers so that a caller that runs tiles
 // back to back needs no barrier between them: waves other than wave 0 may start the next
 // tile while wave 0 still sums and stores this one.
 //
@@ -287,13 +337,12 @@ constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 // stops between blocks.  Needs runs of at most NSLOT sub-tasks per wave.
 // PLAIN: no prologue and no residual (their fields of `a` are not read).
 template <int BITS, bool G64, int NSLOT, bool MULTI, bool PLAIN>
-__device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb_run, unsigned char *smem, int &red_sel)
+__device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, int ncb_run, unsigned char *smem, int &red_sel)
 {
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int cb = vblock / a.ksplit, slice = vblock - cb * a.ksplit;
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
     const int nst = nU * BITS;                                             // sub-tasks of this workgroup
     const int s_begin = min(wave * a.spw, nst), s_end = min(s_begin + a.spw, nst);
@@ -307,6 +356,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb
     float *rstd_scratch = red0 + 2 * nw * HLQ_CB;                          // [RSTD_SCRATCH]
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
+    HLQ_STAMP_DECL;
     HLQ_STAMP(0);
     // Activations first, then the weight stream.  Every load below is unconditional (a wave
     // whose run is shorter than NSLOT re-reads its last sub-task), so the number of loads
@@ -325,9 +375,9 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb
     const uint32_t mask = 0x3Cu;
     float acc = 0.f;
     Sub slot[NSLOT];
+    const CbBase here = cb_base<BITS>(a, cb, u0);
     {   // the first sub-task's loads start the weight stream ...
-        const int st = min(s_begin, s_last);
-        load_sub<BITS, G64>(slot[0], a, cb, u0 + st / BITS, st % BITS, lane);
+        load_sub<BITS, G64>(slot[0], here, u0, min(s_begin, s_last), lane);
     }
     asm volatile("" ::: "memory");
 
@@ -340,8 +390,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb
     // ... and the rest of the run's loads follow.
 #pragma unroll
     for (int d = 1; d < NSLOT; d++) {
-        const int st = min(s_begin + d, s_last);
-        load_sub<BITS, G64>(slot[d], a, cb, u0 + st / BITS, st % BITS, lane);
+        load_sub<BITS, G64>(slot[d], here, u0, min(s_begin + d, s_last), lane);
     }
     for (int ci = lane + 64; ci < nchunks; ci += 64) {      // runs of more than two units (not the common case)
         load_chunk(a, prologue, K, k0 + (size_t)ci * 4, raw, raw2);
@@ -362,7 +411,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb
         float total = accf;
         if (nw > 1) {
             red[wave * HLQ_CB + lane] = accf;
-            __syncthreads();
+            lds_barrier();
             if (wave == 0) {
                 total = 0.f;
                 for (int w = 0; w < nw; w++) total += red[w * HLQ_CB + lane];
@@ -418,7 +467,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb
 
     if (MULTI) {
         for (int c = 0; c < ncb_run; c++) {
-            const int cbn = min(cb + c + 1, cb + ncb_run - 1);        // past the run: a reload nobody reads
+            const CbBase next = cb_base<BITS>(a, min(cb + c + 1, cb + ncb_run - 1), u0);   // past the run: a reload nobody reads
             float accc = 0.f;
             HLQ_STAMP(2);
 #pragma unroll
@@ -428,13 +477,13 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb
                     const int u = st / BITS;
                     accc = process_sub<G64>(slot[d], u - ub, st % BITS, (u0 + u) & 1, lut_base, xs_inv, mask, accc);
                 }
-                const int sn = min(st, s_last);
-                load_sub<BITS, G64>(slot[d], a, cbn, u0 + sn / BITS, sn % BITS, lane);
+                load_sub<BITS, G64>(slot[d], next, u0, min(st, s_last), lane);
             }
             HLQ_STAMP(3);
             finish(cb + c, accc);
             HLQ_STAMP(6);
         }
+        HLQ_STAMP_FLUSH;
         return;
     }
 
@@ -449,13 +498,13 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int vblock, int ncb
                 acc = process_sub<G64>(slot[d], u - ub, st % BITS, (u0 + u) & 1, lut_base, xs_inv, mask, acc);
             }
             if (base + NSLOT < s_end) {                     // wave-uniform: only runs longer than NSLOT refill
-                const int sn = min(st + NSLOT, s_last);
-                load_sub<BITS, G64>(slot[d], a, cb, u0 + sn / BITS, sn % BITS, lane);
+                load_sub<BITS, G64>(slot[d], here, u0, min(st + NSLOT, s_last), lane);
             }
         }
     }
     HLQ_STAMP(3);
     finish(cb, acc);
+    HLQ_STAMP_FLUSH;
 }
 
 template <int BITS, bool G64, int NSLOT>
@@ -463,7 +512,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 {
     extern __shared__ __align__(256) unsigned char smem[];
     int sel = 0;
-    gemv_tile<BITS, G64, NSLOT, false, false>(a, blockIdx.x, 1, smem, sel);
+    gemv_tile<BITS, G64, NSLOT, false, false>(a, blockIdx.y, blockIdx.x, 1, smem, sel);      // grid = (slices, column blocks)
 }
 
 // One GEMV with more column blocks than the chip has CUs: every workgroup takes a run of
@@ -473,9 +522,9 @@ template <int BITS, bool G64, int NSLOT>
 __global__ __launch_bounds__(1024) void hlq_gemv_run_kernel(const GemvArgs a, int run)
 {
     extern __shared__ __align__(256) unsigned char smem[];
-    const int cb0 = (blockIdx.x / a.ksplit) * run, slice = blockIdx.x % a.ksplit;
+    const int cb0 = blockIdx.y * run;               // grid = (slices, runs of column blocks)
     int sel = 0;
-    gemv_tile<BITS, G64, NSLOT, true, false>(a, cb0 * a.ksplit + slice, min(run, a.ncb - cb0), smem, sel);
+    gemv_tile<BITS, G64, NSLOT, true, false>(a, cb0, blockIdx.x, min(run, a.ncb - cb0), smem, sel);
 }
 
 // Many independent GEMVs in one launch: the tiles of all of them form one list that the
@@ -486,7 +535,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_run_kernel(const GemvArgs a, in
 // per GEMV, and with two workgroups per CU the sum-and-store of one tile hides under the
 // lookups of another.
 struct GroupItem {
-    int problem, vblock;     // vblock = first column block * ksplit + slice
+    int problem, cb, slice;  // first column block and K slice
     int ncb_run;             // consecutive column blocks of that slice
 };
 
@@ -499,7 +548,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *__
     for (int i = blockIdx.x; i < n_items; i += gridDim.x) {
         const GroupItem it = items[i];
         const GemvArgs a = problems[it.problem];
-        gemv_tile<BITS, G64, NSLOT, true, true>(a, it.vblock, it.ncb_run, smem, sel);
+        gemv_tile<BITS, G64, NSLOT, true, true>(a, it.cb, it.slice, it.ncb_run, smem, sel);
     }
 }
 
@@ -557,10 +606,10 @@ int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
         static bool big_lds_run_done[64] = {};
         if (!allow_big_lds((const void *)kern_run, lds, MAX_LDS, big_lds_run_done)) return ELUTQ_ERR_HIP;
         const int groups = (a.ncb + run - 1) / run;
-        hipLaunchKernelGGL(kern_run, dim3(groups * a.ksplit), dim3(waves * 64), lds, stream, a, run);
+        hipLaunchKernelGGL(kern_run, dim3(a.ksplit, groups), dim3(waves * 64), lds, stream, a, run);
         return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
     }
-    hipLaunchKernelGGL(kern, dim3(a.ncb * a.ksplit), dim3(waves * 64), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3(a.ksplit, a.ncb), dim3(waves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
 
@@ -649,6 +698,13 @@ void choose_shape(const HlqGeo &g, int &ksplit, int &waves)
 {
     if (ksplit <= 0) {
         ksplit = g.ncb >= 64 ? 1 : NUM_CU / g.ncb;
+        // runs longer than a wave's slots (3 and 4 planes at K = 4096): slice while that still leaves
+        // at most one workgroup per CU
+        const int by_slots = (g.U * g.bits + 16 * DEPTH - 1) / (16 * DEPTH);
+        if (by_slots > 1 && g.ncb < 128) {
+            const int fill = NUM_CU / g.ncb > by_slots ? NUM_CU / g.ncb : by_slots;
+            if (ksplit < fill) ksplit = fill;
+        }
         if (ksplit > 4) ksplit = 4;
         const int by_len = (g.U + 31) / 32;
         if (ksplit < by_len) ksplit = by_len;
@@ -851,7 +907,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
         for (int sl = 0; sl < sh.ksplit; sl++)
             for (int cb0 = 0; cb0 < sh.g.ncb; cb0 += cbs_per_item) {
                 const int len = sh.g.ncb - cb0 < cbs_per_item ? sh.g.ncb - cb0 : cbs_per_item;
-                items.push_back(GroupItem{i, cb0 * sh.ksplit + sl, len});
+                items.push_back(GroupItem{i, cb0, sl, len});
             }
     }
     GemvGroupPlan *pl = new GemvGroupPlan();
