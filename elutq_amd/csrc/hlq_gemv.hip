@@ -25,6 +25,7 @@
 //  * slices are combined through a workspace by the last workgroup to arrive (fixed
 //    summation order, so results are deterministic).
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <vector>
 #include <stdint.h>
 
@@ -94,31 +95,35 @@ __device__ __forceinline__ int lds_ld(uint32_t addr, int imm)
 __device__ __forceinline__ float h2f_lo(uint32_t v) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(v & 0xffffu)); }
 __device__ __forceinline__ float h2f_hi(uint32_t v) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(v >> 16)); }
 
-// a.byte0 = mask & src.byte<SEL>; bytes 1..3 of `a` are kept (they hold the table base).
-#define HLQ_SDWA_AND(a, mask, src, SEL)                                                        \
-    asm("v_and_b32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD "  \
+// dst = base | src.byte<SEL>: the table address of one lookup.  `src` is a plane dword (or its
+// rotation by 4) masked to bits 2..5 of every byte, i.e. 4 * nibble; `base` (wave-uniform, a
+// multiple of 256) is the LDS address of the unit's tables.
+#define HLQ_SDWA_OR(dst, base, src, SEL)                                                       \
+    asm("v_or_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD "         \
         "src1_sel:BYTE_" #SEL                                                                  \
-        : "+v"(a)                                                                              \
-        : "v"(mask), "v"(src))
+        : "=v"(dst)                                                                            \
+        : "s"(base), "v"(src))
 
 // Eight lookups for one plane dword (32 k): chunks 8*D .. 8*D+7 of the unit.  Issue and sum are
 // separate so that the lookups of the next dword are on their way to LDS before the wave waits
 // for the results of this one (LDS returns a wave's reads in order).
 template <int D>
-__device__ __forceinline__ void lookup_issue(uint32_t w, uint32_t (&a)[8], uint32_t mask, int (&v)[8])
+__device__ __forceinline__ void lookup_issue(uint32_t w, uint32_t base, int (&v)[8])
 {
-    const uint32_t r = __builtin_amdgcn_alignbit(w, w, 4);
-    HLQ_SDWA_AND(a[0], mask, w, 0);
-    HLQ_SDWA_AND(a[1], mask, r, 0);
-    HLQ_SDWA_AND(a[2], mask, w, 1);
-    HLQ_SDWA_AND(a[3], mask, r, 1);
-    HLQ_SDWA_AND(a[4], mask, w, 2);
-    HLQ_SDWA_AND(a[5], mask, r, 2);
-    HLQ_SDWA_AND(a[6], mask, w, 3);
-    HLQ_SDWA_AND(a[7], mask, r, 3);
-    constexpr int base = D * 8 * TBL_BYTES;
+    const uint32_t wm = w & 0x3C3C3C3Cu;
+    const uint32_t rm = __builtin_amdgcn_alignbit(w, w, 4) & 0x3C3C3C3Cu;
+    uint32_t a[8];
+    HLQ_SDWA_OR(a[0], base, wm, 0);
+    HLQ_SDWA_OR(a[1], base, rm, 0);
+    HLQ_SDWA_OR(a[2], base, wm, 1);
+    HLQ_SDWA_OR(a[3], base, rm, 1);
+    HLQ_SDWA_OR(a[4], base, wm, 2);
+    HLQ_SDWA_OR(a[5], base, rm, 2);
+    HLQ_SDWA_OR(a[6], base, wm, 3);
+    HLQ_SDWA_OR(a[7], base, rm, 3);
+    constexpr int off = D * 8 * TBL_BYTES;
 #pragma unroll
-    for (int j = 0; j < 8; j++) v[j] = lds_ld(a[j], base + j * TBL_BYTES);
+    for (int j = 0; j < 8; j++) v[j] = lds_ld(a[j], off + j * TBL_BYTES);
 }
 
 __device__ __forceinline__ int lookup_sum(const int (&v)[8], int acc)
@@ -162,7 +167,7 @@ __device__ __forceinline__ CbBase cb_base(const GemvArgs &a, int cb, int u0)
 
 // st = sub-task index inside the slice (unit u0 + st / BITS, plane st % BITS); planes of a
 // slice are contiguous in st.
-template <int BITS, bool G64>
+template <int BITS, bool G64, bool SC = true, bool ZZ = true>
 __device__ __forceinline__ void load_sub(Sub &t, const CbBase &p, int u0, int st, int lane)
 {
     const uint32_t u = (uint32_t)(u0 + st / BITS), b = (uint32_t)(st % BITS);
@@ -170,41 +175,58 @@ __device__ __forceinline__ void load_sub(Sub &t, const CbBase &p, int u0, int st
     const u32x4 v = __builtin_nontemporal_load(
         (const HLQ_GLOBAL u32x4 *)(p.planes + ((uint32_t)st * (uint32_t)(HLQ_CB * 16) + (uint32_t)lane * 16u)));
     t.w = make_uint4(v.x, v.y, v.z, v.w);
-    t.sc = *(const HLQ_GLOBAL uint32_t *)(p.scales + ((row * BITS + b) * (uint32_t)(HLQ_CB * 4) + (uint32_t)lane * 4u));
-    // used by plane 0 only; loaded always so that every sub-task is 3 loads
-    t.zz = *(const HLQ_GLOBAL uint32_t *)(p.zeros + (row * (uint32_t)(HLQ_CB * 4) + (uint32_t)lane * 4u));
+    if (SC) t.sc = *(const HLQ_GLOBAL uint32_t *)(p.scales + ((row * BITS + b) * (uint32_t)(HLQ_CB * 4) + (uint32_t)lane * 4u));
+    if (ZZ) t.zz = *(const HLQ_GLOBAL uint32_t *)(p.zeros + (row * (uint32_t)(HLQ_CB * 4) + (uint32_t)lane * 4u));
+}
+
+// Sub-tasks that share scale / zero dwords form a meta group: the planes of one unit at
+// G = 64, of a unit pair at G = 128.  When every wave's run starts on a group boundary and the
+// slots hold whole groups (`PAIRED`), position d of a pass is a compile-time (unit, plane) of
+// its group: only the first unit's positions load the scale dword of their plane, only position 0
+// the zero dword -- 7 loads instead of 12 for the four sub-tasks of a w2g128 pair -- and the
+// later positions reuse the values.  Otherwise every sub-task loads both (3 loads each, so
+// that the load count behind any point is still a compile-time constant).
+template <int BITS, bool G64>
+struct MetaGroup {
+    static constexpr int SIZE = G64 ? BITS : 2 * BITS;           // sub-tasks per group
+    static constexpr bool fits(int nslot) { return nslot % SIZE == 0; }
+    static constexpr bool sc_at(int d) { return d % SIZE < BITS; }
+    static constexpr bool zz_at(int d) { return d % SIZE == 0; }
+};
+
+template <int BITS, bool G64, bool PAIRED, int D>
+__device__ __forceinline__ void load_slot(Sub &t, const CbBase &p, int u0, int st, int lane)
+{
+    using MG = MetaGroup<BITS, G64>;
+    load_sub<BITS, G64, !PAIRED || MG::sc_at(D), !PAIRED || MG::zz_at(D)>(t, p, u0, st, lane);
 }
 
 // The two 64-k halves of a unit have their own table scale (2^-p) and activation sum; at
 // G = 64 they are also two quantization groups (lo / hi half of the meta dwords), at G = 128
 // one group (the half of the meta dwords selected by the unit's parity).
 template <bool G64>
-__device__ __forceinline__ float process_sub(const Sub &t, int lu, int b, int odd, uint32_t lut_base,
-                                             const float2 *xs_inv, uint32_t mask, float acc)
+__device__ __forceinline__ float process_sub(const uint4 &w, uint32_t sc_raw, uint32_t zz_raw, int lu, int b, int odd,
+                                             uint32_t lut_base, const float2 *xs_inv, float acc)
 {
-    // two sets of address registers (table base in the upper bytes) alternate between the dwords
-    uint32_t a0[8], a1[8];
     int v0[8], v1[8];
-    const uint32_t ub = lut_base + (uint32_t)lu * UNIT_LUT_BYTES;
-#pragma unroll
-    for (int j = 0; j < 8; j++) a0[j] = a1[j] = ub;
+    const uint32_t ub = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lut_base + (uint32_t)lu * UNIT_LUT_BYTES));
     const float2 h0 = xs_inv[2 * lu], h1 = xs_inv[2 * lu + 1];      // .x = sum of x, .y = 2^-p
-    lookup_issue<0>(t.w.x, a0, mask, v0);
-    lookup_issue<1>(t.w.y, a1, mask, v1);
+    lookup_issue<0>(w.x, ub, v0);
+    lookup_issue<1>(w.y, ub, v1);
     __builtin_amdgcn_sched_barrier(0);
     int i0 = lookup_sum(v0, 0);
-    lookup_issue<2>(t.w.z, a0, mask, v0);
+    lookup_issue<2>(w.z, ub, v0);
     __builtin_amdgcn_sched_barrier(0);
     i0 = lookup_sum(v1, i0);
-    lookup_issue<3>(t.w.w, a1, mask, v1);
+    lookup_issue<3>(w.w, ub, v1);
     __builtin_amdgcn_sched_barrier(0);
     int i1 = lookup_sum(v0, 0);
     i1 = lookup_sum(v1, i1);
-    const uint32_t sc = G64 ? t.sc : (odd ? (t.sc >> 16) * 0x10001u : (t.sc & 0xffffu) * 0x10001u);
+    const uint32_t sc = G64 ? sc_raw : (odd ? (sc_raw >> 16) * 0x10001u : (sc_raw & 0xffffu) * 0x10001u);
     acc = fmaf((float)i0 * h0.y, h2f_lo(sc), acc);
     acc = fmaf((float)i1 * h1.y, h2f_hi(sc), acc);
     if (b == 0) {
-        const uint32_t zz = G64 ? t.zz : (odd ? (t.zz >> 16) * 0x10001u : (t.zz & 0xffffu) * 0x10001u);
+        const uint32_t zz = G64 ? zz_raw : (odd ? (zz_raw >> 16) * 0x10001u : (zz_raw & 0xffffu) * 0x10001u);
         acc = fmaf(h2f_lo(zz), h0.x, acc);
         acc = fmaf(h2f_hi(zz), h1.x, acc);
     }
@@ -319,6 +341,16 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
 constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 
 // One workgroup = one column block x one K slice.  Its (unit, plane) sub-tasks are dealt to
@@ -336,9 +368,14 @@ constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
 // consumed is refilled with the same sub-task of the next block, so the weight stream never
 // stops between blocks.  Needs runs of at most NSLOT sub-tasks per wave.
 // PLAIN: no prologue and no residual (their fields of `a` are not read).
-template <int BITS, bool G64, int NSLOT, bool MULTI, bool PLAIN>
+template <int BITS, bool G64, int NSLOT, bool MULTI, bool PLAIN, bool PAIRED>
 __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, int ncb_run, unsigned char *smem, int &red_sel)
 {
+    HLQ_STAMP_DECL;
+#ifdef HLQ_TIMING_ENTRY
+    HLQ_STAMP(7);
+    asm volatile("" ::: "memory");
+#endif
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
@@ -356,7 +393,6 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     float *rstd_scratch = red0 + 2 * nw * HLQ_CB;                          // [RSTD_SCRATCH]
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
-    HLQ_STAMP_DECL;
     HLQ_STAMP(0);
     // Activations first, then the weight stream.  Every load below is unconditional (a wave
     // whose run is shorter than NSLOT re-reads its last sub-task), so the number of loads
@@ -372,12 +408,11 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     load_chunk(a, prologue, K, nchunks ? k0 + (size_t)min(lane, nchunks - 1) * 4 : 0, raw, raw2);
     asm volatile("" ::: "memory");      // keep both activation loads ahead of the weight loads
 
-    const uint32_t mask = 0x3Cu;
     float acc = 0.f;
     Sub slot[NSLOT];
     const CbBase here = cb_base<BITS>(a, cb, u0);
     {   // the first sub-task's loads start the weight stream ...
-        load_sub<BITS, G64>(slot[0], here, u0, min(s_begin, s_last), lane);
+        load_slot<BITS, G64, PAIRED, 0>(slot[0], here, u0, min(s_begin, s_last), lane);
     }
     asm volatile("" ::: "memory");
 
@@ -388,10 +423,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     asm volatile("" ::: "memory");
 
     // ... and the rest of the run's loads follow.
-#pragma unroll
-    for (int d = 1; d < NSLOT; d++) {
-        load_sub<BITS, G64>(slot[d], here, u0, min(s_begin + d, s_last), lane);
-    }
+    static_for<1, NSLOT>([&](auto dc) __attribute__((always_inline)) {
+        constexpr int d = decltype(dc)::value;
+        load_slot<BITS, G64, PAIRED, d>(slot[d], here, u0, min(s_begin + d, s_last), lane);
+    });
     for (int ci = lane + 64; ci < nchunks; ci += 64) {      // runs of more than two units (not the common case)
         load_chunk(a, prologue, K, k0 + (size_t)ci * 4, raw, raw2);
         build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0);
@@ -465,20 +500,34 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         }
     };
 
+    // Position d of a pass over the slots: the sub-task's plane and unit parity are compile-time
+    // in PAIRED mode, where the scale / zero dwords are taken over from the positions that loaded them.
+    using MG = MetaGroup<BITS, G64>;
+    uint32_t sc_keep[BITS] = {}, zz_keep = 0;
+    auto run_slot = [&](auto dc, int st, float accv) __attribute__((always_inline)) -> float {
+        constexpr int d = decltype(dc)::value;
+        const int u = st / BITS;
+        if constexpr (PAIRED) {
+            constexpr int pos = d % MG::SIZE, b = pos % BITS, odd = pos / BITS;     // odd only matters at G = 128
+            if (MG::sc_at(d)) sc_keep[b] = slot[d].sc;
+            if (MG::zz_at(d)) zz_keep = slot[d].zz;
+            return process_sub<G64>(slot[d].w, sc_keep[b], zz_keep, u - ub, b, odd, lut_base, xs_inv, accv);
+        } else {
+            return process_sub<G64>(slot[d].w, slot[d].sc, slot[d].zz, u - ub, st % BITS, (u0 + u) & 1, lut_base, xs_inv, accv);
+        }
+    };
+
     if (MULTI) {
         for (int c = 0; c < ncb_run; c++) {
             const CbBase next = cb_base<BITS>(a, min(cb + c + 1, cb + ncb_run - 1), u0);   // past the run: a reload nobody reads
             float accc = 0.f;
             HLQ_STAMP(2);
-#pragma unroll
-            for (int d = 0; d < NSLOT; d++) {
+            static_for<0, NSLOT>([&](auto dc) __attribute__((always_inline)) {
+                constexpr int d = decltype(dc)::value;
                 const int st = s_begin + d;
-                if (st < s_end) {
-                    const int u = st / BITS;
-                    accc = process_sub<G64>(slot[d], u - ub, st % BITS, (u0 + u) & 1, lut_base, xs_inv, mask, accc);
-                }
-                load_sub<BITS, G64>(slot[d], next, u0, min(st, s_last), lane);
-            }
+                if (st < s_end) accc = run_slot(dc, st, accc);
+                load_slot<BITS, G64, PAIRED, d>(slot[d], next, u0, min(st, s_last), lane);
+            });
             HLQ_STAMP(3);
             finish(cb + c, accc);
             HLQ_STAMP(6);
@@ -490,41 +539,37 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     // Slot d holds sub-task base + d; it is refilled with sub-task base + d + NSLOT as soon as
     // it has been consumed (past the end of the run: a reload nobody reads).
     for (int base = s_begin; base < s_end; base += NSLOT) {
-#pragma unroll
-        for (int d = 0; d < NSLOT; d++) {
+        static_for<0, NSLOT>([&](auto dc) __attribute__((always_inline)) {
+            constexpr int d = decltype(dc)::value;
             const int st = base + d;
-            if (st < s_end) {
-                const int u = st / BITS;
-                acc = process_sub<G64>(slot[d], u - ub, st % BITS, (u0 + u) & 1, lut_base, xs_inv, mask, acc);
-            }
-            if (base + NSLOT < s_end) {                     // wave-uniform: only runs longer than NSLOT refill
-                load_sub<BITS, G64>(slot[d], here, u0, min(st + NSLOT, s_last), lane);
-            }
-        }
+            if (st < s_end) acc = run_slot(dc, st, acc);
+            if (base + NSLOT < s_end)                      // wave-uniform: only runs longer than NSLOT refill
+                load_slot<BITS, G64, PAIRED, d>(slot[d], here, u0, min(st + NSLOT, s_last), lane);
+        });
     }
     HLQ_STAMP(3);
     finish(cb, acc);
     HLQ_STAMP_FLUSH;
 }
 
-template <int BITS, bool G64, int NSLOT>
+template <int BITS, bool G64, int NSLOT, bool PAIRED>
 __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 {
     extern __shared__ __align__(256) unsigned char smem[];
     int sel = 0;
-    gemv_tile<BITS, G64, NSLOT, false, false>(a, blockIdx.y, blockIdx.x, 1, smem, sel);      // grid = (slices, column blocks)
+    gemv_tile<BITS, G64, NSLOT, false, false, PAIRED>(a, blockIdx.y, blockIdx.x, 1, smem, sel);      // grid = (slices, column blocks)
 }
 
 // One GEMV with more column blocks than the chip has CUs: every workgroup takes a run of
 // consecutive column blocks (tables built once, weights prefetched across the blocks) instead
 // of the launch holding two workgroups per CU that each build the same tables.
-template <int BITS, bool G64, int NSLOT>
+template <int BITS, bool G64, int NSLOT, bool PAIRED>
 __global__ __launch_bounds__(1024) void hlq_gemv_run_kernel(const GemvArgs a, int run)
 {
     extern __shared__ __align__(256) unsigned char smem[];
     const int cb0 = blockIdx.y * run;               // grid = (slices, runs of column blocks)
     int sel = 0;
-    gemv_tile<BITS, G64, NSLOT, true, false>(a, cb0, blockIdx.x, min(run, a.ncb - cb0), smem, sel);
+    gemv_tile<BITS, G64, NSLOT, true, false, PAIRED>(a, cb0, blockIdx.x, min(run, a.ncb - cb0), smem, sel);
 }
 
 // Many independent GEMVs in one launch: the tiles of all of them form one list that the
@@ -539,7 +584,7 @@ struct GroupItem {
     int ncb_run;             // consecutive column blocks of that slice
 };
 
-template <int BITS, bool G64, int NSLOT>
+template <int BITS, bool G64, int NSLOT, bool PAIRED>
 __global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *__restrict__ problems,
                                                               const GroupItem *__restrict__ items, int n_items)
 {
@@ -548,7 +593,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *__
     for (int i = blockIdx.x; i < n_items; i += gridDim.x) {
         const GroupItem it = items[i];
         const GemvArgs a = problems[it.problem];
-        gemv_tile<BITS, G64, NSLOT, true, true>(a, it.cb, it.slice, it.ncb_run, smem, sel);
+        gemv_tile<BITS, G64, NSLOT, true, true, PAIRED>(a, it.cb, it.slice, it.ncb_run, smem, sel);
     }
 }
 
@@ -593,16 +638,25 @@ inline bool allow_big_lds(const void *kern, size_t lds, int limit, bool (&done)[
 }
 
 
+// Every wave's run starts on a meta-group boundary, the slots hold whole groups and (at G = 128)
+// every slice starts on an even unit: the conditions of the PAIRED load pattern.
 template <int BITS, bool G64, int NSLOT>
-int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
+bool paired_ok(int spw, int ups, int ksplit)
 {
-    auto kern = hlq_gemv_kernel<BITS, G64, NSLOT>;
+    using MG = MetaGroup<BITS, G64>;
+    return MG::fits(NSLOT) && spw % MG::SIZE == 0 && (G64 || ksplit == 1 || ups % 2 == 0);
+}
+
+template <int BITS, bool G64, int NSLOT, bool PAIRED>
+int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
+{
+    auto kern = hlq_gemv_kernel<BITS, G64, NSLOT, PAIRED>;
     static bool big_lds_done[64] = {};        // per template instance
     if (!allow_big_lds((const void *)kern, lds, MAX_LDS, big_lds_done)) return ELUTQ_ERR_HIP;
     // more tiles than CUs and runs that fit the slots: runs of column blocks, one workgroup per CU
     const int run = (a.ncb * a.ksplit + NUM_CU_RUN - 1) / NUM_CU_RUN;
     if (run > 1 && a.spw <= NSLOT && waves == 16) {
-        auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT>;
+        auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT, PAIRED>;
         static bool big_lds_run_done[64] = {};
         if (!allow_big_lds((const void *)kern_run, lds, MAX_LDS, big_lds_run_done)) return ELUTQ_ERR_HIP;
         const int groups = (a.ncb + run - 1) / run;
@@ -611,6 +665,15 @@ int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
     }
     hipLaunchKernelGGL(kern, dim3(a.ksplit, a.ncb), dim3(waves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
+}
+
+template <int BITS, bool G64, int NSLOT>
+int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
+{
+    if constexpr (MetaGroup<BITS, G64>::fits(NSLOT)) {
+        if (paired_ok<BITS, G64, NSLOT>(a.spw, a.ups, a.ksplit)) return launch_gemv_p<BITS, G64, NSLOT, true>(a, waves, lds, stream);
+    }
+    return launch_gemv_p<BITS, G64, NSLOT, false>(a, waves, lds, stream);
 }
 
 // NSLOT = sub-tasks a wave keeps in flight: its whole run when that is at most DEPTH.
@@ -638,11 +701,11 @@ int dispatch_gemv(const GemvArgs &a, int bits, int group, int waves, size_t lds,
 }
 
 // grid < 0: no launch, returns the number of workgroups of this shape a CU holds at once
-template <int BITS, bool G64, int NSLOT>
-int launch_group_n(const GemvArgs *d_problems, const GroupItem *d_items, int n_items, int grid, int waves, size_t lds,
+template <int BITS, bool G64, int NSLOT, bool PAIRED>
+int launch_group_p(const GemvArgs *d_problems, const GroupItem *d_items, int n_items, int grid, int waves, size_t lds,
                    hipStream_t stream)
 {
-    auto kern = hlq_gemv_group_kernel<BITS, G64, NSLOT>;
+    auto kern = hlq_gemv_group_kernel<BITS, G64, NSLOT, PAIRED>;
     static bool big_lds_done[64] = {};
     if (!allow_big_lds((const void *)kern, lds, MAX_LDS, big_lds_done)) return ELUTQ_ERR_HIP;
     if (grid < 0) {
@@ -655,27 +718,45 @@ int launch_group_n(const GemvArgs *d_problems, const GroupItem *d_items, int n_i
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
 
+// paired: every problem of the group meets paired_ok for this slot count
+template <int BITS, bool G64, int NSLOT>
+int launch_group_n(bool paired, const GemvArgs *p, const GroupItem *it, int n, int grid, int waves, size_t lds, hipStream_t st)
+{
+    if constexpr (MetaGroup<BITS, G64>::fits(NSLOT)) {
+        if (paired) return launch_group_p<BITS, G64, NSLOT, true>(p, it, n, grid, waves, lds, st);
+    }
+    return launch_group_p<BITS, G64, NSLOT, false>(p, it, n, grid, waves, lds, st);
+}
+
 template <int BITS, bool G64>
-int launch_group(int nslot, const GemvArgs *p, const GroupItem *it, int n, int grid, int waves, size_t lds, hipStream_t st)
+int launch_group(int nslot, bool paired, const GemvArgs *p, const GroupItem *it, int n, int grid, int waves, size_t lds,
+                 hipStream_t st)
 {
     switch (nslot) {
-    case 1: return launch_group_n<BITS, G64, 1>(p, it, n, grid, waves, lds, st);
-    case 2: return launch_group_n<BITS, G64, 2>(p, it, n, grid, waves, lds, st);
-    case 3: return launch_group_n<BITS, G64, 3>(p, it, n, grid, waves, lds, st);
-    default: return launch_group_n<BITS, G64, 4>(p, it, n, grid, waves, lds, st);
+    case 1: return launch_group_n<BITS, G64, 1>(paired, p, it, n, grid, waves, lds, st);
+    case 2: return launch_group_n<BITS, G64, 2>(paired, p, it, n, grid, waves, lds, st);
+    case 3: return launch_group_n<BITS, G64, 3>(paired, p, it, n, grid, waves, lds, st);
+    default: return launch_group_n<BITS, G64, 4>(paired, p, it, n, grid, waves, lds, st);
     }
 }
 
-int dispatch_group(int bits, bool g64, int nslot, const GemvArgs *p, const GroupItem *it, int n, int grid, int waves,
-                   size_t lds, hipStream_t st)
+int dispatch_group(int bits, bool g64, int nslot, bool paired, const GemvArgs *p, const GroupItem *it, int n, int grid,
+                   int waves, size_t lds, hipStream_t st)
 {
     switch (bits) {
-    case 1: return g64 ? launch_group<1, true>(nslot, p, it, n, grid, waves, lds, st) : launch_group<1, false>(nslot, p, it, n, grid, waves, lds, st);
-    case 2: return g64 ? launch_group<2, true>(nslot, p, it, n, grid, waves, lds, st) : launch_group<2, false>(nslot, p, it, n, grid, waves, lds, st);
-    case 3: return g64 ? launch_group<3, true>(nslot, p, it, n, grid, waves, lds, st) : launch_group<3, false>(nslot, p, it, n, grid, waves, lds, st);
-    case 4: return g64 ? launch_group<4, true>(nslot, p, it, n, grid, waves, lds, st) : launch_group<4, false>(nslot, p, it, n, grid, waves, lds, st);
+    case 1: return g64 ? launch_group<1, true>(nslot, paired, p, it, n, grid, waves, lds, st) : launch_group<1, false>(nslot, paired, p, it, n, grid, waves, lds, st);
+    case 2: return g64 ? launch_group<2, true>(nslot, paired, p, it, n, grid, waves, lds, st) : launch_group<2, false>(nslot, paired, p, it, n, grid, waves, lds, st);
+    case 3: return g64 ? launch_group<3, true>(nslot, paired, p, it, n, grid, waves, lds, st) : launch_group<3, false>(nslot, paired, p, it, n, grid, waves, lds, st);
+    case 4: return g64 ? launch_group<4, true>(nslot, paired, p, it, n, grid, waves, lds, st) : launch_group<4, false>(nslot, paired, p, it, n, grid, waves, lds, st);
     }
     return ELUTQ_ERR_BITS;
+}
+
+// paired_ok for run-time plane count / group size / slot count
+bool paired_ok_rt(int bits, bool g64, int nslot, int spw, int ups, int ksplit)
+{
+    const int size = g64 ? bits : 2 * bits;
+    return nslot % size == 0 && spw % size == 0 && (g64 || ksplit == 1 || ups % 2 == 0);
 }
 
 int check_shape(int K, int N, int bits, int group)
@@ -817,6 +898,7 @@ static int group_shape(const elutq_gemv_problem &p, int bits, int group, GroupSh
 
 struct GemvGroupPlan {
     int bits, group, nslot, n_items, grid;
+    bool paired;
     size_t lds;
     GemvArgs *d_problems;
     GroupItem *d_items;
@@ -912,8 +994,10 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
     }
     GemvGroupPlan *pl = new GemvGroupPlan();
     pl->bits = bits; pl->group = group; pl->nslot = nslot; pl->n_items = (int)items.size(); pl->lds = lds;
+    pl->paired = true;
+    for (auto &sh : shapes) pl->paired = pl->paired && paired_ok_rt(bits, group == 64, nslot, sh.wp.spw, sh.ups, sh.ksplit);
     // as many workgroups as the chip holds at once: each walks the list with that stride
-    int per_cu = dispatch_group(bits, group == 64, nslot, nullptr, nullptr, 0, -1, 16, lds, nullptr);
+    int per_cu = dispatch_group(bits, group == 64, nslot, pl->paired, nullptr, nullptr, 0, -1, 16, lds, nullptr);
     if (per_cu < 1) per_cu = 1;
     if (per_cu > 2) per_cu = 2;
     const int slots = NUM_CU * per_cu;
@@ -936,7 +1020,7 @@ int elutq_hlq_gemv_group_run(void *plan, void *stream)
 {
     if (!plan) return ELUTQ_ERR_NULL;
     const GemvGroupPlan *pl = (const GemvGroupPlan *)plan;
-    return dispatch_group(pl->bits, pl->group == 64, pl->nslot, pl->d_problems, pl->d_items, pl->n_items, pl->grid, 16,
+    return dispatch_group(pl->bits, pl->group == 64, pl->nslot, pl->paired, pl->d_problems, pl->d_items, pl->n_items, pl->grid, 16,
                           pl->lds, (hipStream_t)stream);
 }
 
