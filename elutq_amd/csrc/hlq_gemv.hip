@@ -269,9 +269,14 @@ __device__ __forceinline__ void chunk_values(int prologue, uint2 raw, uint2 raw2
 // Always two loads (without a prologue the second one re-reads the chunk): a fixed number
 // of loads lets the compiler wait for these with an exact vector-memory count while the
 // weight loads issued after them are still in flight.
+template <bool PLAIN>
 __device__ __forceinline__ void load_chunk(const GemvArgs &a, int prologue, int K, size_t k, uint2 &raw, uint2 &raw2)
 {
     raw = *(const HLQ_GLOBAL uint2 *)(a.x + k);
+    if (PLAIN) {            // no prologue at compile time: one load
+        raw2 = raw;
+        return;
+    }
     const HLQ_GLOBAL uint16_t *second = prologue == 1 ? a.norm_w + k : (prologue == 2 ? a.x + (size_t)K + k : a.x + k);
     raw2 = *(const HLQ_GLOBAL uint2 *)second;
 }
@@ -305,32 +310,6 @@ __device__ __forceinline__ void build_chunk(int prologue, uint2 raw, uint2 raw2,
     if (leader) *half = make_float2(s, inv);
 }
 
-// 1 / rms of the whole activation vector for the fused RMSNorm prologue: the workgroup sums
-// the squares together (one chunk per thread and pass), two barriers.  `scratch` is LDS of
-// RSTD_SCRATCH floats.  Every workgroup does this for itself (2K bytes from cache).
-constexpr int RSTD_SCRATCH = 80;
-__device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scratch, int tid, int nthreads)
-{
-    float ssq = 0.f;
-    for (int i = tid; i < K / 4; i += nthreads) {
-        const uint2 r = *(const HLQ_GLOBAL uint2 *)(a.x + (size_t)i * 4);
-        const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
-        ssq += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
-    }
-    HLQ_ROW_REDUCE(ssq, op_add);
-    if ((tid & 15) == 0) scratch[tid >> 4] = ssq;
-    __syncthreads();
-    if (tid < 64) {
-        float v = tid < (nthreads >> 4) ? scratch[tid] : 0.f;
-        HLQ_ROW_REDUCE(v, op_add);
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
-        if (tid == 0) scratch[64] = v;
-    }
-    __syncthreads();
-    return rsqrtf(scratch[64] / (float)K + a.eps);
-}
-
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
 // outstanding global load of the wave (its fence covers all address spaces), which here would
 // be the weight loads that are meant to stay in flight across the barrier.
@@ -339,6 +318,40 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// 1 / rms of the whole activation vector for the fused RMSNorm prologue: the workgroup sums
+// the squares together (one chunk per thread and pass), two barriers.  `scratch` is LDS of
+// RSTD_SCRATCH floats.  Every workgroup does this for itself (2K bytes from cache).
+constexpr int RSTD_SCRATCH = 80;
+
+// The chunk of x this thread squares first; issued ahead of the other loads of the tile so that
+// the reduction below overlaps with them.
+__device__ __forceinline__ uint2 rstd_first_load(const GemvArgs &a, int K, int tid)
+{
+    return *(const HLQ_GLOBAL uint2 *)(a.x + (size_t)min(tid, K / 4 - 1) * 4);
+}
+
+__device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scratch, int tid, int nthreads, uint2 first)
+{
+    auto sq4 = [](uint2 r) __attribute__((always_inline)) {
+        const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
+        return (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
+    };
+    float ssq = tid < K / 4 ? sq4(first) : 0.f;
+    for (int i = tid + nthreads; i < K / 4; i += nthreads) ssq += sq4(*(const HLQ_GLOBAL uint2 *)(a.x + (size_t)i * 4));
+    HLQ_ROW_REDUCE(ssq, op_add);
+    if ((tid & 15) == 0) scratch[tid >> 4] = ssq;
+    lds_barrier();
+    if (tid < 64) {
+        float v = tid < (nthreads >> 4) ? scratch[tid] : 0.f;
+        HLQ_ROW_REDUCE(v, op_add);
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        if (tid == 0) scratch[64] = v;
+    }
+    lds_barrier();
+    return rsqrtf(scratch[64] / (float)K + a.eps);
 }
 
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
@@ -402,10 +415,18 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     const size_t k0 = (size_t)(u0 + ub) * HLQ_UNIT;
     const int nchunks = nuw * 32;
     float rstd = 1.f;
-    if (prologue == 1) rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x);
+    // what the last step adds to the output is fetched first of all, so that its latency is not
+    // left at the end of the kernel (wave 0 finishes a tile; a run of column blocks loads it there)
+    uint16_t pre_bias = 0, pre_res = 0;
+    if (!MULTI && wave == 0 && cb * HLQ_CB + lane < a.N) {
+        if (a.bias) pre_bias = a.bias[cb * HLQ_CB + lane];
+        if (residual) pre_res = residual[cb * HLQ_CB + lane];
+    }
+    uint2 rfirst = make_uint2(0, 0);
+    if (prologue == 1) rfirst = rstd_first_load(a, K, tid);
     uint2 raw, raw2;
     // lanes past the run (and waves without one, whose k0 is the end of the slice) re-read a valid chunk
-    load_chunk(a, prologue, K, nchunks ? k0 + (size_t)min(lane, nchunks - 1) * 4 : 0, raw, raw2);
+    load_chunk<PLAIN>(a, prologue, K, nchunks ? k0 + (size_t)min(lane, nchunks - 1) * 4 : 0, raw, raw2);
     asm volatile("" ::: "memory");      // keep both activation loads ahead of the weight loads
 
     float acc = 0.f;
@@ -415,6 +436,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         load_slot<BITS, G64, PAIRED, 0>(slot[0], here, u0, min(s_begin, s_last), lane);
     }
     asm volatile("" ::: "memory");
+    if (prologue == 1) rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst);
 
     // ... the tables are built as soon as the activations are in (a wave that first queued all
     // its weight loads would sit in the memory pipeline's back-pressure instead) ...
@@ -428,7 +450,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         load_slot<BITS, G64, PAIRED, d>(slot[d], here, u0, min(s_begin + d, s_last), lane);
     });
     for (int ci = lane + 64; ci < nchunks; ci += 64) {      // runs of more than two units (not the common case)
-        load_chunk(a, prologue, K, k0 + (size_t)ci * 4, raw, raw2);
+        load_chunk<PLAIN>(a, prologue, K, k0 + (size_t)ci * 4, raw, raw2);
         build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0);
     }
     HLQ_STAMP(1);
@@ -455,8 +477,8 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         HLQ_STAMP(4);
         if (a.ksplit == 1) {
             if (wave == 0 && n < a.N) {
-                if (a.bias) total += (float)__builtin_bit_cast(_Float16, a.bias[n]);
-                if (residual) total += (float)__builtin_bit_cast(_Float16, residual[n]);
+                if (a.bias) total += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
+                if (residual) total += (float)__builtin_bit_cast(_Float16, MULTI ? residual[n] : pre_res);
                 a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)total);
             }
             return;
@@ -490,8 +512,8 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                         if (s0 + j < a.ksplit) sum += v[j];
                 }
                 if (n < a.N) {
-                    if (a.bias) sum += (float)__builtin_bit_cast(_Float16, a.bias[n]);
-                    if (residual) sum += (float)__builtin_bit_cast(_Float16, residual[n]);
+                    if (a.bias) sum += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
+                    if (residual) sum += (float)__builtin_bit_cast(_Float16, MULTI ? residual[n] : pre_res);
                     a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
                 }
                 if (lane == 0) __hip_atomic_store(&a.counters[cbf], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -552,24 +574,24 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     HLQ_STAMP_FLUSH;
 }
 
-template <int BITS, bool G64, int NSLOT, bool PAIRED>
+template <int BITS, bool G64, int NSLOT, bool PAIRED, bool PLAIN>
 __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 {
     extern __shared__ __align__(256) unsigned char smem[];
     int sel = 0;
-    gemv_tile<BITS, G64, NSLOT, false, false, PAIRED>(a, blockIdx.y, blockIdx.x, 1, smem, sel);      // grid = (slices, column blocks)
+    gemv_tile<BITS, G64, NSLOT, false, PLAIN, PAIRED>(a, blockIdx.y, blockIdx.x, 1, smem, sel);      // grid = (slices, column blocks)
 }
 
 // One GEMV with more column blocks than the chip has CUs: every workgroup takes a run of
 // consecutive column blocks (tables built once, weights prefetched across the blocks) instead
 // of the launch holding two workgroups per CU that each build the same tables.
-template <int BITS, bool G64, int NSLOT, bool PAIRED>
+template <int BITS, bool G64, int NSLOT, bool PAIRED, bool PLAIN>
 __global__ __launch_bounds__(1024) void hlq_gemv_run_kernel(const GemvArgs a, int run)
 {
     extern __shared__ __align__(256) unsigned char smem[];
     const int cb0 = blockIdx.y * run;               // grid = (slices, runs of column blocks)
     int sel = 0;
-    gemv_tile<BITS, G64, NSLOT, true, false, PAIRED>(a, cb0, blockIdx.x, min(run, a.ncb - cb0), smem, sel);
+    gemv_tile<BITS, G64, NSLOT, true, PLAIN, PAIRED>(a, cb0, blockIdx.x, min(run, a.ncb - cb0), smem, sel);
 }
 
 // Many independent GEMVs in one launch: the tiles of all of them form one list that the
@@ -647,16 +669,17 @@ bool paired_ok(int spw, int ups, int ksplit)
     return MG::fits(NSLOT) && spw % MG::SIZE == 0 && (G64 || ksplit == 1 || ups % 2 == 0);
 }
 
-template <int BITS, bool G64, int NSLOT, bool PAIRED>
-int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
+// PLAIN: no prologue and no residual, known when the kernel is compiled
+template <int BITS, bool G64, int NSLOT, bool PAIRED, bool PLAIN>
+int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
-    auto kern = hlq_gemv_kernel<BITS, G64, NSLOT, PAIRED>;
+    auto kern = hlq_gemv_kernel<BITS, G64, NSLOT, PAIRED, PLAIN>;
     static bool big_lds_done[64] = {};        // per template instance
     if (!allow_big_lds((const void *)kern, lds, MAX_LDS, big_lds_done)) return ELUTQ_ERR_HIP;
     // more tiles than CUs and runs that fit the slots: runs of column blocks, one workgroup per CU
     const int run = (a.ncb * a.ksplit + NUM_CU_RUN - 1) / NUM_CU_RUN;
     if (run > 1 && a.spw <= NSLOT && waves == 16) {
-        auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT, PAIRED>;
+        auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT, PAIRED, PLAIN>;
         static bool big_lds_run_done[64] = {};
         if (!allow_big_lds((const void *)kern_run, lds, MAX_LDS, big_lds_run_done)) return ELUTQ_ERR_HIP;
         const int groups = (a.ncb + run - 1) / run;
@@ -665,6 +688,13 @@ int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
     }
     hipLaunchKernelGGL(kern, dim3(a.ksplit, a.ncb), dim3(waves * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
+}
+
+template <int BITS, bool G64, int NSLOT, bool PAIRED>
+int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
+{
+    if (a.prologue == 0 && !a.residual) return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, true>(a, waves, lds, stream);
+    return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, false>(a, waves, lds, stream);
 }
 
 template <int BITS, bool G64, int NSLOT>
