@@ -257,21 +257,25 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.f;
 
+    // The rows of the next block are requested before the current block is worked on, so that a
+    // block's memory round trip lies under the arithmetic of the one before.  The loads are
+    // unconditional (rows clamped to the last cached one: past the end every lane re-reads one row,
+    // which costs next to nothing), so they can be waited for by count.
+    const int last_row = max(pos - 1, 0);        // rows below pos do not change during the launch
     for (int blk = sp; blk * BLOCK_ROWS < pos; blk += S) {
         const int base = blk * BLOCK_ROWS;
-        if (blk != sp) {                                 // later blocks of a long context
+        uint4 kn[BATCH], vn[BATCH];
 #pragma unroll
-            for (int b = 0; b < BATCH; b++) {
-                const int p = min(base + (wave + WAVES * b) * 4 + r, a.max_seq - 1);
-                const size_t row = ((size_t)p * a.nkv + g) * D;
-                kk[b] = ((const uint4 *)(a.kc + row))[seg];
-                vv[b] = ((const uint4 *)(a.vc + row))[seg];
-            }
-            // keep the whole batch of loads ahead of the first use (the scheduler would otherwise
-            // sink each load to its consumer and serialise the memory round trips)
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
+        for (int b = 0; b < BATCH; b++) {
+            const int p = min(base + S * BLOCK_ROWS + (wave + WAVES * b) * 4 + r, last_row);
+            const size_t row = ((size_t)p * a.nkv + g) * D;
+            kn[b] = ((const uint4 *)(a.kc + row))[seg];
+            vn[b] = ((const uint4 *)(a.vc + row))[seg];
         }
+        // keep the whole batch of loads ahead of the arithmetic (the scheduler would otherwise
+        // sink each load to its consumer and serialise the memory round trips)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
         // one running-max update per batch: scores first, then a single rescale of the stream
         float sc[BATCH], mx = m;
 #pragma unroll
@@ -298,6 +302,8 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
             }
             m = mx;
         }
+#pragma unroll
+        for (int b = 0; b < BATCH; b++) { kk[b] = kn[b]; vv[b] = vn[b]; }
         ATTN_STAMP(stamp_i); stamp_i++;
     }
     if (wave == 0 && sp == 0) {                          // the token being decoded, from LDS (row 0 only)
@@ -498,7 +504,7 @@ extern "C" int elutq_decode_rope_attn_split_f16(const void *d_qkv, void *d_k_cac
     if (head_dim != FAST_D)
         hipLaunchKernelGGL(rope_attn_kernel, dim3(n_heads), dim3(ATTN_WAVES * 64), 0, (hipStream_t)stream, a);
     else if (splits == 1)
-        hipLaunchKernelGGL((rope_attn_d128_kernel<8, 8>), dim3(n_heads), dim3(8 * 64), 0, (hipStream_t)stream, a);
+        hipLaunchKernelGGL((rope_attn_d128_kernel<8, 4>), dim3(n_heads), dim3(8 * 64), 0, (hipStream_t)stream, a);
     else
         hipLaunchKernelGGL((rope_attn_d128_kernel<4, 4>), dim3(n_heads * splits), dim3(4 * 64), 0, (hipStream_t)stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
