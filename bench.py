@@ -336,6 +336,23 @@ def main():
             torch.cuda.empty_cache()
         other_formats[f"w{bits}g{group}"] = res
 
+    # ---- one GEMV large enough that the launch and its start-up no longer matter: an lm_head-sized
+    # layer (vocabulary 128256) at w2g128, over a ring of distinct weight sets
+    k, n = 4096, 128256
+    nbytes = algorithmic_bytes(k, n, BITS, GROUP)
+    ring = [Gemv(lib, make_device_layer(k, n, BITS, GROUP, seed=30_000 + i, device=dev), xs[k],
+                 torch.empty(1, n, dtype=torch.float16, device=dev), ws) for i in range(4)]
+
+    def launch_big(stream, ring=ring):
+        for c in ring:
+            c(stream)
+
+    sec = time_graph(torch, launch_big, max(3, min(a.steps, 10)), 2) / len(ring)
+    large_shape = {f"{k}x{n}": {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                                "bytes": nbytes, "ring_sets": len(ring)}}
+    del ring
+    torch.cuda.empty_cache()
+
     dom = per_shape["4096x14336"]
     roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": dom["GBps"] / HBM_PEAK_GBPS,
@@ -357,6 +374,7 @@ def main():
         "frac_hbm_peak": value / HBM_PEAK_GBPS,
         "per_shape": per_shape,
         "per_shape_other_formats": other_formats,
+        "large_shape": large_shape,
         "roofline": roofline,
         # supplementary: the same 224 GEMVs handed to elutq_hlq_gemv_group_* (they are independent in this
         # sweep); `value` above stays the one-call-per-GEMV figure of the drop-in entry point
