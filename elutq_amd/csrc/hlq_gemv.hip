@@ -460,7 +460,12 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     __builtin_amdgcn_wave_barrier();
     HLQ_STAMP(2);
 
-    // Combine the waves of this workgroup, then the slices of this column block.
+    // Combine the waves of this workgroup, then the slices of this column block.  The wave that
+    // does it waits for its partial-sum stores to be acknowledged, and that wait covers every load
+    // it has in flight: in a run of column blocks those are the next block's weights, fetched a
+    // moment ago.  Where the last wave has no sub-tasks (a slice of 28 units at 2 planes keeps 14
+    // waves busy) it loads nothing inside the run and takes this part over.
+    const int fin = (MULTI && a.ksplit > 1 && (nw - 1) * a.spw >= nst) ? nw - 1 : 0;
     auto finish = [&](int cbf, float accf) __attribute__((always_inline)) {
         float *red = red0 + red_sel * nw * HLQ_CB;
         red_sel ^= 1;
@@ -469,14 +474,14 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         if (nw > 1) {
             red[wave * HLQ_CB + lane] = accf;
             lds_barrier();
-            if (wave == 0) {
+            if (wave == fin) {
                 total = 0.f;
                 for (int w = 0; w < nw; w++) total += red[w * HLQ_CB + lane];
             }
         }
         HLQ_STAMP(4);
         if (a.ksplit == 1) {
-            if (wave == 0 && n < a.N) {
+            if (wave == fin && n < a.N) {
                 if (a.bias) total += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
                 if (residual) total += (float)__builtin_bit_cast(_Float16, MULTI ? residual[n] : pre_res);
                 a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)total);
@@ -488,7 +493,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         // waits for its stores to be acknowledged before it takes a ticket, and the reader's
         // loads depend on the ticket it drew -- so no cache write-back / invalidate is needed.
         const size_t npad = (size_t)a.ncb * HLQ_CB;
-        if (wave == 0) {
+        if (wave == fin) {
             __hip_atomic_store(&a.partial[(size_t)slice * npad + n], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             HLQ_STAMP(5);
@@ -544,12 +549,13 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
             const CbBase next = cb_base<BITS>(a, min(cb + c + 1, cb + ncb_run - 1), u0);   // past the run: a reload nobody reads
             float accc = 0.f;
             HLQ_STAMP(2);
-            static_for<0, NSLOT>([&](auto dc) __attribute__((always_inline)) {
-                constexpr int d = decltype(dc)::value;
-                const int st = s_begin + d;
-                if (st < s_end) accc = run_slot(dc, st, accc);
-                load_slot<BITS, G64, PAIRED, d>(slot[d], next, u0, min(st, s_last), lane);
-            });
+            if (s_begin < s_end)                              // wave-uniform; a wave without sub-tasks loads nothing here
+                static_for<0, NSLOT>([&](auto dc) __attribute__((always_inline)) {
+                    constexpr int d = decltype(dc)::value;
+                    const int st = s_begin + d;
+                    if (st < s_end) accc = run_slot(dc, st, accc);
+                    load_slot<BITS, G64, PAIRED, d>(slot[d], next, u0, min(st, s_last), lane);
+                });
             HLQ_STAMP(3);
             finish(cb + c, accc);
             HLQ_STAMP(6);
