@@ -8,8 +8,8 @@
 //   y[m][n] = sum_g ( c[n,g] * (sum_{k in g} x[m][k])  +  sum_b sum_{k in g} x[m][k] * (+-s[b,n,g]/2) )
 //
 // where the sign is + for a set plane bit.  The B operand of v_mfma_f32_32x32x16_f16 is
-// built in registers from the packed planes: one v_alignbit moves two plane bits (k and
-// k + 16 of a 32-k dword) onto the sign bits of a packed fp16 pair, one v_bfi merges them
+// built in registers from the packed planes: one shift (a rotation where the bits wrap) moves two
+// plane bits (k and k + 16 of a 32-k dword) onto the sign bits of a packed fp16 pair, one v_bfi merges them
 // with |s|/2 -- so every B element is exactly +-s/2, every product exact in fp32, and the
 // fp32 accumulator of the MFMA sums planes and groups alike; nothing is rounded before the
 // final fp16 store.  The centre term uses per-row sums of x over 64-k halves, taken while
@@ -270,8 +270,12 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
                             for (int q = 0; q < 4; q++) {
                                 // stored dwords are rotated left by HLQ_ROT: bit k = 4s + q goes to the sign of
                                 // the low fp16, bit k + 16 to the sign of the high one
-                                const uint32_t sh = (uint32_t)(4 * s + q + HLQ_ROT - 15) & 31u;
-                                const uint32_t rot = __builtin_amdgcn_alignbit(bits[b][j], bits[b][j], sh);
+                                // (positions k + HLQ_ROT and k + 16 + HLQ_ROT move to 15 and 31).  Without a wrap a plain
+                                // shift does it -- a 32-bit-encoded instruction, which the SIMD retires in 2.4
+                                // cycles where v_alignbit (64-bit encoding) takes 4.25
+                                const int mv = 15 - (4 * s + q + HLQ_ROT);       // left shift that is needed (compile time)
+                                const uint32_t src = bits[b][j];
+                                const uint32_t rot = mv > 0 ? src << mv : (mv == 0 ? src : __builtin_amdgcn_alignbit(src, src, (uint32_t)-mv));
                                 o[q] = (rot & 0x80008000u) | (mag[b][j] & 0x7fff7fffu);
                             }
                             const half8 bop = __builtin_bit_cast(half8, make_uint4(o[0], o[1], o[2], o[3]));
