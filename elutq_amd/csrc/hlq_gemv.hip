@@ -364,7 +364,9 @@ __device__ __forceinline__ void static_for(F &&f)
     }
 }
 
-constexpr int DEPTH = 4;    // sub-tasks a wave keeps in flight
+// Sub-tasks a wave keeps in flight at most.  Three planes get six slots: a unit pair (one meta
+// group at G = 128) is six sub-tasks, and K = 4096 gives a wave exactly that run.
+constexpr int depth_of(int bits) { return bits == 3 ? 6 : 4; }
 
 // One workgroup = one column block x one K slice.  Its (unit, plane) sub-tasks are dealt to
 // the waves in contiguous runs of `spw`; every wave builds the activation tables of the
@@ -712,15 +714,22 @@ int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
     return launch_gemv_p<BITS, G64, NSLOT, false>(a, waves, lds, stream);
 }
 
-// NSLOT = sub-tasks a wave keeps in flight: its whole run when that is at most DEPTH.
+// NSLOT = sub-tasks a wave keeps in flight: its whole run when that is at most depth_of(BITS).
 template <int BITS, bool G64>
 int launch_gemv(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
+    constexpr int DEPTH = depth_of(BITS);
     switch (a.spw < DEPTH ? a.spw : DEPTH) {
     case 1: return launch_gemv_n<BITS, G64, 1>(a, waves, lds, stream);
     case 2: return launch_gemv_n<BITS, G64, 2>(a, waves, lds, stream);
     case 3: return launch_gemv_n<BITS, G64, 3>(a, waves, lds, stream);
-    default: return launch_gemv_n<BITS, G64, 4>(a, waves, lds, stream);
+    case 4: return launch_gemv_n<BITS, G64, 4>(a, waves, lds, stream);
+    default:
+        if constexpr (DEPTH == 6) {
+            if (a.spw == 5) return launch_gemv_n<BITS, G64, 5>(a, waves, lds, stream);
+            return launch_gemv_n<BITS, G64, 6>(a, waves, lds, stream);
+        }
+        return launch_gemv_n<BITS, G64, 4>(a, waves, lds, stream);
     }
 }
 
@@ -772,7 +781,13 @@ int launch_group(int nslot, bool paired, const GemvArgs *p, const GroupItem *it,
     case 1: return launch_group_n<BITS, G64, 1>(paired, p, it, n, grid, waves, lds, st);
     case 2: return launch_group_n<BITS, G64, 2>(paired, p, it, n, grid, waves, lds, st);
     case 3: return launch_group_n<BITS, G64, 3>(paired, p, it, n, grid, waves, lds, st);
-    default: return launch_group_n<BITS, G64, 4>(paired, p, it, n, grid, waves, lds, st);
+    case 4: return launch_group_n<BITS, G64, 4>(paired, p, it, n, grid, waves, lds, st);
+    default:
+        if constexpr (depth_of(BITS) == 6) {
+            if (nslot == 5) return launch_group_n<BITS, G64, 5>(paired, p, it, n, grid, waves, lds, st);
+            return launch_group_n<BITS, G64, 6>(paired, p, it, n, grid, waves, lds, st);
+        }
+        return launch_group_n<BITS, G64, 4>(paired, p, it, n, grid, waves, lds, st);
     }
 }
 
@@ -815,10 +830,10 @@ void choose_shape(const HlqGeo &g, int &ksplit, int &waves)
 {
     if (ksplit <= 0) {
         ksplit = g.ncb >= 64 ? 1 : NUM_CU / g.ncb;
-        // runs longer than a wave's slots (3 and 4 planes at K = 4096): slice while that still leaves
+        // more than four sub-tasks per wave (3 and 4 planes at K = 4096): slice while that still leaves
         // at most one workgroup per CU
-        const int by_slots = (g.U * g.bits + 16 * DEPTH - 1) / (16 * DEPTH);
-        if (by_slots > 1 && g.ncb < 128) {
+        const int by_slots = (g.U * g.bits + 16 * depth_of(g.bits) - 1) / (16 * depth_of(g.bits));
+        if (g.U * g.bits > 16 * 4 && g.ncb < 128) {
             const int fill = NUM_CU / g.ncb > by_slots ? NUM_CU / g.ncb : by_slots;
             if (ksplit < fill) ksplit = fill;
         }
@@ -920,7 +935,8 @@ static int group_shape(const elutq_gemv_problem &p, int bits, int group, GroupSh
     if (!p.d_planes || !p.d_scales || !p.d_zeros || !p.d_x || !p.d_y) return ELUTQ_ERR_NULL;
     sh.g = hlq_geo(p.K, p.N, bits, group);
     // the list supplies the parallelism: slice K only as far as LDS and the run length ask for
-    // (a wave's run must fit its DEPTH slots: at most 16 * DEPTH sub-tasks per slice)
+    // (a wave's run must fit its slots: at most 16 * depth_of(bits) sub-tasks per slice)
+    const int DEPTH = depth_of(bits);
     int ksplit = (sh.g.U * bits + 16 * DEPTH - 1) / (16 * DEPTH);
     int ups = (sh.g.U + ksplit - 1) / ksplit;
     while (ups > 1 && (gemv_lds_bytes(ups, bits, 16) > (size_t)MAX_LDS / 2 ||            // two workgroups per CU
@@ -1017,7 +1033,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
             a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + poff[i]);
         }
         a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr;
-        const int ns = a.spw < DEPTH ? a.spw : DEPTH;
+        const int ns = a.spw < depth_of(bits) ? a.spw : depth_of(bits);
         if (ns > nslot) nslot = ns;
         const size_t l = gemv_lds_bytes(sh.ups, bits, 16);
         if (l > lds) lds = l;
