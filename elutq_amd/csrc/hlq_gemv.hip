@@ -883,11 +883,14 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return ELUTQ_ERR_TUNING;
+    const bool auto_waves = waves <= 0;
     choose_shape(g, ksplit, waves);
     int ups = (g.U + ksplit - 1) / ksplit;
     // shrink the slice so its tables fit in LDS, then the slice count so that no slice is empty
     while (gemv_lds_bytes(ups, bits, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
     ksplit = (g.U + ups - 1) / ups;
+    // a slice of at most 16 sub-tasks: eight waves with two each start sooner than sixteen with one
+    if (auto_waves && ups * bits <= 16) waves = 8;
 
     GemvArgs a;
     a.planes = (const HLQ_GLOBAL uint4 *)d_planes;
