@@ -354,6 +354,19 @@ __device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scr
     return rsqrtf(scratch[64] / (float)K + a.eps);
 }
 
+// A SIMD issues from its oldest wave first, so the waves of a workgroup finish their runs one
+// after the other and the last one works alone at the end.  Every wave therefore lowers its own
+// priority as it gets on with its run (3 at the start, 0 in the last quarter): the waves that are
+// behind are served first and all finish together.
+__device__ __forceinline__ void progress_prio(int done, int total)
+{
+    const int d4 = done * 4;                 // quarter of the run the wave is in, without a division
+    if (d4 < total) __builtin_amdgcn_s_setprio(3);
+    else if (d4 < 2 * total) __builtin_amdgcn_s_setprio(2);
+    else if (d4 < 3 * total) __builtin_amdgcn_s_setprio(1);
+    else __builtin_amdgcn_s_setprio(0);
+}
+
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
 template <int B, int E, typename F>
 __device__ __forceinline__ void static_for(F &&f)
@@ -408,6 +421,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     float *rstd_scratch = red0 + 2 * nw * HLQ_CB;                          // [RSTD_SCRATCH]
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
+    __builtin_amdgcn_s_setprio(3);
     HLQ_STAMP(0);
     // Activations first, then the weight stream.  Every load below is unconditional (a wave
     // whose run is shorter than NSLOT re-reads its last sub-task), so the number of loads
@@ -555,6 +569,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                 static_for<0, NSLOT>([&](auto dc) __attribute__((always_inline)) {
                     constexpr int d = decltype(dc)::value;
                     const int st = s_begin + d;
+                    progress_prio(d, a.spw);
                     if (st < s_end) accc = run_slot(dc, st, accc);
                     load_slot<BITS, G64, PAIRED, d>(slot[d], next, u0, min(st, s_last), lane);
                 });
@@ -572,6 +587,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         static_for<0, NSLOT>([&](auto dc) __attribute__((always_inline)) {
             constexpr int d = decltype(dc)::value;
             const int st = base + d;
+            progress_prio(st - s_begin, a.spw);
             if (st < s_end) acc = run_slot(dc, st, acc);
             if (base + NSLOT < s_end)                      // wave-uniform: only runs longer than NSLOT refill
                 load_slot<BITS, G64, PAIRED, d>(slot[d], here, u0, min(st + NSLOT, s_last), lane);
