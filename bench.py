@@ -359,7 +359,7 @@ def main():
                 # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
                 # `bench.py --mode kernel`, each scaled by what the same counter reads for `--mode copy`
                 # (summary under profiles/); a property of the kernel's access pattern, not of this run.
-                "traffic": 17_634_000,
+                "traffic": 17_644_000,
                 "kernel": "hlq_gemv_kernel<2,false> K=4096 N=14336", "us_per_launch": dom["us"],
                 "bytes_per_launch": dom["bytes"]}
 
