@@ -67,6 +67,24 @@ def make_layer(k: int, n: int, bits: int = 2, group: int = 128, m: int = 1, seed
                       bias=bvec, x=x.numpy())
 
 
+def make_sparse_plane(k: int, n: int, group: int = 128, density: float = 0.25, seed: int = 0,
+                      scale_range=(0.02, 0.08)):
+    """A seeded block-sparse extra plane in the form the reference's loader consumes
+    (C++/ops/src/arm/parameters.cpp:19-64): every (32-channel tile, group) pair is a block with
+    probability `density`; blocks are listed by ascending channel start, then ascending k start.
+    Returns (bits uint8 0/1 [nblk, 32, G], scale fp16 [nblk, 32], mask uint32 [nblk, 2])."""
+    assert n % 32 == 0 and k % group == 0
+    g = torch.Generator().manual_seed(seed)
+    pick = torch.rand(n // 32, k // group, generator=g) < density
+    idx = pick.nonzero()                                           # row-major: tile, then group
+    mask = torch.stack([idx[:, 0] * 32, idx[:, 1] * group], 1).to(torch.int64).numpy().astype(np.uint32)
+    nblk = mask.shape[0]
+    bits = torch.randint(0, 2, (nblk, 32, group), generator=g, dtype=torch.uint8).numpy()
+    lo, hi = scale_range
+    scale = (torch.rand(nblk, 32, generator=g) * (hi - lo) + lo).to(torch.float16).numpy()
+    return bits, scale, mask
+
+
 # (K, N) of the LLaMA-3-8B projections and of the LLaMA-2-13B prefill shapes.
 LLAMA3_8B_SHAPES = {
     "q_proj": (4096, 4096), "k_proj": (4096, 1024), "v_proj": (4096, 1024), "o_proj": (4096, 4096),

@@ -16,6 +16,11 @@ Reference lines each function follows (paths relative to the reference root):
   gemv_fp16_chain               C++/ops/src/arm/arm_gemm.cpp:248-308 +
                                 C++/ops/src/arm/arm_t_mac_kernal.cpp:364-469
   gemm_rows                     C++/ops/src/arm/arm_gemm.cpp:362-387
+  sparse_export_arrays          C++/ops/src/arm/parameters.cpp:19-64 (what the loader reads)
+  rearrange_sparse_reference    C++/ops/src/arm/arm_t_mac_kernal.cpp:554-647
+  dequantize_sparse             C++/ops/src/arm/arm_t_mac_kernal.cpp:678-788 (which weights a block adds to)
+  gemv_sparse_fp16_chain        C++/ops/src/arm/arm_gemm.cpp:725-808 +
+                                C++/ops/src/arm/arm_t_mac_kernal.cpp:678-788
 
 Parity pins (tests/test_oracle_*.py): the reference ships no tests, golden
 vectors or fixtures for this path, so every function is pinned by mathematics:
@@ -27,7 +32,12 @@ shapes; lut_float by brute force over the 16 subsets; gemv_fp16_chain against
 the C restatement (oracle/lut_gemv_ref.c, an independent implementation that
 indexes the rearranged buffers the way the reference kernel does) bit-for-bit,
 and against integer-only inputs where every fp16 operation is exact so the
-chain must equal the float64 result bit-for-bit.
+chain must equal the float64 result bit-for-bit.  The sparse extra plane has no
+producer in the reference (its exporter always writes use_sparse = false), so its
+format is the one the C++ loader and kernel consume; it is pinned by the cases
+that reduce to the dense path (blocks on every tile and group == one more dense
+plane, bit for bit; no blocks == the base layer), by brute force over the
+loader's index expressions, and by the C restatement bit for bit.
 """
 from __future__ import annotations
 
@@ -37,6 +47,8 @@ __all__ = [
     "pack_planes", "unpack_planes", "export_arrays", "weight_config",
     "dequantize", "gemv_f64", "gemm_f64", "rearrange_reference",
     "lut_float", "gemv_fp16_chain", "gemm_rows", "rel_err",
+    "SparsePlane", "sparse_export_arrays", "sparse_weight_config", "rearrange_sparse_reference",
+    "dequantize_sparse", "gemv_sparse_f64", "gemv_sparse_fp16_chain",
 ]
 
 
@@ -255,6 +267,109 @@ def gemm_rows(x, w_quant, w_scale, w_zero, group, bias=None, fused=True) -> np.n
     """m > 1 in the reference is a row loop over the GEMV (arm_gemm.cpp:380-385)."""
     x = np.asarray(x, dtype=np.float16)
     return np.stack([gemv_fp16_chain(r, w_quant, w_scale, w_zero, group, bias, fused) for r in x])
+
+
+# --------------------------------------------------------------------------- #
+# Block-sparse extra plane (use_sparse = true): parameters.cpp:19-64,
+# arm_t_mac_kernal.cpp:554-647 and 678-788, arm_gemm.cpp:683-868.
+#
+# Beside `base_bit` dense planes the layer holds one more plane that exists only
+# on listed blocks of 32 output channels x G input channels.  weight_mask.bin is
+# a list of uint32 pairs (channel start, k start), grouped by channel start in
+# ascending order (the thread split at arm_gemm.cpp:840-846 relies on that).
+# Block i's bits follow the dense planes in w_quant.bin as uint8 [32][G/8]
+# (LSB-first along K like every plane), its 32 fp16 scales follow the dense
+# scales in w_scale.bin; there is no zero term for the extra plane.
+# --------------------------------------------------------------------------- #
+class SparsePlane:
+    """bits uint8 0/1 [nblk, 32, G]; scale fp16 [nblk, 32]; mask uint32 [nblk, 2] = (channel start, k start)."""
+
+    def __init__(self, bits, scale, mask, group: int):
+        self.bits = np.asarray(bits, dtype=np.uint8)
+        self.scale = np.asarray(scale, dtype=np.float16)
+        self.mask = np.asarray(mask, dtype=np.uint32).reshape(-1, 2)
+        self.group = int(group)
+        nblk = self.mask.shape[0]
+        assert self.bits.shape == (nblk, 32, group) and self.scale.shape == (nblk, 32)
+        assert np.all(np.diff(self.mask[:, 0].astype(np.int64)) >= 0), "blocks must be grouped by ascending channel start"
+
+    @property
+    def packed(self) -> np.ndarray:
+        """uint8 [nblk, 32, G/8], the bytes that follow the dense planes in w_quant.bin."""
+        return pack_planes(self.bits) if self.bits.size else np.zeros((0, 32, self.group // 8), np.uint8)
+
+
+def sparse_export_arrays(w_quant, w_scale, sp: SparsePlane):
+    """-> (w_quant.bin bytes, w_scale.bin bytes, weight_mask.bin bytes) of a sparse layer:
+    the dense payloads (export_arrays) with the block data appended (parameters.cpp:36-64)."""
+    wq = np.ascontiguousarray(w_quant, dtype=np.uint8).tobytes() + sp.packed.tobytes()
+    ws = np.ascontiguousarray(w_scale, dtype=np.float16).tobytes() + sp.scale.tobytes()
+    return wq, ws, np.ascontiguousarray(sp.mask, dtype=np.uint32).tobytes()
+
+
+def sparse_weight_config(k: int, n: int, base_bits: int, has_bias: bool, sp: SparsePlane, groupsize: int | None = None) -> dict:
+    """Keys the loader reads for a sparse layer (parameters.cpp:17-27); weight_data_len is what
+    the rearrangement checks: K*N*base_bit/8 + mask_len*2*G (arm_t_mac_kernal.cpp:594)."""
+    cfg = weight_config(k, n, base_bits, has_bias, groupsize)
+    mask_len = int(sp.mask.size)
+    cfg["use_sparse"] = True
+    cfg["sparse_mask_len"] = mask_len
+    cfg["weight_data_len"] = int(k * n * base_bits // 8 + mask_len * 2 * sp.group)
+    return cfg
+
+
+def rearrange_sparse_reference(w_quant, w_scale, w_zero, sp: SparsePlane):
+    """Flat (weight u8, scale f16, zero f16) as t_mac_g4_rearrange_weight_sparse_impl leaves them:
+    dense planes [bit][tile32][K/8][32] (no thread dimension), then every block as [G/8][32];
+    dense scales [bit][tile32][g][32] followed by the block scales untouched; zeros [tile32][g][32]."""
+    wq, ws, wz = rearrange_reference(w_quant, w_scale, w_zero, sp.group, 1)
+    blocks = sp.packed.transpose(0, 2, 1).reshape(-1)
+    return np.concatenate([wq, blocks]), np.concatenate([ws, sp.scale.reshape(-1)]), wz
+
+
+def dequantize_sparse(w_quant, w_scale, w_zero, sp: SparsePlane, dtype=np.float64) -> np.ndarray:
+    """Dense W [N, K] of a sparse layer: the base planes' W plus, on every block,
+    scale[blk, ch] where the block's bit is set."""
+    w = dequantize(w_quant, w_scale, w_zero, sp.group, dtype)
+    for i, (c0, k0) in enumerate(sp.mask.astype(np.int64)):
+        w[c0:c0 + 32, k0:k0 + sp.group] += sp.bits[i].astype(dtype) * sp.scale[i].astype(dtype)[:, None]
+    return w
+
+
+def gemv_sparse_f64(x, w_quant, w_scale, w_zero, sp: SparsePlane, bias=None) -> np.ndarray:
+    y = dequantize_sparse(w_quant, w_scale, w_zero, sp) @ np.asarray(x).astype(np.float64).reshape(-1)
+    return y if bias is None else y + np.asarray(bias).astype(np.float64)
+
+
+def gemv_sparse_fp16_chain(x, w_quant, w_scale, w_zero, sp: SparsePlane, bias=None, fused=True) -> np.ndarray:
+    """The reference's op order for a sparse layer (arm_gemm.cpp:725-808): zero fold and dense
+    planes exactly as in gemv_fp16_chain, then the extra plane as the last one
+    (arm_t_mac_kernal.cpp:678-788): per block acc = sequential fp16 sum of LUT[lo] then LUT[hi]
+    per byte; over a run of blocks with the same channel start c = acc*s for the first,
+    c += acc*s afterwards; out[channels] = fp16(out + c) once per run; bias last."""
+    x = np.asarray(x, dtype=np.float16).reshape(-1)
+    y = gemv_fp16_chain(x, w_quant, w_scale, w_zero, sp.group, None, fused)
+    lut = lut_float(x)
+    packed = sp.packed
+    nblk = sp.mask.shape[0]
+    c = None
+    for i in range(nblk):
+        c0, k0 = int(sp.mask[i, 0]), int(sp.mask[i, 1])
+        acc = np.zeros(32, dtype=np.float16)
+        for l in range(0, sp.group, 8):
+            byte = packed[i, :, l // 8]
+            t = (k0 + l) // 4
+            acc = _h(acc.astype(np.float32) + lut[t, byte & 15].astype(np.float32))
+            acc = _h(acc.astype(np.float32) + lut[t + 1, byte >> 4].astype(np.float32))
+        if i == 0 or c0 != int(sp.mask[i - 1, 0]):
+            c = _h(acc.astype(np.float32) * sp.scale[i].astype(np.float32))
+        else:
+            c = _mac16(c, acc, sp.scale[i], fused)
+        if i == nblk - 1 or c0 != int(sp.mask[i + 1, 0]):
+            y[c0:c0 + 32] = _h(y[c0:c0 + 32].astype(np.float32) + c.astype(np.float32))
+    if bias is not None:
+        y = _h(y.astype(np.float32) + np.asarray(bias, dtype=np.float16).astype(np.float32))
+    return y
 
 
 # --------------------------------------------------------------------------- #

@@ -13,6 +13,10 @@
  *   run_chunk             arm_gemm.cpp:248-308          (zero fold, planes, bias)
  *   elutq_ref_gemv        arm_gemm.cpp:312-360          (N split over threads)
  *   elutq_ref_gemm        arm_gemm.cpp:362-387          (m > 1: row loop)
+ *   elutq_ref_rearrange_sparse  arm_t_mac_kernal.cpp:554-647 (loader permutation, use_sparse)
+ *   update_plane_sparse   arm_t_mac_kernal.cpp:678-788  (block-sparse extra plane)
+ *   run_chunk_sparse      arm_gemm.cpp:725-808          (zero fold, dense planes, extra plane, bias)
+ *   elutq_ref_gemv_sparse arm_gemm.cpp:811-868          (N split; blocks split by channel start)
  *   elutq_ref_gemv_fast   same data flow with AVX2 pshufb lookups (the x86
  *                         counterpart of vqtbl1q_u8) and fp32 accumulators; used
  *                         only as the timed CPU baseline, never as a checker.
@@ -222,6 +226,159 @@ int elutq_ref_gemm(int m, int k, int n, const h16 *input, h16 *output, const uin
         if (rc) return rc;
     }
     return 0;
+}
+
+/* ------------------------------------------------------------------------- *
+ * use_sparse = true: `bits - 1` dense planes and one block-sparse extra plane.
+ * mask_data holds mask_len uint32: pairs (channel start, k start) of blocks of
+ * 32 channels x Actk inputs, grouped by ascending channel start.
+ * ------------------------------------------------------------------------- */
+
+/* arm_t_mac_kernal.cpp:554-647.  weight / w_scale hold the dense part followed
+ * by the blocks' bits ([32][Actk/8] each) / scales ([32] each); the scale tail
+ * is left as it is (the reference permutes the dense part in place). */
+int elutq_ref_rearrange_sparse(int out_channel, int in_channel, int bits, int Actk,
+                               const uint32_t *mask_data, uint32_t mask_len,
+                               const uint8_t *weight, const h16 *w_scale, const h16 *w_zero,
+                               uint8_t *weight_out, h16 *w_scale_out, h16 *w_zero_out)
+{
+    (void)mask_data;
+    int base_bit = bits - 1;
+    long index = 0;
+    for (int bit = 0; bit < base_bit; bit++) {
+        const uint8_t *ws = weight + (long)bit * out_channel * in_channel / 8;
+        for (int i = 0; i < out_channel; i += 32)
+            for (int j = 0; j < in_channel / 8; j++)
+                for (int k = 0; k < 32; k++)
+                    weight_out[index++] = ws[(long)(i + k) * in_channel / 8 + j];
+    }
+    long len = (long)mask_len;
+    const uint8_t *wsp = weight + (long)base_bit * out_channel * in_channel / 8;
+    for (long i = 0; i < len; i += 2)
+        for (int j = 0; j < Actk / 8; j++)
+            for (int k = 0; k < 32; k++)
+                weight_out[index++] = wsp[i * 2 * Actk + (long)k * Actk / 8 + j];
+    if (index != (long)in_channel * out_channel * base_bit / 8 + len * 2 * Actk) return 0;
+
+    index = 0;
+    for (int bit = 0; bit < base_bit; bit++) {
+        const h16 *ss = w_scale + (long)bit * out_channel * in_channel / Actk;
+        for (int i = 0; i < out_channel; i += 32)
+            for (int j = 0; j < in_channel; j += Actk)
+                for (int k = 0; k < 32; k++)
+                    w_scale_out[index++] = ss[(long)(i + k) * in_channel / Actk + j / Actk];
+    }
+    if (index != (long)base_bit * in_channel * out_channel / Actk) return 0;
+    memcpy(w_scale_out + index, w_scale + index, sizeof(h16) * (size_t)(len / 2 * 32));
+
+    index = 0;
+    for (int i = 0; i < out_channel; i += 32)
+        for (int j = 0; j < in_channel; j += Actk)
+            for (int k = 0; k < 32; k++)
+                w_zero_out[index++] = w_zero[(long)(i + k) * in_channel / Actk + j / Actk];
+    if (index != (long)in_channel * out_channel / Actk) return 0;
+    return 1;
+}
+
+/* arm_t_mac_kernal.cpp:678-788.  `out` is the layer's whole output vector:
+ * the channel start in the mask is absolute. */
+static void update_plane_sparse(h16 *out, const uint8_t *weight, const h16 *lut, const h16 *w_scale,
+                                const uint32_t *mask_data, int len, int ActK, int fused)
+{
+    h16 c[32];
+    for (int i = 0; i < len; i += 2) {
+        int x = (int)mask_data[i];
+        int y = (int)mask_data[i + 1];
+        h16 acc[32];
+        memset(acc, 0, sizeof(acc));
+        for (int l = 0; l < ActK; l += 8) {
+            const uint8_t *w = weight + (long)i * 2 * ActK + 4 * l;
+            const h16 *lut_lo = lut + (long)((y + l) / 4) * 16;
+            const h16 *lut_hi = lut + (long)((y + l) / 4 + 1) * 16;
+            for (int ch = 0; ch < 32; ch++) {
+                acc[ch] = hadd(acc[ch], lut_lo[w[ch] & 15]);
+                acc[ch] = hadd(acc[ch], lut_hi[w[ch] >> 4]);
+            }
+        }
+        const h16 *s = w_scale + (long)(i / 2) * 32;
+        if (i == 0 || x != (int)mask_data[i - 2])
+            for (int ch = 0; ch < 32; ch++) c[ch] = hmul(acc[ch], s[ch]);
+        else
+            for (int ch = 0; ch < 32; ch++) c[ch] = hmac(c[ch], acc[ch], s[ch], fused);
+        if (i == len - 2 || x != (int)mask_data[i + 2])
+            for (int ch = 0; ch < 32; ch++) out[x + ch] = hadd(out[x + ch], c[ch]);
+    }
+}
+
+/* arm_gemm.cpp:725-808 (MultiThreadGemvW_lowbit_Activation_FP_Sparse::Run): all
+ * pointers are the layer's, the thread's share is channels [start, end) and
+ * mask entries [mask_start, mask_end). */
+static void run_chunk_sparse(int k, int n, int start, int end, int mask_start, int mask_end,
+                             const h16 *input, const uint8_t *weight, const h16 *w_scale,
+                             const h16 *w_zero, const h16 *bias, const uint32_t *mask_data,
+                             h16 *output, int Actk, int bit, h16 *input_sum, h16 *lut, int fused)
+{
+    for (int i = 0; i < k; i += Actk) {
+        h16 s = 0;
+        for (int j = 0; j < Actk; j++) s = hadd(s, input[i + j]);
+        input_sum[i / Actk] = s;
+    }
+    int cnt_per_row = k / Actk;
+    for (int i = start; i < end; i += 32) {
+        h16 o[32];
+        memset(o, 0, sizeof(o));
+        for (int j = 0; j < cnt_per_row; j++) {
+            const h16 *z = w_zero + (long)i * k / Actk + 32 * j;
+            for (int ch = 0; ch < 32; ch++) o[ch] = hmac(o[ch], input_sum[j], z[ch], fused);
+        }
+        memcpy(output + i, o, sizeof(o));
+    }
+    elutq_ref_lut(k, input, lut);
+    for (int i = 0; i < bit; i++) {
+        if (i == bit - 1) {
+            long weight_bias = (long)i * k * n / 8 + 2L * mask_start * Actk;
+            long w_scale_bias = (long)i * k * n / Actk + (long)mask_start * 16;
+            update_plane_sparse(output, weight + weight_bias, lut, w_scale + w_scale_bias,
+                                mask_data + mask_start, mask_end - mask_start, Actk, fused);
+        } else {
+            long weight_bias = (long)i * k * n / 8 + (long)start * k / 8;
+            long w_scale_bias = (long)i * k * n / Actk + (long)start * k / Actk;
+            update_plane_scalar(output + start, weight + weight_bias, k, end - start, lut,
+                                w_scale + w_scale_bias, Actk, fused);
+        }
+    }
+    if (bias)
+        for (int j = start; j < end; j++) output[j] = hadd(output[j], bias[j]);
+}
+
+/* arm_gemm.cpp:811-868: channels split into ceil(n/T) chunks; a thread takes the
+ * mask entries whose channel start falls into its chunk (linear scans over the
+ * sorted list).  `bit` counts the extra plane.  Returns 0, or -1 if scratch
+ * allocation fails. */
+int elutq_ref_gemv_sparse(int k, int n, const h16 *input, h16 *output, const uint8_t *weight,
+                          const h16 *w_scale, const h16 *w_zero, const h16 *bias,
+                          const uint32_t *mask_data, uint32_t mask_len, int Actk, int bit,
+                          int threadnum, int fused)
+{
+    int chunk_size = (n + threadnum - 1) / threadnum;
+    int fail = 0;
+#pragma omp parallel for num_threads(threadnum) schedule(static, 1)
+    for (int i = 0; i < threadnum; i++) {
+        int start = chunk_size * i;
+        int end = MINI(start + chunk_size, n);
+        if (start >= end) continue;
+        uint32_t ms = 0, me = 0;
+        while (ms < mask_len && mask_data[ms] < (uint32_t)start) ms += 2;
+        while (me < mask_len && mask_data[me] < (uint32_t)end) me += 2;
+        h16 *input_sum = (h16 *)malloc(sizeof(h16) * (size_t)(k / Actk));
+        h16 *lut = (h16 *)malloc(sizeof(h16) * (size_t)k * 4);
+        if (!input_sum || !lut) { fail = 1; free(input_sum); free(lut); continue; }
+        run_chunk_sparse(k, n, start, end, (int)ms, (int)me, input, weight, w_scale, w_zero, bias,
+                         mask_data, output, Actk, bit, input_sum, lut, fused);
+        free(input_sum);
+        free(lut);
+    }
+    return fail ? -1 : 0;
 }
 
 /* ------------------------------------------------------------------------- *

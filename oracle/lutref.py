@@ -41,6 +41,10 @@ def load():
     lib.elutq_ref_gemv.restype = ci
     lib.elutq_ref_gemm.argtypes = [ci, ci, ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci]
     lib.elutq_ref_gemm.restype = ci
+    lib.elutq_ref_rearrange_sparse.argtypes = [ci, ci, ci, ci, vp, ctypes.c_uint32, vp, vp, vp, vp, vp, vp]
+    lib.elutq_ref_rearrange_sparse.restype = ci
+    lib.elutq_ref_gemv_sparse.argtypes = [ci, ci, vp, vp, vp, vp, vp, vp, vp, ctypes.c_uint32, ci, ci, ci, ci]
+    lib.elutq_ref_gemv_sparse.restype = ci
     lib.elutq_ref_gemv_fast.argtypes = [ci, ci, vp, vp, vp, vp, vp, vp, ci, ci, ci]
     lib.elutq_ref_gemv_fast.restype = ci
     _lib = lib
@@ -105,6 +109,43 @@ class RefWeight:
                                         _p(self.zero), _p(self.bias), self.group, self.bits, self.threads)
         if rc:
             raise MemoryError("elutq_ref_gemv_fast")
+        return y
+
+
+class RefSparseWeight:
+    """A use_sparse layer after the reference's loader: `w_quant_bytes` / `w_scale_bytes` /
+    `mask_bytes` are the contents of w_quant.bin / w_scale.bin / weight_mask.bin (dense part
+    followed by the block data), `base_bits` the number of dense planes."""
+
+    def __init__(self, w_quant_bytes: bytes, w_scale_bytes: bytes, w_zero, mask_bytes: bytes,
+                 k: int, n: int, base_bits: int, group: int, bias=None):
+        lib = load()
+        if n % 32:
+            raise ValueError("reference layout needs 32-channel tiles")
+        self.k, self.n, self.bits, self.group = int(k), int(n), int(base_bits) + 1, int(group)
+        wq = np.frombuffer(w_quant_bytes, dtype=np.uint8).copy()
+        ws = np.frombuffer(w_scale_bytes, dtype=np.float16).copy()
+        wz = np.ascontiguousarray(w_zero, dtype=np.float16)
+        self.mask = np.frombuffer(mask_bytes, dtype=np.uint32).copy()
+        self.weight, self.scale, self.zero = np.empty_like(wq), np.empty_like(ws), np.empty(wz.size, np.float16)
+        ok = lib.elutq_ref_rearrange_sparse(self.n, self.k, self.bits, self.group, _p(self.mask), self.mask.size,
+                                            _p(wq), _p(ws), _p(wz), _p(self.weight), _p(self.scale), _p(self.zero))
+        if ok != 1:
+            raise RuntimeError("elutq_ref_rearrange_sparse: element count mismatch")
+        self.bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.float16)
+
+    def gemv(self, x, threads: int = 1, fused: bool = True) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float16).reshape(-1)
+        assert x.size == self.k
+        chunk = (self.n + threads - 1) // threads
+        if chunk % 32:
+            raise ValueError("reference layout needs 32-channel tiles in every thread chunk")
+        y = np.empty(self.n, dtype=np.float16)
+        rc = load().elutq_ref_gemv_sparse(self.k, self.n, _p(x), _p(y), _p(self.weight), _p(self.scale),
+                                          _p(self.zero), _p(self.bias), _p(self.mask), self.mask.size,
+                                          self.group, self.bits, threads, int(fused))
+        if rc:
+            raise MemoryError("elutq_ref_gemv_sparse")
         return y
 
 
