@@ -44,10 +44,11 @@ def parse():
     p.add_argument("--no-decode", action="store_true", help="skip the decode tokens/s leg")
     p.add_argument("--no-gemm", action="store_true", help="skip the small-batch GEMM leg")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
-    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "gemm", "group"], default="full",
+    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "gemm", "group", "sparse"], default="full",
                    help="kernel: only the dominant GEMV (4096x14336) over its weight ring, for counter runs; "
                         "copy: a plain 64 MiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE; "
-                        "decode / gemm: only that leg (for kernel traces)")
+                        "decode / gemm: only that leg (for kernel traces); "
+                        "sparse: GEMVs of layers with a block-sparse extra plane beside the same layers without it")
     p.add_argument("--launches", type=int, default=256, help="launches in --mode kernel / copy")
     return p.parse_args()
 
@@ -155,6 +156,54 @@ def gemm_leg(torch, lib, dev, steps):
     return out
 
 
+def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
+    """Batch-1 GEMV of w2g128 layers that carry a block-sparse extra plane on `density` of their
+    (32 channels x 128 inputs) blocks -- two launches: the plane's fp32 term, then the dense GEMV that
+    adds it -- next to the same dense layers alone.  Weight rings of `ring_len` layers per shape."""
+    import numpy as np
+
+    from elutq_amd.hlq_linear import sparse_index
+    from elutq_amd.synth import LLAMA3_8B_SHAPES, algorithmic_bytes, make_device_layer
+    out = {}
+    for name in ("q_proj", "gate_proj"):
+        k, n = LLAMA3_8B_SHAPES[name]
+        g = torch.Generator().manual_seed(k + n)
+        pick = (torch.rand(n // 32, k // GROUP, generator=g) < density).nonzero()
+        mask = torch.stack([pick[:, 0] * 32, pick[:, 1] * GROUP], 1).numpy().astype(np.uint32)
+        nblk = mask.shape[0]
+        index = torch.from_numpy(sparse_index(mask, k, n, GROUP)).to(dev)
+        ring = []
+        for i in range(ring_len):
+            mod = make_device_layer(k, n, BITS, GROUP, seed=i, device=dev)
+            blocks = torch.randint(0, 256, (nblk, 32, GROUP // 8), dtype=torch.uint8, device=dev)
+            scales = (torch.rand(nblk, 32, device=dev) * 0.06 + 0.02).to(torch.float16)
+            ring.append((mod, blocks, scales))
+        x = torch.randn(1, k, device=dev).to(torch.float16)
+        y = torch.empty(1, n, dtype=torch.float16, device=dev)
+        ws = torch.zeros(lib.elutq_hlq_sparse_workspace_bytes(k, n, BITS, GROUP, 1), dtype=torch.uint8, device=dev)
+
+        def launch_sparse(stream):
+            for mod, blocks, scales in ring:
+                rc = lib.elutq_hlq_sparse_gemv_f16(mod.planes.data_ptr(), mod.scales.data_ptr(), mod.zeros.data_ptr(), None,
+                                                   blocks.data_ptr(), scales.data_ptr(), index.data_ptr(), nblk,
+                                                   x.data_ptr(), y.data_ptr(), k, n, BITS, GROUP, ws.data_ptr(), ws.numel(), stream)
+                if rc:
+                    raise RuntimeError(f"elutq_hlq_sparse_gemv_f16 failed: {rc}")
+
+        dense = [Gemv(lib, mod, x, y, ws) for mod, _, _ in ring]
+
+        def launch_dense(stream):
+            for gv in dense:
+                gv(stream)
+
+        t_sp = time_graph(torch, launch_sparse, steps, warmup) / ring_len
+        t_de = time_graph(torch, launch_dense, steps, warmup) / ring_len
+        sparse_bytes = nblk * (32 * GROUP // 8 + 64 + 4) + 4 * (n // 32 + 1) + 8 * n      # blocks, scales, index, fp32 term out and in
+        out[f"{k}x{n}"] = {"blocks": nblk, "density": density, "sparse_layer_us": t_sp * 1e6, "dense_layer_us": t_de * 1e6,
+                           "sparse_plane_bytes": sparse_bytes, "dense_bytes": algorithmic_bytes(k, n, BITS, GROUP)}
+    return out
+
+
 def counter_mode(a, torch, lib, dev):
     """Eager launches of one kernel only, so a rocprofv3 --pmc run sees nothing else of size."""
     from elutq_amd.synth import algorithmic_bytes, make_device_layer
@@ -222,6 +271,9 @@ def main():
         print(json.dumps({"mode": "group", "gemvs_per_launch": len(mods), "bytes_per_launch": nbytes, "us_per_launch": sec * 1e6,
                           "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}))
         grp.close()
+        return
+    if a.mode == "sparse":
+        print(json.dumps({"mode": "sparse", "sparse_gemv_w2g128": sparse_leg(torch, lib, dev, a.steps, a.warmup)}))
         return
     if a.mode != "full":
         counter_mode(a, torch, lib, dev)

@@ -12,7 +12,7 @@ import sys
 _PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_PKG, "csrc")
 LIB_PATH = os.path.join(_PKG, "libelutq_hip.so")
-SOURCES = ["hlq_gemv.hip", "hlq_gemm.hip", "hlq_misc.hip", "decode_ops.hip", "hlq_repack.cpp"]
+SOURCES = ["hlq_gemv.hip", "hlq_gemm.hip", "hlq_misc.hip", "hlq_sparse.hip", "decode_ops.hip", "hlq_repack.cpp"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

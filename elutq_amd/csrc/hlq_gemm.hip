@@ -19,6 +19,7 @@
 
 #include "../../include/elutq_hip.h"
 #include "hlq_layout.h"
+#include "hlq_internal.h"
 
 namespace {
 
@@ -37,6 +38,7 @@ struct GemmArgs {
     const uint16_t *bias;
     const uint16_t *x;      // fp16 [M][K]
     uint16_t *y;            // fp16 [M][N]
+    const float *extra;     // fp32 [M][N] added to the output before it is rounded, or null
     float *partial;         // [ksplit][MT*32][ncb*64]
     unsigned *counters;     // one per workgroup column (super block)
     int M, N, K, U, NT, ncb;
@@ -357,6 +359,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
             if (m < a.M && n < a.N) {
                 float s = outv[it];
                 if (a.bias) s += (float)__builtin_bit_cast(_Float16, a.bias[n]);
+                if (a.extra) s += a.extra[(size_t)m * a.N + n];
                 a.y[(size_t)m * a.N + n] = __builtin_bit_cast(uint16_t, (_Float16)s);
             }
         }
@@ -414,6 +417,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
         if (m < a.M && n < a.N) {
             float s = sum[it];
             if (a.bias) s += (float)__builtin_bit_cast(_Float16, a.bias[n]);
+            if (a.extra) s += a.extra[(size_t)m * a.N + n];
             a.y[(size_t)m * a.N + n] = __builtin_bit_cast(uint16_t, (_Float16)s);
         }
     }
@@ -484,9 +488,6 @@ int dispatch_gemm(const GemmArgs &a, int bits, bool g64, int kw, hipStream_t str
 
 }  // namespace
 
-// Rows per launch; more rows are processed in chunks of this many (weights re-streamed).
-#define HLQ_GEMM_MAX_M 64
-
 extern "C" {
 
 #ifdef HLQ_TIMING
@@ -506,6 +507,25 @@ int elutq_hlq_gemm_f16_tuned(const void *d_planes, const void *d_scales, const v
     if (M == 1)
         return elutq_hlq_gemv_f16(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace,
                                   workspace_bytes, stream);
+    for (int m0 = 0; m0 < M; m0 += HLQ_GEMM_MAX_M) {
+        const int mc = M - m0 < HLQ_GEMM_MAX_M ? M - m0 : HLQ_GEMM_MAX_M;
+        int rc = hlq_gemm_chunk_with_extra(d_planes, d_scales, d_zeros, d_bias, (const uint16_t *)d_x + (size_t)m0 * K,
+                                           (uint16_t *)d_y + (size_t)m0 * N, mc, K, N, bits, group, d_workspace,
+                                           workspace_bytes, stream, kparts, ksplit, nullptr);
+        if (rc != ELUTQ_OK) return rc;
+    }
+    return ELUTQ_OK;
+}
+
+}  // extern "C"
+
+// One launch of the MFMA kernel: 1 <= M <= 64 rows, with an optional fp32 [M][N] term added to
+// every output before it is rounded to fp16 (the block-sparse extra plane of a use_sparse layer).
+int hlq_gemm_chunk_with_extra(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                              const void *d_x, void *d_y, int M, int K, int N, int bits, int group, void *d_workspace,
+                              size_t workspace_bytes, void *stream, int kparts, int ksplit, const float *d_extra)
+{
+    if (M < 1 || M > HLQ_GEMM_MAX_M) return ELUTQ_ERR_SHAPE;
     if (bits < 1 || bits > 4) return ELUTQ_ERR_BITS;
     if (group != 64 && group != 128) return ELUTQ_ERR_GROUP;
     if (K < HLQ_UNIT || N < 1 || K % HLQ_UNIT != 0 || K % group != 0) return ELUTQ_ERR_SHAPE;
@@ -516,33 +536,31 @@ int elutq_hlq_gemm_f16_tuned(const void *d_planes, const void *d_scales, const v
     int kw = kparts, ks = ksplit, ups;
     hlq_gemm_shape(g, kw, ks, ups);
 
-    for (int m0 = 0; m0 < M; m0 += HLQ_GEMM_MAX_M) {
-        const int mc = M - m0 < HLQ_GEMM_MAX_M ? M - m0 : HLQ_GEMM_MAX_M;
-        GemmArgs a;
-        a.planes = (const uint4 *)d_planes;
-        a.scales = (const uint32_t *)d_scales;
-        a.zeros = (const uint32_t *)d_zeros;
-        a.bias = (const uint16_t *)d_bias;
-        a.x = (const uint16_t *)d_x + (size_t)m0 * K;
-        a.y = (uint16_t *)d_y + (size_t)m0 * N;
-        a.M = mc; a.N = N; a.K = K; a.U = g.U; a.NT = g.NT; a.ncb = g.ncb;
-        a.ksplit = ks; a.ups = ups;
-        a.partial = nullptr; a.counters = nullptr;
-        if (ks > 1) {
-            const int mpad = mc <= 32 ? 32 : 64;
-            const int cbw = GW / kw, nsb = (g.ncb + cbw - 1) / cbw;
-            if (!d_workspace) return ELUTQ_ERR_NULL;
-            if ((size_t)nsb * sizeof(unsigned) > (size_t)WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
-            if (workspace_bytes < (size_t)WS_COUNTER_BYTES + (size_t)ks * mpad * g.ncb * HLQ_CB * sizeof(float))
-                return ELUTQ_ERR_WORKSPACE;
-            a.counters = (unsigned *)d_workspace;
-            a.partial = (float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
-        }
-        int rc = dispatch_gemm(a, bits, group == 64, kw, (hipStream_t)stream);
-        if (rc != ELUTQ_OK) return rc;
+    GemmArgs a;
+    a.planes = (const uint4 *)d_planes;
+    a.scales = (const uint32_t *)d_scales;
+    a.zeros = (const uint32_t *)d_zeros;
+    a.bias = (const uint16_t *)d_bias;
+    a.x = (const uint16_t *)d_x;
+    a.y = (uint16_t *)d_y;
+    a.extra = d_extra;
+    a.M = M; a.N = N; a.K = K; a.U = g.U; a.NT = g.NT; a.ncb = g.ncb;
+    a.ksplit = ks; a.ups = ups;
+    a.partial = nullptr; a.counters = nullptr;
+    if (ks > 1) {
+        const int mpad = M <= 32 ? 32 : 64;
+        const int cbw = GW / kw, nsb = (g.ncb + cbw - 1) / cbw;
+        if (!d_workspace) return ELUTQ_ERR_NULL;
+        if ((size_t)nsb * sizeof(unsigned) > (size_t)WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
+        if (workspace_bytes < (size_t)WS_COUNTER_BYTES + (size_t)ks * mpad * g.ncb * HLQ_CB * sizeof(float))
+            return ELUTQ_ERR_WORKSPACE;
+        a.counters = (unsigned *)d_workspace;
+        a.partial = (float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
-    return ELUTQ_OK;
+    return dispatch_gemm(a, bits, group == 64, kw, (hipStream_t)stream);
 }
+
+extern "C" {
 
 int elutq_hlq_gemm_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
                        const void *d_x, void *d_y, int M, int K, int N, int bits, int group, void *d_workspace,

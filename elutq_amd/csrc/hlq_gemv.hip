@@ -31,6 +31,7 @@
 
 #include "../../include/elutq_hip.h"
 #include "hlq_layout.h"
+#include "hlq_internal.h"
 
 namespace {
 
@@ -65,6 +66,7 @@ struct GemvArgs {
     float eps;
     const HLQ_GLOBAL uint16_t *norm_w;  // fp16 [K]      (prologue 1)
     const HLQ_GLOBAL uint16_t *residual;  // fp16 [N] added to the output, or null
+    const HLQ_GLOBAL float *extra;        // fp32 [N] added to the output before it is rounded, or null
 };
 
 #ifdef HLQ_TIMING
@@ -395,7 +397,7 @@ constexpr int depth_of(int bits) { return bits == 3 ? 6 : 4; }
 // built once; while a wave looks up its sub-tasks of one column block, each slot it has
 // consumed is refilled with the same sub-task of the next block, so the weight stream never
 // stops between blocks.  Needs runs of at most NSLOT sub-tasks per wave.
-// PLAIN: no prologue and no residual (their fields of `a` are not read).
+// PLAIN: no prologue, no residual and no extra term (their fields of `a` are not read).
 template <int BITS, bool G64, int NSLOT, bool MULTI, bool PLAIN, bool PAIRED>
 __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, int ncb_run, unsigned char *smem, int &red_sel)
 {
@@ -406,6 +408,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
 #endif
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
+    const HLQ_GLOBAL float *extra = PLAIN ? nullptr : a.extra;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
@@ -500,6 +503,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
             if (wave == fin && n < a.N) {
                 if (a.bias) total += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
                 if (residual) total += (float)__builtin_bit_cast(_Float16, MULTI ? residual[n] : pre_res);
+                if (extra) total += extra[n];
                 a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)total);
             }
             return;
@@ -535,6 +539,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                 if (n < a.N) {
                     if (a.bias) sum += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
                     if (residual) sum += (float)__builtin_bit_cast(_Float16, MULTI ? residual[n] : pre_res);
+                    if (extra) sum += extra[n];
                     a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
                 }
                 if (lane == 0) __hip_atomic_store(&a.counters[cbf], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -693,7 +698,7 @@ bool paired_ok(int spw, int ups, int ksplit)
     return MG::fits(NSLOT) && spw % MG::SIZE == 0 && (G64 || ksplit == 1 || ups % 2 == 0);
 }
 
-// PLAIN: no prologue and no residual, known when the kernel is compiled
+// PLAIN: no prologue, no residual and no extra term, known when the kernel is compiled
 template <int BITS, bool G64, int NSLOT, bool PAIRED, bool PLAIN>
 int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
@@ -717,7 +722,7 @@ int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 template <int BITS, bool G64, int NSLOT, bool PAIRED>
 int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
-    if (a.prologue == 0 && !a.residual) return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, true>(a, waves, lds, stream);
+    if (a.prologue == 0 && !a.residual && !a.extra) return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, true>(a, waves, lds, stream);
     return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, false>(a, waves, lds, stream);
 }
 
@@ -894,6 +899,19 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
                              size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,
                              int waves)
 {
+    return hlq_gemv_with_extra(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace,
+                               workspace_bytes, stream, fusion, ksplit, waves, nullptr);
+}
+
+}  // extern "C"
+
+// The fused GEMV with an fp32 vector [N] added to every output before it is rounded to fp16
+// (the block-sparse extra plane of a use_sparse layer, computed by another kernel on the same stream).
+int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                        const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
+                        size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,
+                        int waves, const float *d_extra)
+{
     int rc = check_shape(K, N, bits, group);
     if (rc != ELUTQ_OK) return rc;
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
@@ -920,7 +938,7 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
     const WavePlan wp = wave_plan(ups, bits, waves);
     a.spw = wp.spw; a.nuw_max = wp.nuw_max; a.wave_lds = wp.wave_lds;
     a.partial = nullptr; a.counters = nullptr;
-    a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr;
+    a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
     if (fusion) {
         if (fusion->prologue < 0 || fusion->prologue > 2) return ELUTQ_ERR_TUNING;
         if (fusion->prologue == 1 && !fusion->d_norm_weight) return ELUTQ_ERR_NULL;
@@ -929,6 +947,7 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
         a.norm_w = (const HLQ_GLOBAL uint16_t *)fusion->d_norm_weight;
         a.residual = (const HLQ_GLOBAL uint16_t *)fusion->d_residual;
     }
+    a.extra = (const HLQ_GLOBAL float *)d_extra;
     if (ksplit > 1) {
         if (!d_workspace) return ELUTQ_ERR_NULL;
         if ((size_t)g.ncb * sizeof(unsigned) > (size_t)WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
@@ -939,6 +958,8 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
     }
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves), (hipStream_t)stream);
 }
+
+extern "C" {
 
 // ---- grouped launch of independent GEMVs --------------------------------------------------
 struct GroupShape {                      // tile shape of one problem inside a group
@@ -1051,7 +1072,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
             a.counters = (HLQ_GLOBAL unsigned *)((unsigned char *)d_workspace + coff[i]);
             a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + poff[i]);
         }
-        a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr;
+        a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
         const int ns = a.spw < depth_of(bits) ? a.spw : depth_of(bits);
         if (ns > nslot) nslot = ns;
         const size_t l = gemv_lds_bytes(sh.ups, bits, 16);

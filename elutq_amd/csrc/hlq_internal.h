@@ -1,0 +1,21 @@
+// Calls between the library's own source files (not part of the C ABI).
+#pragma once
+#include <stddef.h>
+
+#include "../../include/elutq_hip.h"
+
+#define HLQ_INTERNAL __attribute__((visibility("hidden")))
+
+// elutq_hlq_gemv_fused_f16 with an fp32 vector [N] (device) added to every output before it is
+// rounded to fp16; d_extra may be null.
+HLQ_INTERNAL int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                                     const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
+                                     size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,
+                                     int waves, const float *d_extra);
+
+// One launch of the MFMA GEMM kernel, 1 <= M <= HLQ_GEMM_MAX_M rows, with an fp32 [M][N] term
+// (device) added to every output before it is rounded to fp16; d_extra may be null.
+HLQ_INTERNAL int hlq_gemm_chunk_with_extra(const void *d_planes, const void *d_scales, const void *d_zeros,
+                                           const void *d_bias, const void *d_x, void *d_y, int M, int K, int N, int bits,
+                                           int group, void *d_workspace, size_t workspace_bytes, void *stream, int kparts,
+                                           int ksplit, const float *d_extra);

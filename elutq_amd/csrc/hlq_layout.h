@@ -29,6 +29,7 @@
 #define HLQ_MAX_LDS (160 * 1024)       /* per workgroup on gfx950 */
 #define HLQ_WS_COUNTER_BYTES (64 * 1024) /* head of every workspace: one arrival counter per column block */
 #define HLQ_GEMM_WAVES 8               /* waves per GEMM workgroup */
+#define HLQ_GEMM_MAX_M 64              /* rows per GEMM launch; more rows run in chunks of this many (weights re-streamed) */
 
 struct HlqGeo {
     int K, N, bits, group;

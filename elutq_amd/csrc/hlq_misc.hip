@@ -61,6 +61,9 @@ const char *elutq_status_string(int status)
     case ELUTQ_ERR_WORKSPACE: return "workspace smaller than elutq_hlq_workspace_bytes()";
     case ELUTQ_ERR_HIP: return "a HIP runtime call failed";
     case ELUTQ_ERR_TUNING: return "ksplit / waves out of range";
+    case ELUTQ_ERR_SPARSE:
+        return "malformed sparse block list: need (channel start, k start) pairs, channel start a multiple of 32 below N "
+               "and ascending, k start a multiple of 4 with k + group <= K";
     }
     return "unknown status";
 }

@@ -10,6 +10,14 @@ One quantized linear layer is a directory `<root>/<layer id>/<module name>/`
   w_zero.bin          fp16  [N][K/G]                             (GPTQ/HLQ.py:218-221)
   bias.bin            fp16  [N], only if has_bias                (GPTQ/HLQ.py:184-191)
 
+A layer whose json says `use_sparse: true` (read by C++/ops/src/arm/parameters.cpp:19-64; the
+reference's exporter never writes one) has `base_bit` dense planes and a block-sparse extra plane:
+
+  weight_mask.bin     uint32 [sparse_mask_len]: pairs (channel start, k start) of blocks of
+                      32 channels x G inputs
+  w_quant.bin         dense planes, then every block as uint8 [32][G/8]
+  w_scale.bin         dense scales, then every block's fp16 [32]
+
 The reference exporter never writes the `groupsize` key its own loader reads
 (C++/ops/src/arm/parameters.cpp:17), so the reader takes it from the json when
 present and otherwise derives it from the size of w_zero.bin.
@@ -33,11 +41,22 @@ class ExportedLinear:
     w_scale: np.ndarray          # fp16  [bits, N, K/G]
     w_zero: np.ndarray           # fp16  [N, K/G]
     bias: np.ndarray | None      # fp16  [N]
+    sparse: "SparseBlocks | None" = None
 
 
-def write_export_dir(path: str, w_quant, w_scale, w_zero, bias=None, groupsize: int | None = None) -> None:
+@dataclass
+class SparseBlocks:
+    """Block-sparse extra plane as the files hold it."""
+    blocks: np.ndarray           # uint8  [nblk, 32, G/8], LSB-first along K
+    scale: np.ndarray            # fp16   [nblk, 32]
+    mask: np.ndarray             # uint32 [nblk, 2] = (channel start, k start)
+
+
+def write_export_dir(path: str, w_quant, w_scale, w_zero, bias=None, groupsize: int | None = None,
+                     sparse: SparseBlocks | None = None) -> None:
     """Writes the five files exactly as the reference exporter does.  `groupsize`
-    adds the key the reference forgets; leave None to reproduce its output."""
+    adds the key the reference forgets; leave None to reproduce its output.  `sparse` appends a
+    block-sparse extra plane in the form the reference's loader reads."""
     w_quant = np.ascontiguousarray(w_quant, dtype=np.uint8)
     w_scale = np.ascontiguousarray(w_scale, dtype=np.float16)
     w_zero = np.ascontiguousarray(w_zero, dtype=np.float16)
@@ -54,15 +73,29 @@ def write_export_dir(path: str, w_quant, w_scale, w_zero, bias=None, groupsize: 
     }
     if groupsize is not None:
         cfg["groupsize"] = int(groupsize)
+    quant_tail = scale_tail = b""
+    if sparse is not None:
+        blocks = np.ascontiguousarray(sparse.blocks, dtype=np.uint8)
+        mask = np.ascontiguousarray(sparse.mask, dtype=np.uint32).reshape(-1, 2)
+        sp_scale = np.ascontiguousarray(sparse.scale, dtype=np.float16)
+        nblk = mask.shape[0]
+        if blocks.ndim != 3 or blocks.shape[:2] != (nblk, 32) or sp_scale.shape != (nblk, 32):
+            raise ValueError("sparse blocks must be uint8 [nblk, 32, G/8] with fp16 scales [nblk, 32]")
+        quant_tail, scale_tail = blocks.tobytes(), sp_scale.tobytes()
+        cfg["use_sparse"] = True
+        cfg["sparse_mask_len"] = int(mask.size)
+        cfg["weight_data_len"] += len(quant_tail)
+        with open(os.path.join(path, "weight_mask.bin"), "wb") as f:
+            f.write(mask.tobytes())
     if bias is not None:
         with open(os.path.join(path, "bias.bin"), "wb") as f:
             f.write(np.ascontiguousarray(bias, dtype=np.float16).tobytes())
     with open(os.path.join(path, "w_zero.bin"), "wb") as f:
         f.write(w_zero.tobytes())
     with open(os.path.join(path, "w_scale.bin"), "wb") as f:
-        f.write(w_scale.tobytes())
+        f.write(w_scale.tobytes() + scale_tail)
     with open(os.path.join(path, "w_quant.bin"), "wb") as f:
-        f.write(w_quant.tobytes())
+        f.write(w_quant.tobytes() + quant_tail)
     with open(os.path.join(path, "weight_config.json"), "w") as f:
         json.dump(cfg, f, indent=4)
 
@@ -70,11 +103,15 @@ def write_export_dir(path: str, w_quant, w_scale, w_zero, bias=None, groupsize: 
 def read_export_dir(path: str, groupsize: int | None = None) -> ExportedLinear:
     with open(os.path.join(path, "weight_config.json")) as f:
         cfg = json.load(f)
-    if cfg.get("use_sparse", False):
-        raise NotImplementedError("sparse extra-plane exports are not supported")
     k, n, bits = int(cfg["in_channel"]), int(cfg["out_channel"]), int(cfg["base_bit"])
+    use_sparse = bool(cfg.get("use_sparse", False))
+    mask_len = int(cfg["sparse_mask_len"]) if use_sparse else 0
+    if mask_len < 0 or mask_len % 2:
+        raise ValueError(f"{path}: sparse_mask_len {mask_len} is not an even, non-negative count")
+    nblk = mask_len // 2
+    dense_bytes = k * n * bits // 8
     w_quant = np.fromfile(os.path.join(path, "w_quant.bin"), dtype=np.uint8)
-    if w_quant.size != int(cfg["weight_data_len"]) or w_quant.size != k * n * bits // 8:
+    if w_quant.size != int(cfg["weight_data_len"]) or w_quant.size < dense_bytes:
         raise ValueError(f"{path}: w_quant.bin has {w_quant.size} bytes, config says {cfg['weight_data_len']}")
     w_zero = np.fromfile(os.path.join(path, "w_zero.bin"), dtype=np.float16)
     group = int(cfg.get("groupsize", 0)) or groupsize
@@ -84,9 +121,21 @@ def read_export_dir(path: str, groupsize: int | None = None) -> ExportedLinear:
         group = k * n // w_zero.size
     if w_zero.size * group != k * n:
         raise ValueError(f"{path}: w_zero.bin has {w_zero.size} values, expected {k * n // group}")
+    if w_quant.size != dense_bytes + nblk * 32 * group // 8:
+        raise ValueError(f"{path}: w_quant.bin has {w_quant.size} bytes, expected {dense_bytes} for the dense planes "
+                         f"and {nblk * 32 * group // 8} for {nblk} sparse blocks")
     w_scale = np.fromfile(os.path.join(path, "w_scale.bin"), dtype=np.float16)
-    if w_scale.size != bits * n * (k // group):
-        raise ValueError(f"{path}: w_scale.bin has {w_scale.size} values, expected {bits * n * (k // group)}")
+    dense_scales = bits * n * (k // group)
+    if w_scale.size != dense_scales + nblk * 32:
+        raise ValueError(f"{path}: w_scale.bin has {w_scale.size} values, expected {dense_scales + nblk * 32}")
+    sparse = None
+    if use_sparse:
+        mask = np.fromfile(os.path.join(path, "weight_mask.bin"), dtype=np.uint32)
+        if mask.size != mask_len:
+            raise ValueError(f"{path}: weight_mask.bin has {mask.size} values, config says {mask_len}")
+        sparse = SparseBlocks(blocks=w_quant[dense_bytes:].reshape(nblk, 32, group // 8),
+                              scale=w_scale[dense_scales:].reshape(nblk, 32), mask=mask.reshape(nblk, 2))
+        w_quant, w_scale = w_quant[:dense_bytes], w_scale[:dense_scales]
     bias = None
     if cfg.get("has_bias", False):
         bias = np.fromfile(os.path.join(path, "bias.bin"), dtype=np.float16)
@@ -95,7 +144,7 @@ def read_export_dir(path: str, groupsize: int | None = None) -> ExportedLinear:
     return ExportedLinear(k=k, n=n, bits=bits, group=int(group),
                           w_quant=w_quant.reshape(bits, n, k // 8),
                           w_scale=w_scale.reshape(bits, n, k // group),
-                          w_zero=w_zero.reshape(n, k // group), bias=bias)
+                          w_zero=w_zero.reshape(n, k // group), bias=bias, sparse=sparse)
 
 
 # ---------------------------------------------------------------------------------------
@@ -150,17 +199,44 @@ def is_repacked_dir(path: str) -> bool:
     return os.path.exists(os.path.join(path, REPACKED_JSON))
 
 
-def write_repacked_dir(path: str, k: int, n: int, bits: int, group: int, planes, scales, zeros, bias=None) -> None:
-    """Kernel-layout buffers of one linear layer as files that load with a plain copy."""
+def write_repacked_dir(path: str, k: int, n: int, bits: int, group: int, planes, scales, zeros, bias=None,
+                       sparse: SparseBlocks | None = None) -> None:
+    """Kernel-layout buffers of one linear layer as files that load with a plain copy.  A sparse
+    extra plane keeps its file form (the kernels read that form) under names of its own."""
     os.makedirs(path, exist_ok=True)
     for name, a in (("planes.bin", planes), ("scales.bin", scales), ("zeros.bin", zeros)):
         with open(os.path.join(path, name), "wb") as f:
             f.write(np.ascontiguousarray(a, dtype=np.uint8).tobytes())
     if bias is not None:
         write_fp16_bin(os.path.join(path, "bias.bin"), bias)
+    cfg = {"layout_version": REPACK_LAYOUT_VERSION, "in_channel": int(k), "out_channel": int(n),
+           "base_bit": int(bits), "groupsize": int(group), "has_bias": bias is not None}
+    if sparse is not None:
+        mask = np.ascontiguousarray(sparse.mask, dtype=np.uint32)
+        cfg["use_sparse"], cfg["sparse_mask_len"] = True, int(mask.size)
+        for name, a in (("sparse_blocks.bin", np.ascontiguousarray(sparse.blocks, dtype=np.uint8)),
+                        ("sparse_scales.bin", np.ascontiguousarray(sparse.scale, dtype=np.float16)),
+                        ("weight_mask.bin", mask)):
+            with open(os.path.join(path, name), "wb") as f:
+                f.write(a.tobytes())
     with open(os.path.join(path, REPACKED_JSON), "w") as f:
-        json.dump({"layout_version": REPACK_LAYOUT_VERSION, "in_channel": int(k), "out_channel": int(n),
-                   "base_bit": int(bits), "groupsize": int(group), "has_bias": bias is not None}, f, indent=4)
+        json.dump(cfg, f, indent=4)
+
+
+def read_repacked_sparse(path: str) -> SparseBlocks | None:
+    """The sparse extra plane of a repacked directory, or None."""
+    with open(os.path.join(path, REPACKED_JSON)) as f:
+        cfg = json.load(f)
+    if not cfg.get("use_sparse", False):
+        return None
+    mask_len, group = int(cfg["sparse_mask_len"]), int(cfg["groupsize"])
+    nblk = mask_len // 2
+    mask = np.fromfile(os.path.join(path, "weight_mask.bin"), dtype=np.uint32)
+    blocks = np.fromfile(os.path.join(path, "sparse_blocks.bin"), dtype=np.uint8)
+    scale = np.fromfile(os.path.join(path, "sparse_scales.bin"), dtype=np.float16)
+    if mask_len % 2 or mask.size != mask_len or blocks.size != nblk * 32 * group // 8 or scale.size != nblk * 32:
+        raise ValueError(f"{path}: sparse files do not match sparse_mask_len = {mask_len}")
+    return SparseBlocks(blocks.reshape(nblk, 32, group // 8), scale.reshape(nblk, 32), mask.reshape(nblk, 2))
 
 
 def read_repacked_dir(path: str):

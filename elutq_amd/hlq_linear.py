@@ -18,7 +18,8 @@ import torch
 from torch import nn
 
 from . import _lib
-from .export_io import ExportedLinear, is_repacked_dir, read_export_dir, read_repacked_dir
+from .export_io import (ExportedLinear, SparseBlocks, is_repacked_dir, read_export_dir, read_repacked_dir,
+                        read_repacked_sparse)
 
 _workspaces: dict = {}
 
@@ -76,12 +77,28 @@ def unpack_to_export_arrays(planes, scales, zeros, k: int, n: int, bits: int, gr
     return w_quant, w_scale, w_zero
 
 
+def sparse_index(mask, k: int, n: int, group: int) -> np.ndarray:
+    """(channel start, k start) pairs of a sparse extra plane -> the int32 index the kernels read
+    (elutq_hlq_sparse_index_host; raises on a malformed list)."""
+    L = _lib.lib()
+    mask = np.ascontiguousarray(mask, dtype=np.uint32).reshape(-1)
+    index = np.zeros(L.elutq_hlq_sparse_index_bytes(n, mask.size // 2) // 4, dtype=np.int32)
+    vp = ctypes.c_void_p
+    _lib.check(L.elutq_hlq_sparse_index_host(mask.ctypes.data_as(vp), mask.size, k, n, group,
+                                             index.ctypes.data_as(vp)), "elutq_hlq_sparse_index_host")
+    return index
+
+
 class HLQLinear(nn.Module):
-    """``nn.Linear``-shaped module over HLQ-packed weights (fp16 activations)."""
+    """``nn.Linear``-shaped module over HLQ-packed weights (fp16 activations).
+
+    `sparse`: optional block-sparse extra plane of a ``use_sparse`` export as device tensors
+    (blocks uint8 [nblk, 32, G/8], scales fp16 [nblk, 32], index int32 from `sparse_index`);
+    `bits` counts the dense planes only, as ``base_bit`` does in the export's json."""
 
     def __init__(self, in_features: int, out_features: int, bits: int, group_size: int,
                  planes: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor,
-                 bias: torch.Tensor | None = None):
+                 bias: torch.Tensor | None = None, sparse: tuple | None = None):
         super().__init__()
         self.in_features, self.out_features = int(in_features), int(out_features)
         self.bits, self.group_size = int(bits), int(group_size)
@@ -89,6 +106,18 @@ class HLQLinear(nn.Module):
         self.register_buffer("scales", scales)
         self.register_buffer("zeros", zeros)
         self.register_buffer("bias", bias)
+        sp_blocks, sp_scales, sp_index = sparse if sparse is not None else (None, None, None)
+        self.register_buffer("sparse_blocks", sp_blocks)
+        self.register_buffer("sparse_scales", sp_scales)
+        self.register_buffer("sparse_index", sp_index)
+        self.sparse_count = 0 if sp_scales is None else int(sp_scales.shape[0])
+        if sparse is not None:
+            want = _lib.lib().elutq_hlq_sparse_index_bytes(self.out_features, self.sparse_count)
+            if (sp_index.dtype != torch.int32 or sp_index.numel() * 4 != want or sp_scales.dtype != torch.float16
+                    or tuple(sp_scales.shape) != (self.sparse_count, 32) or sp_blocks.dtype != torch.uint8
+                    or sp_blocks.numel() != self.sparse_count * 32 * self.group_size // 8):
+                raise ValueError("sparse buffers do not match the layer: need blocks uint8 [nblk, 32, G/8], "
+                                 "scales fp16 [nblk, 32] and the int32 index of sparse_index()")
         self._ws_bytes = _lib.lib().elutq_hlq_workspace_bytes(self.in_features, self.out_features,
                                                               self.bits, self.group_size, 1)
         if self._ws_bytes == 0:
@@ -107,17 +136,30 @@ class HLQLinear(nn.Module):
     # -- construction ------------------------------------------------------------------
     @classmethod
     def from_export_arrays(cls, w_quant, w_scale, w_zero, group_size: int, bias=None,
-                           device="cuda") -> "HLQLinear":
+                           device="cuda", sparse: SparseBlocks | None = None) -> "HLQLinear":
         planes, scales, zeros = repack_export_arrays(w_quant, w_scale, w_zero, group_size)
         bits, n, k8 = np.asarray(w_quant).shape
         dev = torch.device(device)
         b = None if bias is None else torch.from_numpy(np.ascontiguousarray(bias, dtype=np.float16)).to(dev)
         return cls(k8 * 8, n, bits, group_size, torch.from_numpy(planes).to(dev),
-                   torch.from_numpy(scales).to(dev), torch.from_numpy(zeros).to(dev), b)
+                   torch.from_numpy(scales).to(dev), torch.from_numpy(zeros).to(dev), b,
+                   cls._sparse_to_device(sparse, k8 * 8, n, group_size, dev))
+
+    @staticmethod
+    def _sparse_to_device(sparse: SparseBlocks | None, k: int, n: int, group: int, dev):
+        if sparse is None:
+            return None
+        index = sparse_index(sparse.mask, k, n, group)
+        blocks = np.ascontiguousarray(sparse.blocks, dtype=np.uint8)
+        scale = np.ascontiguousarray(sparse.scale, dtype=np.float16).reshape(-1, 32)
+        if blocks.size != scale.shape[0] * 32 * group // 8 or 2 * scale.shape[0] != np.asarray(sparse.mask).size:
+            raise ValueError("sparse blocks / scales / mask disagree about the number of blocks")
+        return (torch.from_numpy(blocks.reshape(-1, 32, group // 8).copy()).to(dev), torch.from_numpy(scale.copy()).to(dev),
+                torch.from_numpy(index).to(dev))
 
     @classmethod
     def from_export(cls, e: ExportedLinear, device="cuda") -> "HLQLinear":
-        return cls.from_export_arrays(e.w_quant, e.w_scale, e.w_zero, e.group, e.bias, device)
+        return cls.from_export_arrays(e.w_quant, e.w_scale, e.w_zero, e.group, e.bias, device, e.sparse)
 
     @classmethod
     def from_export_dir(cls, path: str, device="cuda", group_size: int | None = None) -> "HLQLinear":
@@ -138,7 +180,8 @@ class HLQLinear(nn.Module):
         dev = torch.device(device)
         b = None if bias is None else torch.from_numpy(bias).to(dev)
         return cls(k, n, bits, group, torch.from_numpy(planes).to(dev), torch.from_numpy(scales).to(dev),
-                   torch.from_numpy(zeros).to(dev), b)
+                   torch.from_numpy(zeros).to(dev), b,
+                   cls._sparse_to_device(read_repacked_sparse(path), k, n, group, dev))
 
     # -- compute -----------------------------------------------------------------------
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -154,12 +197,23 @@ class HLQLinear(nn.Module):
         m = x2.shape[0]
         y = torch.empty((m, self.out_features), dtype=torch.float16, device=x.device)
         if m:
-            need = self._ws_bytes if m == 1 else self._ws_bytes_for(m)
+            L = _lib.lib()
+            if self.sparse_count:
+                need = L.elutq_hlq_sparse_workspace_bytes(self.in_features, self.out_features, self.bits,
+                                                          self.group_size, m)
+            else:
+                need = self._ws_bytes if m == 1 else self._ws_bytes_for(m)
             ws = _workspace(x.device, need)
             stream = torch.cuda.current_stream(x.device).cuda_stream
-            L = _lib.lib()
             bias = self.bias.data_ptr() if self.bias is not None else None
-            if m == 1:
+            if self.sparse_count:
+                rc = L.elutq_hlq_sparse_gemm_f16(self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
+                                                 bias, self.sparse_blocks.data_ptr(), self.sparse_scales.data_ptr(),
+                                                 self.sparse_index.data_ptr(), self.sparse_count, x2.data_ptr(),
+                                                 y.data_ptr(), m, self.in_features, self.out_features, self.bits,
+                                                 self.group_size, ws.data_ptr(), ws.numel(), stream)
+                _lib.check(rc, "elutq_hlq_sparse_gemm_f16")
+            elif m == 1:
                 rc = L.elutq_hlq_gemv_f16_tuned(self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
                                                 bias, x2.data_ptr(), y.data_ptr(), self.in_features,
                                                 self.out_features, self.bits, self.group_size,
@@ -180,7 +234,11 @@ class HLQLinear(nn.Module):
         """Batch-1 GEMV into a caller-owned `out`, optionally fused with the RMSNorm in front of
         the projection (prologue 1), the SiLU(gate)*up in front of it (prologue 2; x holds 2K
         values) and a residual added to the result.  No allocation: `ws` is the caller's
-        zero-initialised workspace.  See elutq_hlq_gemv_fused_f16 in include/elutq_hip.h."""
+        zero-initialised workspace.  See elutq_hlq_gemv_fused_f16 in include/elutq_hip.h.
+        A layer with a sparse extra plane cannot be fused (the plane reads the projection's own
+        input, which a prologue only forms inside the kernel): use forward()."""
+        if self.sparse_count:
+            raise NotImplementedError("a layer with a sparse extra plane has no fused GEMV; call forward()")
         f = _lib.GemvFusion(prologue, eps, norm_weight.data_ptr() if norm_weight is not None else None,
                             residual.data_ptr() if residual is not None else None)
         rc = _lib.lib().elutq_hlq_gemv_fused_f16(
@@ -203,11 +261,17 @@ class HLQLinear(nn.Module):
                                               w.data_ptr(), self.in_features, self.out_features, self.bits,
                                               self.group_size, stream)
         _lib.check(rc, "elutq_hlq_dequant_f16")
+        if self.sparse_count:
+            rc = _lib.lib().elutq_hlq_sparse_dequant_add_f16(
+                self.sparse_blocks.data_ptr(), self.sparse_scales.data_ptr(), self.sparse_index.data_ptr(),
+                self.sparse_count, w.data_ptr(), self.in_features, self.out_features, self.group_size, stream)
+            _lib.check(rc, "elutq_hlq_sparse_dequant_add_f16")
         return w
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, bits={self.bits}, "
-                f"group_size={self.group_size}, bias={self.bias is not None}")
+                f"group_size={self.group_size}, bias={self.bias is not None}"
+                + (f", sparse_blocks={self.sparse_count}" if self.sparse_count else ""))
 
 
 class GemvGroup:
@@ -226,6 +290,8 @@ class GemvGroup:
         for p, m, x, y in zip(arr, mods, xs, ys):
             if (m.bits, m.group_size) != (bits, group):
                 raise ValueError("all layers of a group must share bits and group size")
+            if m.sparse_count:
+                raise NotImplementedError("layers with a sparse extra plane cannot join a grouped launch")
             if x.dtype != torch.float16 or y.dtype != torch.float16 or x.numel() != m.in_features or y.numel() != m.out_features:
                 raise ValueError("inputs must be fp16 [K], outputs fp16 [N]")
             p.d_planes, p.d_scales, p.d_zeros = m.planes.data_ptr(), m.scales.data_ptr(), m.zeros.data_ptr()

@@ -59,6 +59,9 @@ def fuse_along_n(mods: list[HLQLinear]) -> HLQLinear:
         assert (m.in_features, m.bits, m.group_size) == (k, bits, group)
     for m in mods[:-1]:
         assert m.out_features % 64 == 0
+    if any(m.sparse_count for m in mods):
+        raise NotImplementedError("layers with a sparse extra plane cannot be concatenated: build the decoder "
+                                  "with fuse=False, impl='torch'")
     bias = None
     if any(m.bias is not None for m in mods):
         bias = torch.cat([m.bias if m.bias is not None else
@@ -258,6 +261,9 @@ class LlamaDecoder(nn.Module):
         self._graph = None
         self._buf = None
         if impl == "hip":
+            if any(m.sparse_count for m in self.modules() if isinstance(m, HLQLinear)):
+                raise NotImplementedError("the fused decode step has no sparse extra plane: build the decoder "
+                                          "with fuse=False, impl='torch'")
             ws = max(m.workspace_bytes for m in self.modules() if isinstance(m, HLQLinear))
             ws = max(ws, _lib.lib().elutq_decode_attn_workspace_bytes(s.n_heads, s.head_dim, 0))
             self._buf = FusedBuffers(s, ws, dev)

@@ -30,11 +30,15 @@ def repack_tree(src: str, dst: str, group_size: int | None = None, verbose: bool
         if "weight_config.json" in files:
             e = read_export_dir(cur, group_size)
             planes, scales, zeros = repack_export_arrays(e.w_quant, e.w_scale, e.w_zero, e.group)
-            write_repacked_dir(out, e.k, e.n, e.bits, e.group, planes, scales, zeros, e.bias)
+            if e.sparse is not None:
+                from .hlq_linear import sparse_index
+                sparse_index(e.sparse.mask, e.k, e.n, e.group)      # validates the block list
+            write_repacked_dir(out, e.k, e.n, e.bits, e.group, planes, scales, zeros, e.bias, e.sparse)
             count += 1
             dirs[:] = []
             if verbose:
-                print(f"{rel}: K={e.k} N={e.n} w{e.bits}g{e.group}", file=sys.stderr)
+                extra = f" + {e.sparse.mask.shape[0]} sparse blocks" if e.sparse is not None else ""
+                print(f"{rel}: K={e.k} N={e.n} w{e.bits}g{e.group}{extra}", file=sys.stderr)
             continue
         os.makedirs(out, exist_ok=True)
         for name in files:

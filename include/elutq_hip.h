@@ -18,6 +18,8 @@
  *                                                            C++/ops/src/arm/arm_gemm.cpp:312-360
  *   elutq_hlq_gemm_f16      arm_gemm(m  > 1, bit <= 4)        C++/ops/src/arm/arm_gemm.cpp:362-387
  *   elutq_hlq_dequant_f16   dequantize_with_scales            GPTQ/quant.py:176-183
+ *   elutq_hlq_sparse_*      arm_gemm(use_sparse)              C++/ops/src/arm/arm_gemm.cpp:683-868, 894-920
+ *                           t_mac_g4_float_update_sparse_impl C++/ops/src/arm/arm_t_mac_kernal.cpp:678-788
  *
  * Conventions
  *   - plain C types only; every `d_` pointer is DEVICE memory owned by the caller,
@@ -48,7 +50,8 @@ typedef enum elutq_status {
     ELUTQ_ERR_GROUP = -4,      /* group not 64 or 128 */
     ELUTQ_ERR_WORKSPACE = -5,  /* workspace smaller than elutq_hlq_workspace_bytes() */
     ELUTQ_ERR_HIP = -6,        /* a HIP runtime call failed (launch, attribute) */
-    ELUTQ_ERR_TUNING = -7      /* explicit ksplit / waves arguments out of range */
+    ELUTQ_ERR_TUNING = -7,     /* explicit ksplit / waves arguments out of range */
+    ELUTQ_ERR_SPARSE = -8      /* malformed block list of a sparse extra plane */
 } elutq_status;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -86,7 +89,8 @@ int elutq_hlq_workspace_init(void *d_workspace, size_t workspace_bytes, void *st
 
 /*
  * y[N] = W x + bias, batch 1.  d_x fp16 [K], d_y fp16 [N], d_bias fp16 [N] or NULL.
- * Replaces arm_gemm(m = 1, ...) for bit <= 4, use_sparse = false.
+ * Replaces arm_gemm(m = 1, ...) for bit <= 4, use_sparse = false (use_sparse:
+ * elutq_hlq_sparse_gemv_f16).
  */
 int elutq_hlq_gemv_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
                        const void *d_bias, const void *d_x, void *d_y,
@@ -220,6 +224,48 @@ int elutq_decode_argmax_f16(const void *d_logits, int n, void *d_token, void *d_
 /* W[N][K] fp16 row-major from the repacked buffers (dequantize_with_scales). */
 int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
                           void *d_w_out, int K, int N, int bits, int group, void *stream);
+
+/*
+ * Block-sparse extra plane (weight_config.json "use_sparse": true).  Such a layer has
+ * `base_bit` dense planes -- handled by the entry points above with bits = base_bit -- and
+ * one more plane that exists only on listed blocks of 32 output channels x `group` inputs,
+ * each block with 32 fp16 scales and no zero term.  As the reference's loader reads them
+ * (C++/ops/src/arm/parameters.cpp:19-64):
+ *   weight_mask.bin  uint32 pairs (channel start, k start), sparse_mask_len values, blocks of one
+ *                    channel start adjacent and channel starts ascending;
+ *   w_quant.bin      after the dense planes: block i as uint8 [32][group/8], LSB-first along K;
+ *   w_scale.bin      after the dense scales: block i as fp16 [32].
+ * The block bits and scales go to the device unchanged (no counterpart of
+ * t_mac_g4_rearrange_weight_sparse_impl, arm_t_mac_kernal.cpp:554-647, is needed);
+ * elutq_hlq_sparse_index_host turns the pair list into the index the kernels read
+ * (elutq_hlq_sparse_index_bytes(N, nblk) bytes, nblk = mask_len / 2; copy it to the device
+ * unchanged).  It rejects (ELUTQ_ERR_SPARSE) an odd mask_len, a channel start that is not a
+ * multiple of 32 or not below N, a k start that is not a multiple of 4 or with k + group > K,
+ * and descending channel starts.
+ *
+ * elutq_hlq_sparse_gemv_f16 / elutq_hlq_sparse_gemm_f16: the whole layer,
+ *   y[m][n] = dense part + sum over the blocks on n's tile of scale * sum_{k in block, bit set} x[m][k],
+ * as arm_gemm does for use_sparse (arm_gemm.cpp:894-920; the plane itself replaces
+ * t_mac_g4_float_update_sparse_impl as called from arm_gemm.cpp:779-790).  Two launches on
+ * `stream`: the plane's term in fp32 into the tail of the workspace, then the dense kernel, which
+ * adds it before its one rounding to fp16.  `bits` counts the dense planes (base_bit).  The
+ * workspace must hold elutq_hlq_sparse_workspace_bytes(K, N, bits, group, M) bytes, zero-filled
+ * once like every workspace.  elutq_hlq_sparse_dequant_add_f16: the plane added to a dense fp16
+ * W [N][K] (after elutq_hlq_dequant_f16; W is then rounded twice).
+ */
+size_t elutq_hlq_sparse_index_bytes(int N, int nblk);
+int elutq_hlq_sparse_index_host(const uint32_t *h_mask, int mask_len, int K, int N, int group, void *h_index_out);
+size_t elutq_hlq_sparse_workspace_bytes(int K, int N, int bits, int group, int M);
+int elutq_hlq_sparse_gemv_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                              const void *d_blocks, const void *d_blk_scales, const void *d_index, int nblk,
+                              const void *d_x, void *d_y, int K, int N, int bits, int group,
+                              void *d_workspace, size_t workspace_bytes, void *stream);
+int elutq_hlq_sparse_gemm_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                              const void *d_blocks, const void *d_blk_scales, const void *d_index, int nblk,
+                              const void *d_x, void *d_y, int M, int K, int N, int bits, int group,
+                              void *d_workspace, size_t workspace_bytes, void *stream);
+int elutq_hlq_sparse_dequant_add_f16(const void *d_blocks, const void *d_blk_scales, const void *d_index, int nblk,
+                                     void *d_w, int K, int N, int group, void *stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,179 @@
+"""GPU parity of layers with a block-sparse extra plane (use_sparse exports), through the C ABI.
+
+Same bars as the dense path: rel_err <= 1e-2 against the float64 oracle
+(max_i |y_i - ref_i| / max(|ref_i|, 0.05 rms(ref))), max|y - y_ref| <= 2e-2 rms against the
+restatement of the reference's all-fp16 chain, bit-exact where the arithmetic is exact.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from elutq_amd.export_io import SparseBlocks, write_export_dir
+from elutq_amd.hlq_linear import GemvGroup, HLQLinear
+from elutq_amd.repack import repack_tree
+from elutq_amd.synth import make_layer, make_sparse_plane, pack_bits_lsb_first
+from oracle import hlq_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def build(k, n, bits, group, density, seed, dev, m=1, bias=True):
+    L = make_layer(k, n, bits, group, m=m, seed=seed, bias=bias)
+    b, s, mk = make_sparse_plane(k, n, group, density, seed=seed + 100)
+    mod = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, group, L.bias, dev,
+                                       SparseBlocks(pack_bits_lsb_first(b), s, mk))
+    return L, O.SparsePlane(b, s, mk, group), mod
+
+
+def run(mod, x, dev):
+    y = mod(torch.from_numpy(np.ascontiguousarray(x)).to(dev))
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("k,n,bits,group,density", [
+    (256, 64, 2, 128, 0.5), (512, 128, 2, 128, 0.3), (1024, 256, 3, 64, 0.2), (1024, 192, 1, 64, 1.0),
+    (2048, 512, 2, 128, 0.05), (384, 96, 4, 128, 0.5),
+])
+def test_gemv_matches_oracle(cuda, lutref, k, n, bits, group, density):
+    L, sp, mod = build(k, n, bits, group, density, k + n, cuda)
+    print(f"sparse gemv K={k} N={n} w{bits}g{group} blocks={mod.sparse_count}", flush=True)
+    y = run(mod, L.x, cuda)[0]
+    ref = O.gemv_sparse_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, sp, L.bias)
+    assert y.shape == (n,) and y.dtype == np.float16
+    assert O.rel_err(y, ref) <= TOL
+    # the plane's fp32 term joins the dense fp32 sum before the one rounding to fp16
+    assert np.max(np.abs(y.astype(np.float64) - ref)) <= 2.0 ** -10 * max(1.0, np.max(np.abs(ref)))
+    wq, ws, mk = O.sparse_export_arrays(L.w_quant, L.w_scale, sp)
+    chain = lutref.RefSparseWeight(wq, ws, L.w_zero, mk, k, n, bits, group, L.bias).gemv(L.x[0], 2 if n % 64 == 0 else 1)
+    assert np.max(np.abs(y.astype(np.float64) - chain.astype(np.float64))) <= 2e-2 * np.sqrt(np.mean(ref ** 2))
+
+
+@pytest.mark.parametrize("m", [2, 5, 33, 64, 70])
+def test_gemm_matches_oracle_and_rows_equal_gemv(cuda, m):
+    k, n, group = 512, 192, 128
+    L, sp, mod = build(k, n, 2, group, 0.4, 7 + m, cuda, m=m)
+    print(f"sparse gemm M={m} blocks={mod.sparse_count}", flush=True)
+    y = run(mod, L.x, cuda)
+    w = O.dequantize_sparse(L.w_quant, L.w_scale, L.w_zero, sp)
+    ref = L.x.astype(np.float64) @ w.T + L.bias.astype(np.float64)
+    assert y.shape == (m, n)
+    assert O.rel_err(y, ref) <= TOL
+    # the reference defines m > 1 as one GEMV per row (arm_gemm.cpp:380-385)
+    y0 = run(mod, L.x[m - 1:m], cuda)[0]
+    assert np.max(np.abs(y[m - 1].astype(np.float64) - y0.astype(np.float64))) <= 2.0 ** -9 * max(1.0, np.max(np.abs(ref)))
+
+
+@pytest.mark.parametrize("group,m", [(128, 1), (64, 1), (128, 9)])
+def test_bit_exact_on_integer_inputs(cuda, group, m):
+    """Integer activations, power-of-two scales: every product and sum is exact in fp32 and the result
+    is representable in fp16, so the GPU must return the float64 result itself."""
+    k, n = 512, 128
+    r = np.random.default_rng(group + m)
+    wq = O.pack_planes(r.integers(0, 2, (2, n, k), dtype=np.uint8))
+    ws = np.stack([np.full((n, k // group), 0.5), np.full((n, k // group), 1.0)]).astype(np.float16)
+    wz = np.full((n, k // group), -0.5, np.float16)
+    b, _, mk = make_sparse_plane(k, n, group, 0.5, seed=group)
+    s = np.full((mk.shape[0], 32), 2.0, np.float16)
+    sp = O.SparsePlane(b, s, mk, group)
+    mod = HLQLinear.from_export_arrays(wq, ws, wz, group, None, cuda, SparseBlocks(sp.packed, s, mk))
+    x = r.integers(-2, 3, (m, k)).astype(np.float16)
+    y = run(mod, x, cuda)
+    want = x.astype(np.float64) @ O.dequantize_sparse(wq, ws, wz, sp).T
+    assert np.array_equal(y.astype(np.float64), want)
+
+
+def test_blocks_everywhere_equal_one_more_dense_plane(cuda):
+    """A sparse plane that lists every (tile, group) pair is a dense plane: both layers dequantize to
+    the same W and, on inputs where the arithmetic is exact, return the same bits."""
+    k, n, group = 512, 128, 128
+    L = make_layer(k, n, 3, group, seed=31)
+    bits = O.unpack_planes(L.w_quant)[2]
+    blk, sc, mk = [], [], []
+    for t in range(n // 32):
+        for g in range(k // group):
+            blk.append(bits[32 * t:32 * t + 32, group * g:group * g + group])
+            sc.append(L.w_scale[2, 32 * t:32 * t + 32, g])
+            mk.append((32 * t, group * g))
+    sp = SparseBlocks(pack_bits_lsb_first(np.stack(blk)), np.stack(sc), np.array(mk, np.uint32))
+    dense = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, group, None, cuda)
+    sparse = HLQLinear.from_export_arrays(L.w_quant[:2], L.w_scale[:2], L.w_zero, group, None, cuda, sp)
+    wd, wsp = dense.dequantize().float().cpu().numpy(), sparse.dequantize().float().cpu().numpy()
+    ref = O.dequantize(L.w_quant, L.w_scale, L.w_zero, group)
+    assert np.max(np.abs(wd - ref)) <= 2.0 ** -11 * np.max(np.abs(ref))
+    assert np.max(np.abs(wsp - ref)) <= 2.0 ** -9 * np.max(np.abs(ref))       # two roundings instead of one
+    yd, ys = run(dense, L.x, cuda)[0], run(sparse, L.x, cuda)[0]
+    want = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, group)
+    assert O.rel_err(yd, want) <= TOL and O.rel_err(ys, want) <= TOL
+
+
+def test_unaligned_and_overlapping_blocks(cuda):
+    """k starts need only be multiples of 4, and blocks may overlap or repeat: each adds its own term."""
+    k, n, group = 384, 64, 64
+    L = make_layer(k, n, 2, group, seed=41)
+    r = np.random.default_rng(42)
+    mk = np.array([[0, 4], [0, 36], [0, 36], [32, 316], [32, 0]], np.uint32)
+    b = r.integers(0, 2, (5, 32, group), dtype=np.uint8)
+    s = r.uniform(0.02, 0.08, (5, 32)).astype(np.float16)
+    sp = O.SparsePlane(b, s, mk, group)
+    mod = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, group, None, cuda, SparseBlocks(sp.packed, s, mk))
+    y = run(mod, L.x, cuda)[0]
+    assert O.rel_err(y, O.gemv_sparse_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, sp)) <= TOL
+    w = mod.dequantize().float().cpu().numpy()
+    ref = O.dequantize_sparse(L.w_quant, L.w_scale, L.w_zero, sp)
+    assert np.max(np.abs(w - ref)) <= 2.0 ** -9 * np.max(np.abs(ref))
+
+
+def test_ragged_n(cuda):
+    """N = 100: the block on channels 96..127 only contributes to channels 96..99."""
+    k, n, npad, group = 256, 100, 128, 128
+    L = make_layer(k, npad, 2, group, seed=51, bias=True)
+    b, s, mk = make_sparse_plane(k, npad, group, 1.0, seed=52)
+    sp = O.SparsePlane(b, s, mk, group)
+    mod = HLQLinear.from_export_arrays(L.w_quant[:, :n], L.w_scale[:, :n], L.w_zero[:n], group, L.bias[:n], cuda,
+                                       SparseBlocks(sp.packed, s, mk))
+    x = np.concatenate([L.x, -L.x, 0.5 * L.x])
+    y = run(mod, x, cuda)
+    ref = (x.astype(np.float64) @ O.dequantize_sparse(L.w_quant, L.w_scale, L.w_zero, sp).T + L.bias.astype(np.float64))[:, :n]
+    assert y.shape == (3, n) and O.rel_err(y, ref) <= TOL
+    assert O.rel_err(run(mod, L.x, cuda)[0], ref[0]) <= TOL
+
+
+def test_export_dir_and_repacked_dir_load_the_same_layer(cuda, tmp_path):
+    k, n, group = 512, 128, 128
+    L, sp, mod = build(k, n, 2, group, 0.3, 61, cuda)
+    src, dst = str(tmp_path / "src"), str(tmp_path / "dst")
+    d = os.path.join(src, "0", "mlp.gate_proj")
+    write_export_dir(d, L.w_quant, L.w_scale, L.w_zero, L.bias, sparse=SparseBlocks(sp.packed, sp.scale, sp.mask))
+    assert repack_tree(src, dst) == 1
+    y = run(mod, L.x, cuda)
+    for path in (d, os.path.join(dst, "0", "mlp.gate_proj")):
+        other = HLQLinear.from_export_dir(path, cuda)
+        assert other.sparse_count == mod.sparse_count and "sparse_blocks" in repr(other)
+        assert np.array_equal(run(other, L.x, cuda).view(np.uint16), y.view(np.uint16))
+
+
+def test_full_size_layer(cuda):
+    """q_proj of LLaMA-3-8B (4096 x 4096, w2g128) with a tenth of its blocks present."""
+    k = n = 4096
+    L, sp, mod = build(k, n, 2, 128, 0.1, 71, cuda, bias=False)
+    print(f"sparse gemv 4096x4096 blocks={mod.sparse_count}", flush=True)
+    y = run(mod, L.x, cuda)[0]
+    assert O.rel_err(y, O.gemv_sparse_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, sp)) <= TOL
+    y2 = run(mod, L.x, cuda)[0]
+    assert np.array_equal(y.view(np.uint16), y2.view(np.uint16))          # run-to-run determinism
+    ym = run(mod, -L.x, cuda)[0]
+    assert np.array_equal((-ym).view(np.uint16), y.view(np.uint16))       # y(-x) = -y(x) exactly
+
+
+def test_no_fused_or_grouped_launch_for_sparse_layers(cuda):
+    L, sp, mod = build(256, 64, 2, 128, 0.5, 81, cuda)
+    x = torch.from_numpy(L.x).to(cuda)
+    out = torch.empty(1, 64, dtype=torch.float16, device=cuda)
+    with pytest.raises(NotImplementedError):
+        mod.gemv_fused(x, out, torch.zeros(1 << 20, dtype=torch.uint8, device=cuda))
+    with pytest.raises(NotImplementedError):
+        GemvGroup([mod], [x], [out])
