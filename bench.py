@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-decode]
 
-Workload (BASELINE config 2): the LLaMA-3-8B layer-shape sweep at HLQ w2g128, batch 1.
+Workload: the LLaMA-3-8B layer-shape sweep at HLQ w2g128, batch 1.
 One "step" streams the seven projections (q, k, v, o, gate, up, down) of all 32 layers --
 224 GEMVs over 224 distinct random weight sets, 2.07 GB of packed planes + scales + zeros,
 far more than the 256 MB Infinity Cache, so every step reads its weights from HBM.  Inputs
@@ -126,7 +126,7 @@ MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
 
 
 def gemm_leg(torch, lib, dev, steps):
-    """BASELINE config 4: small-batch GEMM, HLQ w2g128, M in {16, 32, 64}, LLaMA-2-13B shapes;
+    """Small-batch GEMM, HLQ w2g128, M in {16, 32, 64}, LLaMA-2-13B shapes;
     each over a ring of weight sets > 400 MB.  Reports both roofline fractions (MFMA and HBM)."""
     from elutq_amd.synth import LLAMA2_13B_PREFILL_SHAPES, algorithmic_bytes, make_device_layer
     out = {}

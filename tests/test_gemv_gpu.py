@@ -150,7 +150,7 @@ def test_dequantize_matches_oracle(cuda):
 @pytest.mark.parametrize("name", ["q_proj", "k_proj", "gate_proj", "down_proj"])
 @pytest.mark.parametrize("bits,group", [(2, 128), (3, 128), (2, 64)])
 def test_llama3_8b_shapes_full_size(cuda, name, bits, group):
-    """BASELINE shapes at full size: oracle comparison plus size-independent properties."""
+    """The LLaMA-3-8B projection shapes at full size: oracle comparison plus size-independent properties."""
     k, n = LLAMA3_8B_SHAPES[name]
     L = make_layer(k, n, bits=bits, group=group, seed=7)
     m = to_mod(L, cuda)
