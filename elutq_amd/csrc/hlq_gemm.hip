@@ -192,19 +192,20 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
     // Two chunk buffers in LDS alternate: while the waves compute on one, the next chunk (its
     // global loads were issued a step earlier) is written to the other, and the loads of the
     // chunk after that are issued.  One barrier per step.
-    UnitData<BITS> cur, nxt;
+    UnitData<BITS> ua, ub;
     StageRegs<MT, KW> xr;
-    load_unit<BITS, G64>(cur, a, cbc, u_begin + kp, u_end, lane);
+    load_unit<BITS, G64>(ua, a, cbc, u_begin + kp, u_end, lane);
     stage_load<MT, KW>(xr, a, u_begin, u_end, tid);
     stage_store<MT, KW>(xr, (_Float16 *)smem, (float *)(smem + MROWS * ROW_HALFS * 2), tid);
     if (u_begin + KW < u_end) {
-        load_unit<BITS, G64>(nxt, a, cbc, u_begin + KW + kp, u_end, lane);
+        load_unit<BITS, G64>(ub, a, cbc, u_begin + KW + kp, u_end, lane);
         stage_load<MT, KW>(xr, a, u_begin + KW, u_end, tid);
     }
     __syncthreads();
 
-    int par = 0;
-    for (int u0 = u_begin; u0 < u_end; u0 += KW, par ^= 1) {
+    // One step: compute on `cur` (the unit of this step), then refill it with the unit two steps
+    // ahead; the caller alternates the two register sets, so no set is ever copied.
+    auto step = [&](UnitData<BITS> &cur, int u0, int par) __attribute__((always_inline)) {
         GEMM_STAMP(stamp_i); stamp_i++;
         const _Float16 *xl = (const _Float16 *)(smem + par * XBUF);
         const float *xs = (const float *)(smem + par * XBUF + MROWS * ROW_HALFS * 2);
@@ -311,11 +312,12 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
             }
         }
         GEMM_STAMP(stamp_i); stamp_i++;
-        if (u0 + KW < u_end) {
-            cur = nxt;
-            if (u0 + 2 * KW < u_end) load_unit<BITS, G64>(nxt, a, cbc, u0 + 2 * KW + kp, u_end, lane);
-        }
+        if (u0 + 2 * KW < u_end) load_unit<BITS, G64>(cur, a, cbc, u0 + 2 * KW + kp, u_end, lane);
         __syncthreads();
+    };
+    for (int u0 = u_begin; u0 < u_end; u0 += 2 * KW) {
+        step(ua, u0, 0);
+        if (u0 + KW < u_end) step(ub, u0 + KW, 1);
     }
 
     GEMM_STAMP(13);

@@ -6,14 +6,15 @@ import numpy as np
 
 from elutq_amd import export_io as io
 from elutq_amd.llama_decode import PROJ_DIRS, LlamaShape, proj_shapes
-from elutq_amd.synth import make_layer
+from elutq_amd.synth import make_layer, make_sparse_plane, pack_bits_lsb_first
 
 TINY = LlamaShape(n_layers=2, hidden=256, n_heads=2, n_kv_heads=1, ffn=384, vocab=300, max_seq=48, bits=2, group=128)
 
 
-def write_tiny_export(root: str, lm_head: str = "fp16", with_groupsize: bool = False) -> dict:
+def write_tiny_export(root: str, lm_head: str = "fp16", with_groupsize: bool = False, sparse_on=()) -> dict:
     """lm_head: 'fp16' (lm_head.bin), 'hlq' (lm_head/lm_head, 4-bit g128 as the reference exports it)
-    or 'tied' (shared_embed_lm_head.bin only).  Returns the arrays that were written."""
+    or 'tied' (shared_embed_lm_head.bin only).  Projections named in `sparse_on` get a block-sparse
+    extra plane on half of their blocks.  Returns the arrays that were written."""
     s = TINY
     r = np.random.default_rng(7)
     out = {"layers": []}
@@ -23,8 +24,12 @@ def write_tiny_export(root: str, lm_head: str = "fp16", with_groupsize: bool = F
         for name, (k, n) in proj_shapes(s).items():
             L = make_layer(k, n, bits=s.bits, group=s.group, seed=seed, bias=(name == "o_proj"))
             seed += 1
+            sp = None
+            if name in sparse_on:
+                b, sc, mk = make_sparse_plane(k, n, s.group, 0.5, seed=seed)
+                sp = io.SparseBlocks(pack_bits_lsb_first(b), sc, mk)
             io.write_export_dir(os.path.join(root, str(i), PROJ_DIRS[name]), L.w_quant, L.w_scale, L.w_zero, L.bias,
-                                groupsize=s.group if with_groupsize else None)
+                                groupsize=s.group if with_groupsize else None, sparse=sp)
             lay[name] = L
         for f in io.LAYER_NORMS:
             lay[f] = (1 + 0.1 * r.standard_normal(s.hidden)).astype(np.float16)
