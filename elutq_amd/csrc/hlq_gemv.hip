@@ -397,8 +397,12 @@ constexpr int depth_of(int bits) { return bits == 3 ? 6 : 4; }
 // built once; while a wave looks up its sub-tasks of one column block, each slot it has
 // consumed is refilled with the same sub-task of the next block, so the weight stream never
 // stops between blocks.  Needs runs of at most NSLOT sub-tasks per wave.
-// PLAIN: no prologue, no residual and no extra term (their fields of `a` are not read).
-template <int BITS, bool G64, int NSLOT, bool MULTI, bool PLAIN, bool PAIRED>
+// VAR: which optional inputs the instance reads, known when the kernel is compiled.
+//   GEMV_FUSED  prologue and residual as `a` says (the decode step's launches)
+//   GEMV_PLAIN  none of them (their fields of `a` are not read)
+//   GEMV_EXTRA  plain, plus the fp32 term `a.extra` added before the output is rounded
+enum { GEMV_FUSED = 0, GEMV_PLAIN = 1, GEMV_EXTRA = 2 };
+template <int BITS, bool G64, int NSLOT, bool MULTI, int VAR, bool PAIRED>
 __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, int ncb_run, unsigned char *smem, int &red_sel)
 {
     HLQ_STAMP_DECL;
@@ -406,9 +410,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     HLQ_STAMP(7);
     asm volatile("" ::: "memory");
 #endif
+    constexpr bool PLAIN = VAR != GEMV_FUSED;
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
-    const HLQ_GLOBAL float *extra = PLAIN ? nullptr : a.extra;
+    const HLQ_GLOBAL float *extra = VAR == GEMV_EXTRA ? a.extra : nullptr;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
@@ -603,12 +608,12 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     HLQ_STAMP_FLUSH;
 }
 
-template <int BITS, bool G64, int NSLOT, bool PAIRED, bool PLAIN>
+template <int BITS, bool G64, int NSLOT, bool PAIRED, int VAR>
 __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 {
     extern __shared__ __align__(256) unsigned char smem[];
     int sel = 0;
-    gemv_tile<BITS, G64, NSLOT, false, PLAIN, PAIRED>(a, blockIdx.y, blockIdx.x, 1, smem, sel);      // grid = (slices, column blocks)
+    gemv_tile<BITS, G64, NSLOT, false, VAR, PAIRED>(a, blockIdx.y, blockIdx.x, 1, smem, sel);      // grid = (slices, column blocks)
 }
 
 // One GEMV with more column blocks than the chip has CUs: every workgroup takes a run of
@@ -620,7 +625,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_run_kernel(const GemvArgs a, in
     extern __shared__ __align__(256) unsigned char smem[];
     const int cb0 = blockIdx.y * run;               // grid = (slices, runs of column blocks)
     int sel = 0;
-    gemv_tile<BITS, G64, NSLOT, true, PLAIN, PAIRED>(a, cb0, blockIdx.x, min(run, a.ncb - cb0), smem, sel);
+    gemv_tile<BITS, G64, NSLOT, true, PLAIN ? GEMV_PLAIN : GEMV_FUSED, PAIRED>(a, cb0, blockIdx.x, min(run, a.ncb - cb0), smem, sel);
 }
 
 // Many independent GEMVs in one launch: the tiles of all of them form one list that the
@@ -644,7 +649,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *__
     for (int i = blockIdx.x; i < n_items; i += gridDim.x) {
         const GroupItem it = items[i];
         const GemvArgs a = problems[it.problem];
-        gemv_tile<BITS, G64, NSLOT, true, true, PAIRED>(a, it.cb, it.slice, it.ncb_run, smem, sel);
+        gemv_tile<BITS, G64, NSLOT, true, GEMV_PLAIN, PAIRED>(a, it.cb, it.slice, it.ncb_run, smem, sel);
     }
 }
 
@@ -698,16 +703,16 @@ bool paired_ok(int spw, int ups, int ksplit)
     return MG::fits(NSLOT) && spw % MG::SIZE == 0 && (G64 || ksplit == 1 || ups % 2 == 0);
 }
 
-// PLAIN: no prologue, no residual and no extra term, known when the kernel is compiled
-template <int BITS, bool G64, int NSLOT, bool PAIRED, bool PLAIN>
+template <int BITS, bool G64, int NSLOT, bool PAIRED, int VAR>
 int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
-    auto kern = hlq_gemv_kernel<BITS, G64, NSLOT, PAIRED, PLAIN>;
+    constexpr bool PLAIN = VAR == GEMV_PLAIN;
+    auto kern = hlq_gemv_kernel<BITS, G64, NSLOT, PAIRED, VAR>;
     static bool big_lds_done[64] = {};        // per template instance
     if (!allow_big_lds((const void *)kern, lds, MAX_LDS, big_lds_done)) return ELUTQ_ERR_HIP;
     // more tiles than CUs and runs that fit the slots: runs of column blocks, one workgroup per CU
     const int run = (a.ncb * a.ksplit + NUM_CU_RUN - 1) / NUM_CU_RUN;
-    if (run > 1 && a.spw <= NSLOT && waves == 16) {
+    if (VAR != GEMV_EXTRA && run > 1 && a.spw <= NSLOT && waves == 16) {       // (the extra term has no run instances)
         auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT, PAIRED, PLAIN>;
         static bool big_lds_run_done[64] = {};
         if (!allow_big_lds((const void *)kern_run, lds, MAX_LDS, big_lds_run_done)) return ELUTQ_ERR_HIP;
@@ -722,8 +727,12 @@ int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 template <int BITS, bool G64, int NSLOT, bool PAIRED>
 int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
-    if (a.prologue == 0 && !a.residual && !a.extra) return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, true>(a, waves, lds, stream);
-    return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, false>(a, waves, lds, stream);
+    if (a.extra) {
+        if (a.prologue != 0 || a.residual) return ELUTQ_ERR_TUNING;     // no instance reads both
+        return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_EXTRA>(a, waves, lds, stream);
+    }
+    if (a.prologue == 0 && !a.residual) return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_PLAIN>(a, waves, lds, stream);
+    return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_FUSED>(a, waves, lds, stream);
 }
 
 template <int BITS, bool G64, int NSLOT>
