@@ -39,7 +39,7 @@ struct GemmArgs {
     const uint16_t *x;      // fp16 [M][K]
     uint16_t *y;            // fp16 [M][N]
     const float *extra;     // fp32 [M][N] added to the output before it is rounded, or null
-    float *partial;         // [ksplit][MT*32][ncb*64]
+    float *partial;         // [ksplit][MR][ncb*64]
     unsigned *counters;     // one per workgroup column (super block)
     int M, N, K, U, NT, ncb;
     int ksplit, ups;        // K slices per super block, units per slice (multiple of KW)
@@ -70,23 +70,24 @@ __device__ __forceinline__ float dpp_f(float v)
 // at 8s are the A operand of MFMA step s and pair q = (k, k + 16) lines up with what one
 // shift extracts from a plane dword.  One task = one such 16-byte slot of one row, built
 // from two 8-byte loads (k = 4s..4s+3 and k + 16); consecutive lanes write consecutive
-// slots, so the LDS stores are conflict-free.  xs[(ul*2 + half) * MT*32 + m] receives the
-// fp32 sum of x[m] over 64-k half `half` of unit ul (eight consecutive lanes).
-template <int MT, int KW>
+// slots, so the LDS stores are conflict-free.  xs[(ul*2 + half) * MR + m] receives the
+// fp32 sum of x[m] over 64-k half `half` of unit ul (eight consecutive lanes).  MR = rows staged
+// (16, 32 or 64).
+template <int MR, int KW>
 struct StageRegs {
     static constexpr int SLOTS = KW * 16;                            // 16-byte slots per row
-    static constexpr int TASKS = MT * 32 * SLOTS;
+    static constexpr int TASKS = MR * SLOTS;
     static constexpr int TPT = TASKS / GEMM_THREADS;
     static_assert(TASKS % GEMM_THREADS == 0, "whole waves of staging tasks");
     uint2 lo[TPT], hi[TPT];
 };
 
-template <int MT, int KW>
-__device__ __forceinline__ void stage_load(StageRegs<MT, KW> &r, const GemmArgs &a, int u0, int u_end, int tid)
+template <int MR, int KW>
+__device__ __forceinline__ void stage_load(StageRegs<MR, KW> &r, const GemmArgs &a, int u0, int u_end, int tid)
 {
-    constexpr int SLOTS = StageRegs<MT, KW>::SLOTS;
+    constexpr int SLOTS = StageRegs<MR, KW>::SLOTS;
 #pragma unroll
-    for (int t = 0; t < StageRegs<MT, KW>::TPT; t++) {
+    for (int t = 0; t < StageRegs<MR, KW>::TPT; t++) {
         const int idx = tid + t * GEMM_THREADS;
         const int m = idx / SLOTS, o = idx % SLOTS, ul = o >> 4, blk = (o >> 2) & 3, sq = o & 3;
         const int mm = m < a.M ? m : a.M - 1, uu = u0 + ul < u_end ? u0 + ul : u_end - 1;
@@ -96,14 +97,14 @@ __device__ __forceinline__ void stage_load(StageRegs<MT, KW> &r, const GemmArgs 
     }
 }
 
-template <int MT, int KW>
-__device__ __forceinline__ void stage_store(const StageRegs<MT, KW> &r, _Float16 *xl, float *xs, int tid)
+template <int MR, int KW>
+__device__ __forceinline__ void stage_store(const StageRegs<MR, KW> &r, _Float16 *xl, float *xs, int tid)
 {
-    constexpr int SLOTS = StageRegs<MT, KW>::SLOTS;
+    constexpr int SLOTS = StageRegs<MR, KW>::SLOTS;
     constexpr int ROW_HALFS = KW * HLQ_UNIT + 8;
     const half2v ones = {(_Float16)1.f, (_Float16)1.f};
 #pragma unroll
-    for (int t = 0; t < StageRegs<MT, KW>::TPT; t++) {
+    for (int t = 0; t < StageRegs<MR, KW>::TPT; t++) {
         const int idx = tid + t * GEMM_THREADS;
         const int m = idx / SLOTS, o = idx % SLOTS;
         float sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.lo[t].x), ones, 0.f, false);
@@ -113,7 +114,7 @@ __device__ __forceinline__ void stage_store(const StageRegs<MT, KW> &r, _Float16
         sum += dpp_f<0xB1>(sum);                 // lanes of a quad: the four slots of a 32-k block
         sum += dpp_f<0x4E>(sum);
         sum += dpp_f<0x141>(sum);                // the other 32-k block of the same 64-k half
-        if ((o & 7) == 0) xs[(o >> 3) * (MT * 32) + m] = sum;
+        if ((o & 7) == 0) xs[(o >> 3) * MR + m] = sum;
         uint4 v;
         v.x = __builtin_amdgcn_perm(r.hi[t].x, r.lo[t].x, 0x05040100u);
         v.y = __builtin_amdgcn_perm(r.hi[t].x, r.lo[t].x, 0x07060302u);
@@ -158,15 +159,20 @@ __device__ __forceinline__ float h2f(uint32_t v, bool hi)
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(hi ? v >> 16 : v & 0xffffu));
 }
 
-template <int BITS, bool G64, int MT, int KW>
+// MR = activation rows of the launch, rounded up to 16, 32 or 64.  The MFMA tile has 32 rows; with
+// MR = 16 only rows 0..15 are staged (lanes of rows 16..31 read rows 0..15 again) and only the
+// accumulator registers of those rows (0..7 of 16) are reduced and stored.
+template <int BITS, bool G64, int MR, int KW>
 __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a)
 {
+    constexpr int MT = (MR + 31) / 32;              // 32-row MFMA tiles
+    constexpr int REGS = MR == 16 ? 8 : 16;         // accumulator registers per tile that hold real rows
     extern __shared__ __align__(256) unsigned char smem[];
     constexpr int CBW = GW / KW;                    // column blocks per workgroup
     constexpr int ROW_HALFS = KW * HLQ_UNIT + 8;    // 16 B pad: conflict-free b128 reads
     constexpr int TILES = MT * 2;
-    constexpr int VALS = TILES * 16 * 64;           // fp32 results per wave
-    constexpr int MROWS = MT * 32;
+    constexpr int VALS = TILES * REGS * 64;         // fp32 results per wave
+    constexpr int MROWS = MR;
     constexpr int XBUF = MROWS * ROW_HALFS * 2 + KW * 2 * MROWS * 4;    // bytes of one staged chunk: x, then row sums
     float *red = (float *)smem;                     // reused after the last step
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -193,13 +199,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
     // global loads were issued a step earlier) is written to the other, and the loads of the
     // chunk after that are issued.  One barrier per step.
     UnitData<BITS> ua, ub;
-    StageRegs<MT, KW> xr;
+    StageRegs<MR, KW> xr;
     load_unit<BITS, G64>(ua, a, cbc, u_begin + kp, u_end, lane);
-    stage_load<MT, KW>(xr, a, u_begin, u_end, tid);
-    stage_store<MT, KW>(xr, (_Float16 *)smem, (float *)(smem + MROWS * ROW_HALFS * 2), tid);
+    stage_load<MR, KW>(xr, a, u_begin, u_end, tid);
+    stage_store<MR, KW>(xr, (_Float16 *)smem, (float *)(smem + MROWS * ROW_HALFS * 2), tid);
     if (u_begin + KW < u_end) {
         load_unit<BITS, G64>(ub, a, cbc, u_begin + KW + kp, u_end, lane);
-        stage_load<MT, KW>(xr, a, u_begin + KW, u_end, tid);
+        stage_load<MR, KW>(xr, a, u_begin + KW, u_end, tid);
     }
     __syncthreads();
 
@@ -211,8 +217,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
         const float *xs = (const float *)(smem + par * XBUF + MROWS * ROW_HALFS * 2);
         if (u0 + KW < u_end) {
             unsigned char *nb = smem + (par ^ 1) * XBUF;
-            stage_store<MT, KW>(xr, (_Float16 *)nb, (float *)(nb + MROWS * ROW_HALFS * 2), tid);
-            if (u0 + 2 * KW < u_end) stage_load<MT, KW>(xr, a, u0 + 2 * KW, u_end, tid);
+            stage_store<MR, KW>(xr, (_Float16 *)nb, (float *)(nb + MROWS * ROW_HALFS * 2), tid);
+            if (u0 + 2 * KW < u_end) stage_load<MR, KW>(xr, a, u0 + 2 * KW, u_end, tid);
         }
         GEMM_STAMP(stamp_i); stamp_i++;
         const int u = u0 + kp;
@@ -229,7 +235,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
             split_tiles(cur.zz, cur.zz, zzj[0], zzj[1]);
             // A operands are read two MFMA steps ahead of their use (three rotating registers sets);
             // scheduling barriers between the steps keep the compiler from sinking the reads
-            const _Float16 *arow = xl + (size_t)col * ROW_HALFS + kp * HLQ_UNIT + h * 32;
+            const _Float16 *arow = xl + (size_t)(MR == 16 ? (col & 15) : col) * ROW_HALFS + kp * HLQ_UNIT + h * 32;
             half8 aop[3][MT];
 #pragma unroll
             for (int st = 0; st < 2; st++)
@@ -293,7 +299,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-                        for (int i4 = 0; i4 < 4; i4++) {
+                        for (int i4 = 0; i4 < REGS / 4; i4++) {
                             const int m0 = mt * 32 + 8 * i4 + 4 * h;
                             float4 sx = *(const float4 *)(xs + (kp * 2 + pr) * MROWS + m0);
                             if (!G64) {
@@ -328,17 +334,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) red[((wave * TILES + mt * 2 + j) * 16 + i) * 64 + lane] = acc[mt][j][i];
+            for (int i = 0; i < REGS; i++) red[((wave * TILES + mt * 2 + j) * REGS + i) * 64 + lane] = acc[mt][j][i];
     __syncthreads();
 
     constexpr int NV = CBW * VALS / GEMM_THREADS;    // results per thread
     const size_t npad = (size_t)a.ncb * HLQ_CB;
-    const int mpad = MT * 32;
+    const int mpad = MROWS;
     // value v = (column block, tile, reg, lane); C layout of the 32x32 MFMA: column = lane % 32,
     // row = 8 * (reg / 4) + 4 * (lane / 32) + reg % 4.
     auto decode = [&](int v, int &m, int &n) {
         const int c = v / VALS, r = v % VALS;
-        const int ln = r & 63, reg = (r >> 6) & 15, tile = r >> 10;
+        const int ln = r & 63, reg = (r >> 6) % REGS, tile = r / (64 * REGS);
         const int mt = tile >> 1, j = tile & 1;
         m = mt * 32 + 8 * (reg >> 2) + 4 * (ln >> 5) + (reg & 3);
         n = (sb * CBW + c) * HLQ_CB + j * 32 + (ln & 31);
@@ -441,19 +447,20 @@ inline bool allow_big_lds(const void *kern, size_t lds, int limit, bool (&done)[
     return true;
 }
 
-template <int MT, int KW>
+template <int MR, int KW>
 size_t gemm_lds_bytes()
 {
-    const size_t x = 2 * ((size_t)MT * 32 * (KW * HLQ_UNIT + 8) * 2 + (size_t)KW * 2 * MT * 32 * sizeof(float));
-    const size_t r = (size_t)GW * MT * 2 * 16 * 64 * 4;
+    constexpr int MT = (MR + 31) / 32, REGS = MR == 16 ? 8 : 16;
+    const size_t x = 2 * ((size_t)MR * (KW * HLQ_UNIT + 8) * 2 + (size_t)KW * 2 * MR * sizeof(float));
+    const size_t r = (size_t)GW * MT * 2 * REGS * 64 * 4;
     return (x > r ? x : r) + 256;
 }
 
-template <int BITS, bool G64, int MT, int KW>
+template <int BITS, bool G64, int MR, int KW>
 int launch_gemm(const GemmArgs &a, hipStream_t stream)
 {
-    auto kern = hlq_gemm_kernel<BITS, G64, MT, KW>;
-    const size_t lds = gemm_lds_bytes<MT, KW>();
+    auto kern = hlq_gemm_kernel<BITS, G64, MR, KW>;
+    const size_t lds = gemm_lds_bytes<MR, KW>();
     static bool big_lds_done[64] = {};        // per template instance
     if (!allow_big_lds((const void *)kern, lds, (int)lds, big_lds_done)) return ELUTQ_ERR_HIP;
     const int cbw = GW / KW, nsb = (a.ncb + cbw - 1) / cbw;
@@ -461,12 +468,12 @@ int launch_gemm(const GemmArgs &a, hipStream_t stream)
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
 
-template <int BITS, bool G64, int MT>
+template <int BITS, bool G64, int MR>
 int launch_gemm_kw(const GemmArgs &a, int kw, hipStream_t stream)
 {
     switch (kw) {
-    case 2: return launch_gemm<BITS, G64, MT, 2>(a, stream);
-    case 4: return launch_gemm<BITS, G64, MT, 4>(a, stream);
+    case 2: return launch_gemm<BITS, G64, MR, 2>(a, stream);
+    case 4: return launch_gemm<BITS, G64, MR, 4>(a, stream);
     }
     return ELUTQ_ERR_TUNING;
 }
@@ -474,7 +481,8 @@ int launch_gemm_kw(const GemmArgs &a, int kw, hipStream_t stream)
 template <int BITS, bool G64>
 int launch_gemm_mt(const GemmArgs &a, int kw, hipStream_t stream)
 {
-    return a.M <= 32 ? launch_gemm_kw<BITS, G64, 1>(a, kw, stream) : launch_gemm_kw<BITS, G64, 2>(a, kw, stream);
+    if (a.M <= 16) return launch_gemm_kw<BITS, G64, 16>(a, kw, stream);
+    return a.M <= 32 ? launch_gemm_kw<BITS, G64, 32>(a, kw, stream) : launch_gemm_kw<BITS, G64, 64>(a, kw, stream);
 }
 
 int dispatch_gemm(const GemmArgs &a, int bits, bool g64, int kw, hipStream_t stream)
