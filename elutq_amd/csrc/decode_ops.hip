@@ -202,8 +202,8 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     __shared__ float sm_o[WAVES][D];
     __shared__ unsigned s_ticket;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int S = a.splits;
-    const int h = blockIdx.x / S, sp = blockIdx.x - h * S, grp = a.nq / a.nkv, g = h / grp;
+    const int SL = a.splits;                             // splits launched; S below = splits that take part
+    const int h = blockIdx.x / SL, sp = blockIdx.x - h * SL, grp = a.nq / a.nkv, g = h / grp;
     const int seg = lane & 15, r = lane >> 4;
 
     // Everything the kernel needs from memory first is requested before anything is waited for:
@@ -229,6 +229,13 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     asm volatile("" ::: "memory");
     const int pos = (int)pos64;
     if (pos64 < 0 || pos64 >= a.max_seq) return;
+    // No more splits than blocks of cached rows, and a context of at most SHORT_BLOCKS blocks is one
+    // workgroup's work: meeting in device memory would cost more than the other workgroups save.
+    // Every workgroup of the head derives the same S from *pos; those beyond it leave at once.
+    constexpr int SHORT_BLOCKS = 3;
+    const int nblocks = (pos + BLOCK_ROWS - 1) / BLOCK_ROWS;
+    const int S = nblocks <= SHORT_BLOCKS ? 1 : min(SL, nblocks);
+    if (sp >= S) return;
     ATTN_STAMP(1);
 
     if (tid < HALF) {                                    // rotary pair (tid, tid + 64) of q and of the new k
@@ -345,7 +352,7 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
         ATTN_STAMP(14);
         return;
     }
-    float *po = a.partial + ((size_t)h * S + sp) * (D + 2);
+    float *po = a.partial + ((size_t)h * SL + sp) * (D + 2);
     if (tid < D) __hip_atomic_store(&po[tid], o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (tid == 0) {
         __hip_atomic_store(&po[D], M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -361,7 +368,7 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
         float pm[ATTN_MAX_SPLITS], pl[ATTN_MAX_SPLITS], pv[ATTN_MAX_SPLITS];
 #pragma unroll
         for (int s = 0; s < ATTN_MAX_SPLITS; s++) {
-            const float *ps = a.partial + ((size_t)h * S + min(s, S - 1)) * (D + 2);
+            const float *ps = a.partial + ((size_t)h * SL + min(s, S - 1)) * (D + 2);
             pv[s] = __hip_atomic_load(&ps[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             pm[s] = __hip_atomic_load(&ps[D], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             pl[s] = __hip_atomic_load(&ps[D + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
