@@ -229,12 +229,14 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     asm volatile("" ::: "memory");
     const int pos = (int)pos64;
     if (pos64 < 0 || pos64 >= a.max_seq) return;
-    // No more splits than blocks of cached rows, and a context of at most SHORT_BLOCKS blocks is one
-    // workgroup's work: meeting in device memory would cost more than the other workgroups save.
-    // Every workgroup of the head derives the same S from *pos; those beyond it leave at once.
+    // How many of the launched workgroups take part follows the context: meeting in device memory
+    // costs about 2 us plus 0.1-0.2 us per partial result, a further 64-row block about 0.6 us.  So a
+    // context of at most SHORT_BLOCKS blocks is one workgroup's work, up to 12 blocks are shared by
+    // at most four, longer contexts by all.  Every workgroup of the head derives the same S from
+    // *pos; those beyond it leave at once.
     constexpr int SHORT_BLOCKS = 3;
     const int nblocks = (pos + BLOCK_ROWS - 1) / BLOCK_ROWS;
-    const int S = nblocks <= SHORT_BLOCKS ? 1 : min(SL, nblocks);
+    const int S = nblocks <= SHORT_BLOCKS ? 1 : min(SL, nblocks <= 12 ? min(nblocks, 4) : ATTN_MAX_SPLITS);
     if (sp >= S) return;
     ATTN_STAMP(1);
 

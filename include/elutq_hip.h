@@ -203,8 +203,8 @@ int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, void *d_v_cac
  * GEMV workspace, which it may share: calls on one stream leave its counters at zero).  One
  * compute unit takes in a cache of a few hundred rows no faster than the whole chip takes in
  * all heads', so long contexts want the split.  The workgroups of a head read *d_pos and take
- * part only as far as the context has 64-row blocks for them (a context of up to 192 positions is
- * one workgroup's work), so short contexts do not pay for the meeting.  head_dim other than 128
+ * part only as far as the context warrants (up to 192 positions: one workgroup; up to 768: at most
+ * four; beyond: all), so short contexts do not pay for the meeting.  head_dim other than 128
  * runs unsplit.
  * No counterpart in the reference beyond the operators elutq_decode_rope_attn_f16 replaces.
  */
