@@ -104,7 +104,7 @@ def test_graph_replay_equals_eager(cuda, impl):
 
 @pytest.mark.parametrize("d,nq,nkv,splits", [(128, 8, 2, 1), (128, 4, 4, 1), (64, 8, 2, 1), (32, 4, 1, 1),
                                              (128, 8, 2, 2), (128, 8, 2, 8), (128, 32, 8, 0), (128, 4, 4, 3), (64, 8, 2, 4)])
-@pytest.mark.parametrize("pos", [0, 1, 3, 4, 5, 37, 63, 64, 65, 255, 300, 513, 1030])
+@pytest.mark.parametrize("pos", [0, 1, 3, 4, 5, 37, 63, 64, 65, 192, 193, 255, 300, 513, 768, 769, 1030])
 def test_rope_cache_attention_kernel(cuda, d, nq, nkv, splits, pos):
     """elutq_decode_rope_attn_f16 / _split_f16 (cached positions divided among `splits`
     workgroups per head, 0 = default) against the PyTorch restatement of the reference ops
