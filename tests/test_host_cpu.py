@@ -130,3 +130,13 @@ def test_algorithmic_bytes_table():
     assert algorithmic_bytes(14336, 4096, 2, 128) == 17_469_440
     assert algorithmic_bytes(4096, 4096, 3, 128) == 7_356_416
     assert algorithmic_bytes(4096, 4096, 2, 64) == 5_783_552
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The path needs no collective and every figure is for one GPU: `bench.py --gpus N`, N > 1, says so
+    and exits with status 2 before it touches a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout == ""
