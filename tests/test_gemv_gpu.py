@@ -162,3 +162,27 @@ def test_llama3_8b_shapes_full_size(cuda, name, bits, group):
     # y(x) + y(-x) == 0 exactly (integer tables negate exactly, fp32 sums are sign symmetric)
     yn = run(m, (-L.x).astype(np.float16), cuda)[0]
     assert np.array_equal(yn.view(np.uint16) ^ 0x8000, y.view(np.uint16)) or np.array_equal(-yn, y)
+
+
+@pytest.mark.parametrize("n", [28672, 128256])
+def test_widest_layers_sampled_columns(cuda, n):
+    """The widest layers of the decode step -- gate|up concatenated (4096 x 28672) and an lm_head-sized layer
+    (4096 x 128256), which run as column-block runs of one workgroup each: 4096 sampled columns against the
+    float64 oracle evaluated on those columns only, plus the size-independent properties."""
+    k, bits, group = 4096, 2, 128
+    L = make_layer(k, n, bits=bits, group=group, seed=11)
+    m = to_mod(L, cuda)
+    print(f"widest layer K={k} N={n}", flush=True)
+    y = run(m, L.x, cuda)[0]
+    idx = np.sort(np.random.default_rng(n).choice(n, 4096, replace=False))
+    idx[:3], idx[-3:] = (0, 1, 63), (n - 64, n - 2, n - 1)            # block edges, first and last
+    ref = O.gemv_f64(L.x[0], L.w_quant[:, idx], L.w_scale[:, idx], L.w_zero[idx], group)
+    assert O.rel_err(y[idx], ref) <= TOL
+    assert np.max(np.abs(y[idx].astype(np.float64) - ref)) <= 2.0 ** -10 * max(1.0, np.max(np.abs(ref)))
+    assert np.array_equal(y, run(m, L.x, cuda)[0])
+    yn = run(m, (-L.x).astype(np.float16), cuda)[0]
+    assert np.array_equal(-yn, y)
+    # a column slice of the layer is a layer of its own: the same columns, the same bits
+    sub = HLQLinear.from_export_arrays(L.w_quant[:, 4096:8192], L.w_scale[:, 4096:8192], L.w_zero[4096:8192], group, None, cuda)
+    ys = run(sub, L.x, cuda)[0]
+    assert np.max(np.abs(ys.astype(np.float64) - y[4096:8192].astype(np.float64))) <= 2.0 ** -10 * max(1.0, np.max(np.abs(ref)))
