@@ -379,9 +379,11 @@ __device__ __forceinline__ void static_for(F &&f)
     }
 }
 
-// Sub-tasks a wave keeps in flight at most.  Three planes get six slots: a unit pair (one meta
-// group at G = 128) is six sub-tasks, and K = 4096 gives a wave exactly that run.
-constexpr int depth_of(int bits) { return bits == 3 ? 6 : 4; }
+// Sub-tasks a wave keeps in flight at most.  Three planes get six slots and four planes eight: a
+// unit pair (one meta group at G = 128) is that many sub-tasks, and K = 4096 gives a wave exactly
+// that run -- so a layer with more column blocks than CUs can run as column-block runs (which need
+// the whole run in slots) without slicing K.
+constexpr int depth_of(int bits) { return bits == 3 ? 6 : (bits == 4 ? 8 : 4); }
 
 // One workgroup = one column block x one K slice.  Its (unit, plane) sub-tasks are dealt to
 // the waves in contiguous runs of `spw`; every wave builds the activation tables of the
@@ -755,9 +757,13 @@ int launch_gemv(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
     case 3: return launch_gemv_n<BITS, G64, 3>(a, waves, lds, stream);
     case 4: return launch_gemv_n<BITS, G64, 4>(a, waves, lds, stream);
     default:
-        if constexpr (DEPTH == 6) {
+        if constexpr (DEPTH >= 6) {
             if (a.spw == 5) return launch_gemv_n<BITS, G64, 5>(a, waves, lds, stream);
-            return launch_gemv_n<BITS, G64, 6>(a, waves, lds, stream);
+            if (a.spw == 6 || DEPTH == 6) return launch_gemv_n<BITS, G64, 6>(a, waves, lds, stream);
+        }
+        if constexpr (DEPTH == 8) {
+            if (a.spw == 7) return launch_gemv_n<BITS, G64, 7>(a, waves, lds, stream);
+            return launch_gemv_n<BITS, G64, 8>(a, waves, lds, stream);
         }
         return launch_gemv_n<BITS, G64, 4>(a, waves, lds, stream);
     }
@@ -813,9 +819,13 @@ int launch_group(int nslot, bool paired, const GemvArgs *p, const GroupItem *it,
     case 3: return launch_group_n<BITS, G64, 3>(paired, p, it, n, grid, waves, lds, st);
     case 4: return launch_group_n<BITS, G64, 4>(paired, p, it, n, grid, waves, lds, st);
     default:
-        if constexpr (depth_of(BITS) == 6) {
+        if constexpr (depth_of(BITS) >= 6) {
             if (nslot == 5) return launch_group_n<BITS, G64, 5>(paired, p, it, n, grid, waves, lds, st);
-            return launch_group_n<BITS, G64, 6>(paired, p, it, n, grid, waves, lds, st);
+            if (nslot == 6 || depth_of(BITS) == 6) return launch_group_n<BITS, G64, 6>(paired, p, it, n, grid, waves, lds, st);
+        }
+        if constexpr (depth_of(BITS) == 8) {
+            if (nslot == 7) return launch_group_n<BITS, G64, 7>(paired, p, it, n, grid, waves, lds, st);
+            return launch_group_n<BITS, G64, 8>(paired, p, it, n, grid, waves, lds, st);
         }
         return launch_group_n<BITS, G64, 4>(paired, p, it, n, grid, waves, lds, st);
     }
