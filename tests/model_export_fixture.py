@@ -12,7 +12,8 @@ TINY = LlamaShape(n_layers=2, hidden=256, n_heads=2, n_kv_heads=1, ffn=384, voca
 
 
 def write_tiny_export(root: str, lm_head: str = "fp16", with_groupsize: bool = False, sparse_on=()) -> dict:
-    """lm_head: 'fp16' (lm_head.bin), 'hlq' (lm_head/lm_head, 4-bit g128 as the reference exports it)
+    """lm_head: 'fp16' (lm_head.bin), 'hlq' (lm_head/lm_head: the reference quantizes the lm_head like any other layer unless
+    told to skip it, GPTQ/llama.py:143-176; 4 bits here, so that one tree holds two formats)
     or 'tied' (shared_embed_lm_head.bin only).  Projections named in `sparse_on` get a block-sparse
     extra plane on half of their blocks.  Returns the arrays that were written."""
     s = TINY
