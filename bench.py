@@ -251,7 +251,8 @@ def main():
     torch.cuda.set_device(dev)
     if a.mode == "decode":
         from elutq_amd.llama_decode import bench_decode
-        print(json.dumps({"mode": "decode", "decode": bench_decode(dev)}))
+        print(json.dumps({"mode": "decode", "decode": bench_decode(dev),
+                          "decode_hlq_lm_head": bench_decode(dev, hlq_lm_head=True)}))
         return
     if a.mode == "gemm":
         print(json.dumps({"mode": "gemm", "gemm_w2g128_llama2_13b": gemm_leg(torch, lib, dev, a.steps)}))
@@ -440,6 +441,11 @@ def main():
         try:
             from elutq_amd.llama_decode import bench_decode
             out["decode"] = bench_decode(dev)
+            # the same model with the lm_head quantized like every other layer, which is what the
+            # reference's exporter writes unless it is told to skip the lm_head (extra information:
+            # the workload of the headline decode figure keeps the fp16 lm_head)
+            torch.cuda.empty_cache()
+            out["decode_hlq_lm_head"] = bench_decode(dev, hlq_lm_head=True)
         except ImportError:
             out["decode"] = None
 

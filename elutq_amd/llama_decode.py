@@ -175,8 +175,10 @@ def proj_shapes(s: LlamaShape) -> dict:
             "gate_proj": (s.hidden, s.ffn), "up_proj": (s.hidden, s.ffn), "down_proj": (s.ffn, s.hidden)}
 
 
-def random_parts(s: LlamaShape, dev, seed: int) -> dict:
-    """Random-init weights of the shape (generated on the device)."""
+def random_parts(s: LlamaShape, dev, seed: int, hlq_lm_head: bool = False) -> dict:
+    """Random-init weights of the shape (generated on the device).  `hlq_lm_head`: the lm_head is an HLQ
+    layer of the model's bits and group size -- what the reference's exporter produces unless told to
+    skip the lm_head (GPTQ/llama.py:143-176) -- instead of an fp16 matrix."""
     g = torch.Generator(device=dev).manual_seed(seed)
     layers = []
     sd = seed * 100_003
@@ -188,7 +190,10 @@ def random_parts(s: LlamaShape, dev, seed: int) -> dict:
         norms = tuple((1.0 + 0.1 * torch.randn(s.hidden, generator=g, device=dev)).to(torch.float16) for _ in range(2))
         layers.append((lin, norms))
     embed = (torch.randn(s.vocab, s.hidden, generator=g, device=dev) * 0.5).to(torch.float16)
-    lm_head = (torch.randn(s.vocab, s.hidden, generator=g, device=dev) * 0.02).to(torch.float16)
+    if hlq_lm_head:
+        lm_head = make_device_layer(s.hidden, s.vocab, s.bits, s.group, seed=sd, device=dev)
+    else:
+        lm_head = (torch.randn(s.vocab, s.hidden, generator=g, device=dev) * 0.02).to(torch.float16)
     norm = (1.0 + 0.1 * torch.randn(s.hidden, generator=g, device=dev)).to(torch.float16)
     return {"layers": layers, "embed": embed, "lm_head": lm_head, "norm": norm}
 
@@ -303,11 +308,12 @@ class LlamaDecoder(nn.Module):
                 x = layer(x, self.pos, cos, sin, mask)
         if self.impl == "hip":
             L, stream = _lib.lib(), torch.cuda.current_stream().cuda_stream
-            _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), b.xb.data_ptr(), self.s.hidden,
-                                                  self.s.rms_eps, stream), "elutq_decode_rmsnorm_f16")
-            if self.lm_head_q is not None:
-                logits = self.lm_head_q.gemv_fused(b.xb, b.logits, b.ws)
+            if self.lm_head_q is not None:       # the final norm rides in the GEMV's prologue
+                logits = self.lm_head_q.gemv_fused(x, b.logits, b.ws, prologue=1, norm_weight=self.norm,
+                                                   eps=self.s.rms_eps)
             else:
+                _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), b.xb.data_ptr(),
+                                                      self.s.hidden, self.s.rms_eps, stream), "elutq_decode_rmsnorm_f16")
                 logits = torch.mm(b.xb, self.lm_head.t(), out=b.logits)
             _lib.check(L.elutq_decode_argmax_f16(logits.data_ptr(), self.s.vocab, self.token.data_ptr(),
                                                  self.pos.data_ptr(), stream), "elutq_decode_argmax_f16")
@@ -342,12 +348,13 @@ class LlamaDecoder(nn.Module):
 
 
 def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | None = None,
-                 impl: str = "hip") -> dict:
+                 impl: str = "hip", hlq_lm_head: bool = False) -> dict:
     """Decode tokens/s of the random-init model: n_gen greedy tokens after an n_ctx-token
     cache; the first generated token is excluded, as in the reference
-    ((generate_num - 1) / elapsed, main.cpp:110)."""
+    ((generate_num - 1) / elapsed, main.cpp:110).  `hlq_lm_head`: see random_parts."""
     s = shape or LlamaShape()
-    model = LlamaDecoder(s, device=device, seed=0, impl=impl)
+    dev = torch.device(device)
+    model = LlamaDecoder(s, device=dev, seed=0, impl=impl, parts=random_parts(s, dev, 0, hlq_lm_head))
     model.fill_cache(n_ctx)
     model.token.fill_(1)
     model.capture()
@@ -366,9 +373,11 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
     return {"tokens_per_s": (n_gen - 1) / dt, "ms_per_token": ms, "n_ctx": n_ctx, "n_gen": n_gen,
             "bytes_per_token": hlq_bytes + lm_bytes + kv_bytes,
             "GBps": (hlq_bytes + lm_bytes + kv_bytes) / (ms * 1e-3) / 1e9,
-            "model": f"LLaMA-3-8B-shaped random init, {s.n_layers} layers, HLQ w{s.bits}g{s.group}, fp16 lm_head",
+            "model": f"LLaMA-3-8B-shaped random init, {s.n_layers} layers, HLQ w{s.bits}g{s.group}, "
+                     + (f"HLQ w{s.bits}g{s.group} lm_head" if hlq_lm_head else "fp16 lm_head"),
             "glue": ("5 launches per layer (rmsnorm+qkv | rope+cache+attention | o+residual | rmsnorm+gate|up | "
                      "silu*up+down+residual), " if impl == "hip" else "PyTorch-ROCm ops around the HLQ GEMVs, ")
-                    + ("own final norm and argmax kernels, torch embedding gather, hipBLASLt fp16 lm_head, "
+                    + ("own final norm and argmax kernels, torch embedding gather, "
+                       + ("HLQ GEMV lm_head, " if hlq_lm_head else "hipBLASLt fp16 lm_head, ")
                        if impl == "hip" else "torch embedding / final norm / hipBLASLt fp16 lm_head / argmax, ")
                     + "one HIP graph per token"}

@@ -52,6 +52,13 @@ def test_decoder_from_export_tree(cuda, tmp_path, kind, impl):
     for toks, logits in outs[1:]:
         assert toks == outs[0][0] and torch.equal(logits, outs[0][1])
     assert all(0 <= t < TINY.vocab for t in outs[0][0]) and int(models[0].pos) == 13
+    if impl == "hip":
+        # the fused step (with an HLQ lm_head: final norm inside its GEMV) against the PyTorch-glue step
+        glue = LlamaDecoder.from_export(src, TINY, device=cuda, fuse=False, impl="torch")
+        glue.fill_cache(9, seed=3)
+        glue.token.fill_(5)
+        first = glue.step().float()
+        assert float((outs[0][1][:1].float() - first).abs().max()) <= 2e-2 * float(first.abs().max())
 
 
 def test_decoder_with_sparse_extra_planes(cuda, tmp_path):
