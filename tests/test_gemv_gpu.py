@@ -186,3 +186,23 @@ def test_widest_layers_sampled_columns(cuda, n):
     sub = HLQLinear.from_export_arrays(L.w_quant[:, 4096:8192], L.w_scale[:, 4096:8192], L.w_zero[4096:8192], group, None, cuda)
     ys = run(sub, L.x, cuda)[0]
     assert np.max(np.abs(ys.astype(np.float64) - y[4096:8192].astype(np.float64))) <= 2.0 ** -10 * max(1.0, np.max(np.abs(ref)))
+
+
+def test_two_streams_with_their_own_workspaces(cuda):
+    """Calls on different streams may overlap as long as each stream has its own workspace (HLQLinear keeps
+    one per stream): split-K GEMVs and a GEMM issued from two streams at once return what they return alone."""
+    La = make_layer(2048, 512, bits=2, group=128, seed=31, bias=True)
+    Lb = make_layer(1024, 768, bits=3, group=64, seed=32, m=9)
+    ma, mb = to_mod(La, cuda, ksplit=4, waves=8), to_mod(Lb, cuda)
+    xa, xb = torch.from_numpy(La.x).to(cuda), torch.from_numpy(Lb.x).to(cuda)
+    ya0, yb0 = ma(xa).clone(), mb(xb).clone()
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs_a, outs_b = [], []
+    for _ in range(40):
+        with torch.cuda.stream(s1):
+            outs_a.append(ma(xa))
+        with torch.cuda.stream(s2):
+            outs_b.append(mb(xb))
+    torch.cuda.synchronize()
+    assert all(torch.equal(o, ya0) for o in outs_a) and all(torch.equal(o, yb0) for o in outs_b)
