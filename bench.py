@@ -158,8 +158,9 @@ def gemm_leg(torch, lib, dev, steps):
 
 def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
     """Batch-1 GEMV of w2g128 layers that carry a block-sparse extra plane on `density` of their
-    (32 channels x 128 inputs) blocks -- two launches: the plane's fp32 term, then the dense GEMV that
-    adds it -- next to the same dense layers alone.  Weight rings of `ring_len` layers per shape."""
+    (32 channels x 128 inputs) blocks, held as blocks -- two launches: the plane's fp32 term, then the
+    dense GEMV that adds it -- next to the same dense layers alone and to layers of one more dense
+    plane (the form the loader gives the plane by default).  Weight rings of `ring_len` layers per shape."""
     import numpy as np
 
     from elutq_amd.hlq_linear import sparse_index
@@ -198,8 +199,18 @@ def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
 
         t_sp = time_graph(torch, launch_sparse, steps, warmup) / ring_len
         t_de = time_graph(torch, launch_dense, steps, warmup) / ring_len
+        # the plane written out as one more dense plane (scale 0 where no block exists): what the loader does
+        # by default -- it costs what any layer with one more plane costs
+        wide = [Gemv(lib, make_device_layer(k, n, BITS + 1, GROUP, seed=100 + i, device=dev), x, y, ws) for i in range(ring_len)]
+
+        def launch_wide(stream):
+            for gv in wide:
+                gv(stream)
+
+        t_wi = time_graph(torch, launch_wide, steps, warmup) / ring_len
         sparse_bytes = nblk * (32 * GROUP // 8 + 64 + 4) + 4 * (n // 32 + 1) + 8 * n      # blocks, scales, index, fp32 term out and in
         out[f"{k}x{n}"] = {"blocks": nblk, "density": density, "sparse_layer_us": t_sp * 1e6, "dense_layer_us": t_de * 1e6,
+                           "as_one_more_dense_plane_us": t_wi * 1e6,
                            "sparse_plane_bytes": sparse_bytes, "dense_bytes": algorithmic_bytes(k, n, BITS, GROUP)}
     return out
 

@@ -52,6 +52,38 @@ class SparseBlocks:
     mask: np.ndarray             # uint32 [nblk, 2] = (channel start, k start)
 
 
+def densify_sparse(w_quant, w_scale, sparse: SparseBlocks, group: int):
+    """The block-sparse extra plane written out as one more dense plane: the blocks' bits where a block
+    exists and zero bits elsewhere, the blocks' scales where a block exists and scale 0 elsewhere -- the
+    same W, term for term (a scale of 0 contributes exactly 0), in the form every dense kernel reads.
+    Returns (w_quant [bits+1, N, K/8], w_scale [bits+1, N, K/G]), or None if the plane does not fit that
+    form: more than four planes in all, a block that does not start at a group boundary, or two blocks on
+    the same (channel tile, group).  Rows of a last, partial channel tile beyond N are dropped."""
+    w_quant = np.ascontiguousarray(w_quant, dtype=np.uint8)
+    w_scale = np.ascontiguousarray(w_scale, dtype=np.float16)
+    bits, n, k8 = w_quant.shape
+    k, ng = k8 * 8, k8 * 8 // group
+    mask = np.ascontiguousarray(sparse.mask, dtype=np.uint32).reshape(-1, 2).astype(np.int64)
+    nblk = mask.shape[0]
+    blocks = np.ascontiguousarray(sparse.blocks, dtype=np.uint8).reshape(nblk, 32, group // 8)
+    scale = np.ascontiguousarray(sparse.scale, dtype=np.float16).reshape(nblk, 32)
+    if bits + 1 > 4:
+        return None
+    c0, k0 = mask[:, 0], mask[:, 1]
+    if nblk and (np.any(k0 % group) or np.any(c0 % 32) or np.any(c0 >= n) or np.any(k0 + group > k)):
+        return None
+    if nblk and np.unique(c0 // 32 * ng + k0 // group).size != nblk:
+        return None
+    npad = (n + 31) // 32 * 32
+    plane = np.zeros((npad // 32, 32, ng, group // 8), dtype=np.uint8)       # [tile][ch][group][byte]
+    sc = np.zeros((npad // 32, 32, ng), dtype=np.float16)
+    plane[c0 // 32, :, k0 // group, :] = blocks
+    sc[c0 // 32, :, k0 // group] = scale
+    plane = plane.reshape(npad, k8)[:n]
+    sc = sc.reshape(npad, ng)[:n]
+    return np.concatenate([w_quant, plane[None]]), np.concatenate([w_scale, sc[None]])
+
+
 def write_export_dir(path: str, w_quant, w_scale, w_zero, bias=None, groupsize: int | None = None,
                      sparse: SparseBlocks | None = None) -> None:
     """Writes the five files exactly as the reference exporter does.  `groupsize`

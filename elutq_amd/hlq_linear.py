@@ -18,8 +18,8 @@ import torch
 from torch import nn
 
 from . import _lib
-from .export_io import (ExportedLinear, SparseBlocks, is_repacked_dir, read_export_dir, read_repacked_dir,
-                        read_repacked_sparse)
+from .export_io import (ExportedLinear, SparseBlocks, densify_sparse, is_repacked_dir, read_export_dir,
+                        read_repacked_dir, read_repacked_sparse)
 
 _workspaces: dict = {}
 
@@ -136,7 +136,21 @@ class HLQLinear(nn.Module):
     # -- construction ------------------------------------------------------------------
     @classmethod
     def from_export_arrays(cls, w_quant, w_scale, w_zero, group_size: int, bias=None,
-                           device="cuda", sparse: SparseBlocks | None = None) -> "HLQLinear":
+                           device="cuda", sparse: SparseBlocks | None = None, sparse_mode: str = "auto") -> "HLQLinear":
+        """`sparse_mode` says how a block-sparse extra plane is held: "dense" writes it out as one more
+        dense plane (scale 0 where no block exists: the same W, every kernel and every fusion applies, at
+        the price of a whole plane of memory); "blocks" keeps the file form (two launches per call, no fused
+        or grouped launch); "auto" = "dense" where the plane fits that form (export_io.densify_sparse),
+        else "blocks".  On this GPU a launch costs more than the plane's bytes, hence the default."""
+        if sparse_mode not in ("auto", "dense", "blocks"):
+            raise ValueError('sparse_mode must be "auto", "dense" or "blocks"')
+        if sparse is not None and sparse_mode != "blocks":
+            dense = densify_sparse(w_quant, w_scale, sparse, group_size)
+            if dense is not None:
+                (w_quant, w_scale), sparse = dense, None
+            elif sparse_mode == "dense":
+                raise ValueError("the sparse extra plane cannot be written as a dense plane (more than four planes, "
+                                 "a block off the group grid, or two blocks on one tile and group)")
         planes, scales, zeros = repack_export_arrays(w_quant, w_scale, w_zero, group_size)
         bits, n, k8 = np.asarray(w_quant).shape
         dev = torch.device(device)
@@ -158,15 +172,17 @@ class HLQLinear(nn.Module):
                 torch.from_numpy(index).to(dev))
 
     @classmethod
-    def from_export(cls, e: ExportedLinear, device="cuda") -> "HLQLinear":
-        return cls.from_export_arrays(e.w_quant, e.w_scale, e.w_zero, e.group, e.bias, device, e.sparse)
+    def from_export(cls, e: ExportedLinear, device="cuda", sparse_mode: str = "auto") -> "HLQLinear":
+        return cls.from_export_arrays(e.w_quant, e.w_scale, e.w_zero, e.group, e.bias, device, e.sparse, sparse_mode)
 
     @classmethod
-    def from_export_dir(cls, path: str, device="cuda", group_size: int | None = None) -> "HLQLinear":
-        """A linear directory of the reference's export, or the same after `python -m elutq_amd.repack`."""
+    def from_export_dir(cls, path: str, device="cuda", group_size: int | None = None,
+                        sparse_mode: str = "auto") -> "HLQLinear":
+        """A linear directory of the reference's export, or the same after `python -m elutq_amd.repack`
+        (which has settled how a sparse extra plane is held: `sparse_mode` applies to export directories)."""
         if is_repacked_dir(path):
             return cls.from_repacked_dir(path, device)
-        return cls.from_export(read_export_dir(path, group_size), device)
+        return cls.from_export(read_export_dir(path, group_size), device, sparse_mode)
 
     @classmethod
     def from_repacked_dir(cls, path: str, device="cuda") -> "HLQLinear":
@@ -182,6 +198,24 @@ class HLQLinear(nn.Module):
         return cls(k, n, bits, group, torch.from_numpy(planes).to(dev), torch.from_numpy(scales).to(dev),
                    torch.from_numpy(zeros).to(dev), b,
                    cls._sparse_to_device(read_repacked_sparse(path), k, n, group, dev))
+
+    def with_bits(self, bits: int) -> "HLQLinear":
+        """The same layer with `bits` planes: the added planes are all zero with scale 0, so W is unchanged.
+        Lets layers of different depth share a launch (q|k|v where only one of them carries an extra plane)."""
+        if bits == self.bits:
+            return self
+        if bits < self.bits or bits > 4 or self.sparse_count:
+            raise ValueError(f"cannot turn a {self.bits}-plane layer into a {bits}-plane one")
+        ncb = (self.out_features + 63) // 64
+        add = bits - self.bits
+
+        def widen(buf: torch.Tensor, unit_bytes: int) -> torch.Tensor:      # [ncb][units][planes][64 * unit_bytes]
+            v = buf.view(ncb, -1, self.bits, 64 * unit_bytes)
+            z = torch.zeros(ncb, v.shape[1], add, 64 * unit_bytes, dtype=buf.dtype, device=buf.device)
+            return torch.cat([v, z], 2).reshape(-1)
+
+        return HLQLinear(self.in_features, self.out_features, bits, self.group_size, widen(self.planes, 16),
+                         widen(self.scales, 4), self.zeros, self.bias)
 
     # -- compute -----------------------------------------------------------------------
     def forward(self, x: torch.Tensor) -> torch.Tensor:

@@ -54,14 +54,16 @@ def fuse_along_n(mods: list[HLQLinear]) -> HLQLinear:
     """One HLQLinear computing the concatenation of the outputs.  The kernel layout is
     column-block major, so this is a concatenation of the packed buffers (every N but the
     last must be a multiple of 64)."""
-    k, bits, group = mods[0].in_features, mods[0].bits, mods[0].group_size
+    if any(m.sparse_count for m in mods):
+        raise NotImplementedError("layers whose sparse extra plane is held as blocks cannot be concatenated: load "
+                                  "them with sparse_mode='dense', or build the decoder with fuse=False, impl='torch'")
+    k, group = mods[0].in_features, mods[0].group_size
+    bits = max(m.bits for m in mods)                 # a layer that carries an extra plane lifts the others
+    mods = [m.with_bits(bits) for m in mods]
     for m in mods:
-        assert (m.in_features, m.bits, m.group_size) == (k, bits, group)
+        assert (m.in_features, m.group_size) == (k, group)
     for m in mods[:-1]:
         assert m.out_features % 64 == 0
-    if any(m.sparse_count for m in mods):
-        raise NotImplementedError("layers with a sparse extra plane cannot be concatenated: build the decoder "
-                                  "with fuse=False, impl='torch'")
     bias = None
     if any(m.bias is not None for m in mods):
         bias = torch.cat([m.bias if m.bias is not None else
@@ -198,7 +200,7 @@ def random_parts(s: LlamaShape, dev, seed: int, hlq_lm_head: bool = False) -> di
     return {"layers": layers, "embed": embed, "lm_head": lm_head, "norm": norm}
 
 
-def parts_from_export(root: str, s: LlamaShape, dev) -> dict:
+def parts_from_export(root: str, s: LlamaShape, dev, sparse_mode: str = "auto") -> dict:
     """Reads the reference's model export tree (written by GPTQ/llama.py:285-343, read by
     C++/examples/models/llama.cpp:59-115), or the same tree after `python -m elutq_amd.repack`.
     The lm_head is the HLQ layer in lm_head/lm_head if that directory exists, else lm_head.bin,
@@ -214,7 +216,7 @@ def parts_from_export(root: str, s: LlamaShape, dev) -> dict:
         base = os.path.join(root, str(i))
         lin = {}
         for name, (k, n) in proj_shapes(s).items():
-            m = HLQLinear.from_export_dir(os.path.join(base, PROJ_DIRS[name]), dev)
+            m = HLQLinear.from_export_dir(os.path.join(base, PROJ_DIRS[name]), dev, sparse_mode=sparse_mode)
             if (m.in_features, m.out_features) != (k, n):
                 raise ValueError(f"{base}/{PROJ_DIRS[name]}: {m.in_features}x{m.out_features}, the shape needs {k}x{n}")
             lin[name] = m
@@ -222,7 +224,7 @@ def parts_from_export(root: str, s: LlamaShape, dev) -> dict:
     embed = vec(io.embedding_file(root), s.vocab * s.hidden).view(s.vocab, s.hidden)
     kind = io.lm_head_kind(root)
     if kind == "hlq":
-        lm_head = HLQLinear.from_export_dir(os.path.join(root, "lm_head", "lm_head"), dev)
+        lm_head = HLQLinear.from_export_dir(os.path.join(root, "lm_head", "lm_head"), dev, sparse_mode=sparse_mode)
         if (lm_head.in_features, lm_head.out_features) != (s.hidden, s.vocab):
             raise ValueError("lm_head/lm_head does not match hidden x vocab")
     elif kind == "fp16":
@@ -267,16 +269,19 @@ class LlamaDecoder(nn.Module):
         self._buf = None
         if impl == "hip":
             if any(m.sparse_count for m in self.modules() if isinstance(m, HLQLinear)):
-                raise NotImplementedError("the fused decode step has no sparse extra plane: build the decoder "
-                                          "with fuse=False, impl='torch'")
+                raise NotImplementedError("the fused decode step takes no sparse extra plane held as blocks: load the "
+                                          "layers with sparse_mode='dense', or build the decoder with fuse=False, "
+                                          "impl='torch'")
             ws = max(m.workspace_bytes for m in self.modules() if isinstance(m, HLQLinear))
             ws = max(ws, _lib.lib().elutq_decode_attn_workspace_bytes(s.n_heads, s.head_dim, 0))
             self._buf = FusedBuffers(s, ws, dev)
 
     @classmethod
-    def from_export(cls, root: str, s: LlamaShape, device="cuda", fuse: bool = True, impl: str = "hip") -> "LlamaDecoder":
+    def from_export(cls, root: str, s: LlamaShape, device="cuda", fuse: bool = True, impl: str = "hip",
+                    sparse_mode: str = "auto") -> "LlamaDecoder":
         """A decoder over a genuinely exported model (bits and group size come from the files)."""
-        return cls(s, device=device, fuse=fuse, impl=impl, parts=parts_from_export(root, s, torch.device(device)))
+        return cls(s, device=device, fuse=fuse, impl=impl,
+                   parts=parts_from_export(root, s, torch.device(device), sparse_mode))
 
     @torch.no_grad()
     def fill_cache(self, n_tokens: int, seed: int = 1) -> None:

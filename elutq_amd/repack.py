@@ -17,11 +17,14 @@ import os
 import shutil
 import sys
 
-from .export_io import read_export_dir, write_repacked_dir
+from .export_io import densify_sparse, read_export_dir, write_repacked_dir
 
 
-def repack_tree(src: str, dst: str, group_size: int | None = None, verbose: bool = False) -> int:
-    """Returns the number of linear layers repacked."""
+def repack_tree(src: str, dst: str, group_size: int | None = None, verbose: bool = False,
+                sparse_mode: str = "auto") -> int:
+    """Returns the number of linear layers repacked.  `sparse_mode` as in HLQLinear.from_export_arrays:
+    "auto" / "dense" write a block-sparse extra plane out as one more dense plane where that is possible,
+    "blocks" keeps its file form beside the dense planes."""
     from .hlq_linear import repack_export_arrays
     count = 0
     for cur, dirs, files in os.walk(src):
@@ -29,15 +32,23 @@ def repack_tree(src: str, dst: str, group_size: int | None = None, verbose: bool
         out = os.path.join(dst, rel) if rel != "." else dst
         if "weight_config.json" in files:
             e = read_export_dir(cur, group_size)
-            planes, scales, zeros = repack_export_arrays(e.w_quant, e.w_scale, e.w_zero, e.group)
-            if e.sparse is not None:
+            w_quant, w_scale, sparse, bits = e.w_quant, e.w_scale, e.sparse, e.bits
+            if sparse is not None:
                 from .hlq_linear import sparse_index
-                sparse_index(e.sparse.mask, e.k, e.n, e.group)      # validates the block list
-            write_repacked_dir(out, e.k, e.n, e.bits, e.group, planes, scales, zeros, e.bias, e.sparse)
+                sparse_index(sparse.mask, e.k, e.n, e.group)        # validates the block list
+                dense = densify_sparse(w_quant, w_scale, sparse, e.group) if sparse_mode != "blocks" else None
+                if dense is not None:
+                    (w_quant, w_scale), sparse, bits = dense, None, e.bits + 1
+                elif sparse_mode == "dense":
+                    raise ValueError(f"{cur}: the sparse extra plane cannot be written as a dense plane")
+            planes, scales, zeros = repack_export_arrays(w_quant, w_scale, e.w_zero, e.group)
+            write_repacked_dir(out, e.k, e.n, bits, e.group, planes, scales, zeros, e.bias, sparse)
             count += 1
             dirs[:] = []
             if verbose:
-                extra = f" + {e.sparse.mask.shape[0]} sparse blocks" if e.sparse is not None else ""
+                extra = ""
+                if e.sparse is not None:
+                    extra = f" + {e.sparse.mask.shape[0]} sparse blocks" + (" as a dense plane" if sparse is None else "")
                 print(f"{rel}: K={e.k} N={e.n} w{e.bits}g{e.group}{extra}", file=sys.stderr)
             continue
         os.makedirs(out, exist_ok=True)
@@ -52,12 +63,15 @@ def main(argv=None) -> int:
     ap.add_argument("dst")
     ap.add_argument("--groupsize", type=int, default=None,
                     help="only needed if neither the json nor the size of w_zero.bin determines it")
+    ap.add_argument("--sparse", choices=["auto", "dense", "blocks"], default="auto",
+                    help="how a block-sparse extra plane is stored: as one more dense plane where possible "
+                         "(auto, the default; dense insists), or in its file form (blocks)")
     ap.add_argument("-v", "--verbose", action="store_true")
     a = ap.parse_args(argv)
     if not os.path.isdir(a.src):
         print(f"{a.src}: not a directory", file=sys.stderr)
         return 2
-    n = repack_tree(a.src, a.dst, a.groupsize, a.verbose)
+    n = repack_tree(a.src, a.dst, a.groupsize, a.verbose, a.sparse)
     print(f"repacked {n} linear layers into {a.dst}")
     return 0 if n else 1
 

@@ -62,27 +62,33 @@ def test_decoder_from_export_tree(cuda, tmp_path, kind, impl):
 
 
 def test_decoder_with_sparse_extra_planes(cuda, tmp_path):
-    """Layers with a sparse extra plane load from both tree forms and run through the plain HLQLinear
-    calls of the PyTorch-glue step; the fused step refuses them."""
+    """Layers with a sparse extra plane: by default the plane is written out as one more dense plane at load, so the
+    fused step runs them (q carries three planes, k and v two: the concatenation lifts k and v); held as blocks they
+    run through the plain HLQLinear calls of the PyTorch-glue step, and the fused step refuses them."""
     src, dst, plain = str(tmp_path / "export"), str(tmp_path / "repacked"), str(tmp_path / "plain")
     write_tiny_export(src, sparse_on=("down_proj", "q_proj"))
     write_tiny_export(plain)
     repack_tree(src, dst)
     with pytest.raises(NotImplementedError):
-        LlamaDecoder.from_export(src, TINY, device=cuda, impl="hip")
+        LlamaDecoder.from_export(src, TINY, device=cuda, impl="hip", sparse_mode="blocks")
     outs = []
-    for root in (src, dst, plain):
-        m = LlamaDecoder.from_export(root, TINY, device=cuda, fuse=False, impl="torch")
+    for root, kw in ((src, dict(impl="hip")), (dst, dict(impl="hip")), (src, dict(fuse=False, impl="torch", sparse_mode="blocks")),
+                     (plain, dict(impl="hip"))):
+        m = LlamaDecoder.from_export(root, TINY, device=cuda, **kw)
         m.fill_cache(9, seed=3)
         m.token.fill_(5)
         logits = torch.cat([m.step().clone() for _ in range(3)])
         outs.append((m, logits))
-    assert outs[0][0].layers[0].down_proj.sparse_count > 0 and outs[2][0].layers[0].down_proj.sparse_count == 0
+    assert outs[0][0].layers[0].down_proj.bits == 3 and outs[0][0].layers[0].qkv.bits == 3
+    assert outs[2][0].layers[0].down_proj.sparse_count > 0 and outs[3][0].layers[0].down_proj.bits == 2
     assert torch.equal(outs[0][1], outs[1][1])                  # export tree == repacked tree
-    assert not torch.equal(outs[0][1], outs[2][1])              # and the planes do take part
-    # every sparse layer equals its own dequantized weight applied densely
+    assert not torch.equal(outs[0][1], outs[3][1])              # the planes do take part
+    # fused step on dense planes against the glue step on blocks: the first step's logits
+    a, b = outs[0][1][:1].float(), outs[2][1][:1].float()
+    assert float((a - b).abs().max()) <= 2e-2 * float(b.abs().max())
+    # every layer held as blocks equals its own dequantized weight applied densely
     x = torch.randn(3, TINY.ffn, device=cuda).to(torch.float16)
-    mod = outs[0][0].layers[1].down_proj
+    mod = outs[2][0].layers[1].down_proj
     want = x.float() @ mod.dequantize().float().T + (mod.bias.float() if mod.bias is not None else 0)
     got = mod(x).float()
     assert float((got - want).abs().max()) <= 2e-2 * float(want.pow(2).mean().sqrt())

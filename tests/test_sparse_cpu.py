@@ -7,8 +7,9 @@ import numpy as np
 import pytest
 
 from elutq_amd import _lib
-from elutq_amd.export_io import SparseBlocks, read_export_dir, read_repacked_sparse, write_export_dir
-from elutq_amd.hlq_linear import sparse_index
+from elutq_amd.export_io import (SparseBlocks, densify_sparse, read_export_dir, read_repacked_dir, read_repacked_sparse,
+                                 write_export_dir)
+from elutq_amd.hlq_linear import sparse_index, unpack_to_export_arrays
 from elutq_amd.repack import repack_tree
 from elutq_amd.synth import make_layer, make_sparse_plane, pack_bits_lsb_first
 from oracle import hlq_oracle as O
@@ -70,12 +71,40 @@ def test_index_rejects_malformed_lists(mask):
     assert e.value.status == -8 and "sparse" in str(e.value)
 
 
-def test_repack_cli_keeps_the_sparse_plane(tmp_path):
+def test_dense_form_of_the_plane_is_the_same_weight():
+    """One more dense plane with scale 0 where no block exists dequantizes to exactly the sparse layer's W;
+    planes that do not fit that form are reported as such."""
+    L, b, s, m, sp = sparse_layer(384, 96, 2, 128, 0.5, 7)
+    wq, ws = densify_sparse(L.w_quant, L.w_scale, sp, 128)
+    assert wq.shape == (3, 96, 48) and ws.shape == (3, 96, 3) and ws.dtype == np.float16
+    assert np.array_equal(wq[:2], L.w_quant) and np.array_equal(ws[:2], L.w_scale)
+    assert np.array_equal(O.dequantize(wq, ws, L.w_zero, 128), O.dequantize_sparse(L.w_quant, L.w_scale, L.w_zero, O.SparsePlane(b, s, m, 128)))
+    # ragged N: the rows of the last tile beyond N are dropped
+    wq2, ws2 = densify_sparse(L.w_quant[:, :70], L.w_scale[:, :70], sp, 128)
+    assert np.array_equal(wq2[2], wq[2, :70]) and np.array_equal(ws2[2], ws[2, :70])
+    one = SparseBlocks(sp.blocks[:1], s[:1], np.array([[0, 0]], np.uint32))
+    assert densify_sparse(L.w_quant, L.w_scale, SparseBlocks(sp.blocks[:1], s[:1], np.array([[0, 4]], np.uint32)), 128) is None
+    assert densify_sparse(L.w_quant, L.w_scale, SparseBlocks(sp.blocks[:2], s[:2], np.array([[32, 128], [32, 128]], np.uint32)), 128) is None
+    assert densify_sparse(np.zeros((4, 96, 48), np.uint8), np.zeros((4, 96, 3), np.float16), one, 128) is None
+    assert densify_sparse(L.w_quant, L.w_scale, one, 128) is not None
+
+
+def test_repack_cli_and_the_sparse_plane(tmp_path):
     L, b, s, m, sp = sparse_layer(256, 64, 2, 128, 0.5, 5)
-    src, dst = str(tmp_path / "src"), str(tmp_path / "dst")
+    src = str(tmp_path / "src")
     write_export_dir(os.path.join(src, "0", "mlp.down_proj"), L.w_quant, L.w_scale, L.w_zero, L.bias, sparse=sp)
     write_export_dir(os.path.join(src, "0", "mlp.up_proj"), L.w_quant, L.w_scale, L.w_zero)
+    # default: the plane becomes a third dense plane
+    dst = str(tmp_path / "dst")
     assert repack_tree(src, dst) == 2
+    k, n, bits, group, planes, scales, zeros, bias = read_repacked_dir(os.path.join(dst, "0", "mlp.down_proj"))
+    assert (k, n, bits, group) == (256, 64, 3, 128) and read_repacked_sparse(os.path.join(dst, "0", "mlp.down_proj")) is None
+    wq, ws, wz = unpack_to_export_arrays(planes, scales, zeros, k, n, bits, group)
+    assert np.array_equal(O.dequantize(wq, ws, wz, 128), O.dequantize_sparse(L.w_quant, L.w_scale, L.w_zero, O.SparsePlane(b, s, m, 128)))
+    # "blocks": the file form is kept beside the two dense planes
+    dst = str(tmp_path / "dst_blocks")
+    assert repack_tree(src, dst, sparse_mode="blocks") == 2
+    assert read_repacked_dir(os.path.join(dst, "0", "mlp.down_proj"))[2] == 2
     got = read_repacked_sparse(os.path.join(dst, "0", "mlp.down_proj"))
     assert np.array_equal(got.blocks, sp.blocks) and np.array_equal(got.scale, s) and np.array_equal(got.mask, m)
     assert read_repacked_sparse(os.path.join(dst, "0", "mlp.up_proj")) is None

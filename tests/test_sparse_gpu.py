@@ -20,11 +20,13 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-def build(k, n, bits, group, density, seed, dev, m=1, bias=True):
+def build(k, n, bits, group, density, seed, dev, m=1, bias=True, mode="blocks"):
+    """mode "blocks": the plane in its file form (the block kernels); "dense": written out as one more plane."""
     L = make_layer(k, n, bits, group, m=m, seed=seed, bias=bias)
     b, s, mk = make_sparse_plane(k, n, group, density, seed=seed + 100)
     mod = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, group, L.bias, dev,
-                                       SparseBlocks(pack_bits_lsb_first(b), s, mk))
+                                       SparseBlocks(pack_bits_lsb_first(b), s, mk), sparse_mode=mode)
+    assert (mod.sparse_count > 0) == (mode == "blocks" and mk.shape[0] > 0)
     return L, O.SparsePlane(b, s, mk, group), mod
 
 
@@ -79,11 +81,14 @@ def test_bit_exact_on_integer_inputs(cuda, group, m):
     b, _, mk = make_sparse_plane(k, n, group, 0.5, seed=group)
     s = np.full((mk.shape[0], 32), 2.0, np.float16)
     sp = O.SparsePlane(b, s, mk, group)
-    mod = HLQLinear.from_export_arrays(wq, ws, wz, group, None, cuda, SparseBlocks(sp.packed, s, mk))
+    mod = HLQLinear.from_export_arrays(wq, ws, wz, group, None, cuda, SparseBlocks(sp.packed, s, mk), sparse_mode="blocks")
+    auto = HLQLinear.from_export_arrays(wq, ws, wz, group, None, cuda, SparseBlocks(sp.packed, s, mk))
+    assert mod.sparse_count > 0 and auto.sparse_count == 0 and auto.bits == 3
     x = r.integers(-2, 3, (m, k)).astype(np.float16)
     y = run(mod, x, cuda)
     want = x.astype(np.float64) @ O.dequantize_sparse(wq, ws, wz, sp).T
     assert np.array_equal(y.astype(np.float64), want)
+    assert np.array_equal(run(auto, x, cuda).astype(np.float64), want)       # the dense form: the same bits
 
 
 def test_blocks_everywhere_equal_one_more_dense_plane(cuda):
@@ -100,7 +105,10 @@ def test_blocks_everywhere_equal_one_more_dense_plane(cuda):
             mk.append((32 * t, group * g))
     sp = SparseBlocks(pack_bits_lsb_first(np.stack(blk)), np.stack(sc), np.array(mk, np.uint32))
     dense = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, group, None, cuda)
-    sparse = HLQLinear.from_export_arrays(L.w_quant[:2], L.w_scale[:2], L.w_zero, group, None, cuda, sp)
+    sparse = HLQLinear.from_export_arrays(L.w_quant[:2], L.w_scale[:2], L.w_zero, group, None, cuda, sp, sparse_mode="blocks")
+    again = HLQLinear.from_export_arrays(L.w_quant[:2], L.w_scale[:2], L.w_zero, group, None, cuda, sp)
+    # written out densely, the full cover IS the three-plane layer: the same buffers
+    assert again.bits == 3 and torch.equal(again.planes, dense.planes) and torch.equal(again.scales, dense.scales)
     wd, wsp = dense.dequantize().float().cpu().numpy(), sparse.dequantize().float().cpu().numpy()
     ref = O.dequantize(L.w_quant, L.w_scale, L.w_zero, group)
     assert np.max(np.abs(wd - ref)) <= 2.0 ** -11 * np.max(np.abs(ref))
@@ -120,6 +128,10 @@ def test_unaligned_and_overlapping_blocks(cuda):
     s = r.uniform(0.02, 0.08, (5, 32)).astype(np.float16)
     sp = O.SparsePlane(b, s, mk, group)
     mod = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, group, None, cuda, SparseBlocks(sp.packed, s, mk))
+    assert mod.sparse_count == 5          # off the group grid and repeated: stays in block form whatever the mode
+    with pytest.raises(ValueError):
+        HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, group, None, cuda, SparseBlocks(sp.packed, s, mk),
+                                     sparse_mode="dense")
     y = run(mod, L.x, cuda)[0]
     assert O.rel_err(y, O.gemv_sparse_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, sp)) <= TOL
     w = mod.dequantize().float().cpu().numpy()
@@ -133,9 +145,13 @@ def test_ragged_n(cuda):
     L = make_layer(k, npad, 2, group, seed=51, bias=True)
     b, s, mk = make_sparse_plane(k, npad, group, 1.0, seed=52)
     sp = O.SparsePlane(b, s, mk, group)
-    mod = HLQLinear.from_export_arrays(L.w_quant[:, :n], L.w_scale[:, :n], L.w_zero[:n], group, L.bias[:n], cuda,
-                                       SparseBlocks(sp.packed, s, mk))
+    sb = SparseBlocks(sp.packed, s, mk)
+    mod = HLQLinear.from_export_arrays(L.w_quant[:, :n], L.w_scale[:, :n], L.w_zero[:n], group, L.bias[:n], cuda, sb,
+                                       sparse_mode="blocks")
+    dense = HLQLinear.from_export_arrays(L.w_quant[:, :n], L.w_scale[:, :n], L.w_zero[:n], group, L.bias[:n], cuda, sb)
     x = np.concatenate([L.x, -L.x, 0.5 * L.x])
+    assert dense.sparse_count == 0 and O.rel_err(run(dense, x, cuda), (x.astype(np.float64) @ O.dequantize_sparse(
+        L.w_quant, L.w_scale, L.w_zero, sp).T + L.bias.astype(np.float64))[:, :n]) <= TOL
     y = run(mod, x, cuda)
     ref = (x.astype(np.float64) @ O.dequantize_sparse(L.w_quant, L.w_scale, L.w_zero, sp).T + L.bias.astype(np.float64))[:, :n]
     assert y.shape == (3, n) and O.rel_err(y, ref) <= TOL
@@ -148,12 +164,20 @@ def test_export_dir_and_repacked_dir_load_the_same_layer(cuda, tmp_path):
     src, dst = str(tmp_path / "src"), str(tmp_path / "dst")
     d = os.path.join(src, "0", "mlp.gate_proj")
     write_export_dir(d, L.w_quant, L.w_scale, L.w_zero, L.bias, sparse=SparseBlocks(sp.packed, sp.scale, sp.mask))
-    assert repack_tree(src, dst) == 1
+    assert repack_tree(src, dst, sparse_mode="blocks") == 1
     y = run(mod, L.x, cuda)
     for path in (d, os.path.join(dst, "0", "mlp.gate_proj")):
-        other = HLQLinear.from_export_dir(path, cuda)
+        other = HLQLinear.from_export_dir(path, cuda, sparse_mode="blocks")
         assert other.sparse_count == mod.sparse_count and "sparse_blocks" in repr(other)
         assert np.array_equal(run(other, L.x, cuda).view(np.uint16), y.view(np.uint16))
+    # the default of loader and CLI: one more dense plane, from either tree form, the same bits
+    dst2 = str(tmp_path / "dst_dense")
+    assert repack_tree(src, dst2) == 1
+    a, b = HLQLinear.from_export_dir(d, cuda), HLQLinear.from_export_dir(os.path.join(dst2, "0", "mlp.gate_proj"), cuda)
+    assert a.sparse_count == 0 and b.sparse_count == 0 and a.bits == b.bits == 3
+    ya = run(a, L.x, cuda)
+    assert np.array_equal(ya.view(np.uint16), run(b, L.x, cuda).view(np.uint16))
+    assert O.rel_err(ya[0], O.gemv_sparse_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, sp, L.bias)) <= TOL
 
 
 def test_full_size_layer(cuda):
@@ -167,6 +191,20 @@ def test_full_size_layer(cuda):
     assert np.array_equal(y.view(np.uint16), y2.view(np.uint16))          # run-to-run determinism
     ym = run(mod, -L.x, cuda)[0]
     assert np.array_equal((-ym).view(np.uint16), y.view(np.uint16))       # y(-x) = -y(x) exactly
+
+
+@pytest.mark.parametrize("k,n,bits,group,density", [(512, 128, 2, 128, 0.3), (1024, 256, 3, 64, 0.2), (4096, 4096, 2, 128, 0.1)])
+def test_dense_form_matches_oracle(cuda, k, n, bits, group, density):
+    """The default way to hold the plane on this GPU: one more dense plane, every dense kernel as it is."""
+    L, sp, mod = build(k, n, bits, group, density, k + n + 1, cuda, m=3, mode="dense")
+    assert mod.bits == bits + 1
+    y = run(mod, L.x, cuda)
+    ref = L.x.astype(np.float64) @ O.dequantize_sparse(L.w_quant, L.w_scale, L.w_zero, sp).T + L.bias.astype(np.float64)
+    assert O.rel_err(y, ref) <= TOL
+    assert O.rel_err(run(mod, L.x[:1], cuda)[0], ref[0]) <= TOL
+    w = mod.dequantize().float().cpu().numpy()
+    wref = O.dequantize_sparse(L.w_quant, L.w_scale, L.w_zero, sp)
+    assert np.max(np.abs(w - wref)) <= 2.0 ** -11 * np.max(np.abs(wref))
 
 
 def test_no_fused_or_grouped_launch_for_sparse_layers(cuda):
