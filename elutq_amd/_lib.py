@@ -32,6 +32,7 @@ SIGNATURES = {
     "elutq_decode_attn_workspace_bytes": (_sz, [_ci] * 3),
     "elutq_decode_rmsnorm_f16": (_ci, [_vp] * 3 + [_ci, ctypes.c_float, _vp]),
     "elutq_decode_argmax_f16": (_ci, [_vp, _ci, _vp, _vp, _vp]),
+    "elutq_decode_argmax_ws_f16": (_ci, [_vp, _ci, _vp, _vp, _vp, _sz, _vp]),
     "elutq_hlq_gemv_group_workspace_bytes": (_sz, [_vp, _ci, _ci, _ci]),
     "elutq_hlq_gemv_group_create": (_ci, [_vp, _ci, _ci, _ci, _vp, _sz, _vp]),
     "elutq_hlq_gemv_group_run": (_ci, [_vp, _vp]),

@@ -462,6 +462,65 @@ __global__ __launch_bounds__(TAIL_THREADS) void argmax_kernel(const uint16_t *lo
     }
 }
 
+// The same pick over a long vector by ARGMAX_WGS workgroups that meet in device memory like the splits
+// of the attention kernel: each takes a contiguous range of 8-value groups, stores its (value, index)
+// with agent-scope stores, waits for their acknowledgement and draws a ticket; the last one merges the
+// pairs (ties go to the lower index, so the result is that of one scan).  One workgroup takes in a
+// vocabulary's logits no faster than about 50 KB/us; the vector needs 16-byte alignment here.
+constexpr int ARGMAX_WGS = 64, ARGMAX_THREADS = 256;
+
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_split_kernel(const uint16_t *logits, int n, long long *token,
+                                                                      long long *pos, float *pval, int *pidx,
+                                                                      unsigned *counter)
+{
+    __shared__ float sv[ARGMAX_THREADS / 64];
+    __shared__ int si[ARGMAX_THREADS / 64];
+    __shared__ unsigned s_ticket;
+    const int tid = threadIdx.x, wg = blockIdx.x;
+    const int nvec = n / 8, per = (nvec + ARGMAX_WGS - 1) / ARGMAX_WGS;
+    const int c_begin = wg * per, c_end = min(c_begin + per, nvec);
+    float best = -INFINITY;
+    int idx = 0x7fffffff;
+    for (int c = c_begin + tid; c < c_end; c += ARGMAX_THREADS) {       // indices rise within a thread
+        const uint4 q = ((const uint4 *)logits)[c];
+        const uint32_t wd[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float lo = h2f((uint16_t)(wd[j] & 0xffffu)), hi = h2f((uint16_t)(wd[j] >> 16));
+            if (lo > best) { best = lo; idx = c * 8 + 2 * j; }
+            if (hi > best) { best = hi; idx = c * 8 + 2 * j + 1; }
+        }
+    }
+    if (wg == ARGMAX_WGS - 1)                                             // the last n % 8 values
+        for (int i = nvec * 8 + tid; i < n; i += ARGMAX_THREADS) {
+            const float v = h2f(logits[i]);
+            if (v > best) { best = v; idx = i; }
+        }
+#pragma unroll
+    for (int sh = 1; sh < 64; sh <<= 1) pick(best, idx, __shfl_xor(best, sh, 64), __shfl_xor(idx, sh, 64));
+    if ((tid & 63) == 0) { sv[tid >> 6] = best; si[tid >> 6] = idx; }
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+        for (int i = 1; i < ARGMAX_THREADS / 64; i++) pick(best, idx, sv[i], si[i]);
+        __hip_atomic_store(&pval[wg], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&pidx[wg], idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        s_ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (s_ticket != (unsigned)ARGMAX_WGS - 1u || tid >= 64) return;
+    best = __hip_atomic_load(&pval[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // ARGMAX_WGS == 64: one pair per lane
+    idx = __hip_atomic_load(&pidx[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int sh = 1; sh < 64; sh <<= 1) pick(best, idx, __shfl_xor(best, sh, 64), __shfl_xor(idx, sh, 64));
+    if (tid == 0) {
+        *token = idx == 0x7fffffff ? 0 : idx;
+        if (pos) *pos += 1;
+        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 }  // namespace
 
 extern "C" size_t elutq_decode_attn_workspace_bytes(int n_heads, int head_dim, int splits)
@@ -533,6 +592,23 @@ extern "C" int elutq_decode_rmsnorm_f16(const void *d_x, const void *d_weight, v
     if (n < 1) return ELUTQ_ERR_SHAPE;
     hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(TAIL_THREADS), 0, (hipStream_t)stream, (const uint16_t *)d_x,
                        (const uint16_t *)d_weight, (uint16_t *)d_out, n, eps);
+    return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
+}
+
+extern "C" int elutq_decode_argmax_ws_f16(const void *d_logits, int n, void *d_token, void *d_pos, void *d_workspace,
+                                          size_t workspace_bytes, void *stream)
+{
+    if (!d_logits || !d_token) return ELUTQ_ERR_NULL;
+    if (n < 1) return ELUTQ_ERR_SHAPE;
+    const size_t need = (size_t)HLQ_WS_COUNTER_BYTES + (size_t)ARGMAX_WGS * (sizeof(float) + sizeof(int));
+    // short or unaligned vectors, or no workspace: the single-workgroup kernel
+    if (!d_workspace || n < 16384 || ((uintptr_t)d_logits & 15) != 0)
+        return elutq_decode_argmax_f16(d_logits, n, d_token, d_pos, stream);
+    if (workspace_bytes < need) return ELUTQ_ERR_WORKSPACE;
+    float *pval = (float *)((unsigned char *)d_workspace + HLQ_WS_COUNTER_BYTES);
+    hipLaunchKernelGGL(argmax_split_kernel, dim3(ARGMAX_WGS), dim3(ARGMAX_THREADS), 0, (hipStream_t)stream,
+                       (const uint16_t *)d_logits, n, (long long *)d_token, (long long *)d_pos, pval,
+                       (int *)(pval + ARGMAX_WGS), (unsigned *)d_workspace);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
 

@@ -320,8 +320,9 @@ class LlamaDecoder(nn.Module):
                 _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), b.xb.data_ptr(),
                                                       self.s.hidden, self.s.rms_eps, stream), "elutq_decode_rmsnorm_f16")
                 logits = torch.mm(b.xb, self.lm_head.t(), out=b.logits)
-            _lib.check(L.elutq_decode_argmax_f16(logits.data_ptr(), self.s.vocab, self.token.data_ptr(),
-                                                 self.pos.data_ptr(), stream), "elutq_decode_argmax_f16")
+            _lib.check(L.elutq_decode_argmax_ws_f16(logits.data_ptr(), self.s.vocab, self.token.data_ptr(),
+                                                    self.pos.data_ptr(), b.ws.data_ptr(), b.ws.numel(), stream),
+                       "elutq_decode_argmax_ws_f16")
             return logits
         xn = rms_norm(x, self.norm, self.s.rms_eps)
         logits = self.lm_head_q(xn) if self.lm_head_q is not None else F.linear(xn, self.lm_head)

@@ -175,13 +175,23 @@ def test_rope_attn_rejects_bad_arguments(cuda):
     assert bool((out == 7).all())
 
 
-@pytest.mark.parametrize("n", [1, 7, 8, 4096, 128256, 128259])
-def test_argmax_kernel(cuda, n):
-    """elutq_decode_argmax_f16: first index of the strict maximum (arm_argmax.cpp:3-30), also
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("n", [1, 7, 8, 4096, 16384, 128256, 128259])
+def test_argmax_kernel(cuda, n, split):
+    """elutq_decode_argmax_f16 / _ws_f16 (64 workgroups that meet in a workspace; two calls in a row must
+    find its counter at zero): first index of the strict maximum (arm_argmax.cpp:3-30), also
     with the maximum repeated, at either end, in the unaligned tail, and with NaNs present;
     the position counter is advanced by one."""
     from elutq_amd import _lib
-    L = _lib.lib()
+    lib = _lib.lib()
+    ws = torch.zeros(65536 + 512, dtype=torch.uint8, device=cuda)
+
+    class L:              # the entry point under test, with the single-workgroup signature
+        @staticmethod
+        def elutq_decode_argmax_f16(logits, count, token, position, st):
+            if split:
+                return lib.elutq_decode_argmax_ws_f16(logits, count, token, position, ws.data_ptr(), ws.numel(), st)
+            return lib.elutq_decode_argmax_f16(logits, count, token, position, st)
     g = torch.Generator(device=cuda).manual_seed(n)
     stream = torch.cuda.current_stream().cuda_stream
     tok = torch.full((1,), -5, dtype=torch.long, device=cuda)
@@ -210,6 +220,12 @@ def test_argmax_kernel(cuda, n):
         assert int(tok) == int(c[1:].float().argmax())
     assert L.elutq_decode_argmax_f16(None, n, tok.data_ptr(), None, stream) == -1
     assert L.elutq_decode_argmax_f16(cases[0].data_ptr(), 0, tok.data_ptr(), None, stream) == -2
+    if split:
+        assert not bool(ws[:4].any())                    # the arrival counter is back at zero
+        if n >= 16384:
+            small = torch.zeros(1024, dtype=torch.uint8, device=cuda)
+            assert _lib.lib().elutq_decode_argmax_ws_f16(cases[0].data_ptr(), n, tok.data_ptr(), None, small.data_ptr(),
+                                                         small.numel(), stream) == -5
 
 
 @pytest.mark.parametrize("n", [64, 4096, 5120, 1000])
