@@ -602,7 +602,7 @@ extern "C" int elutq_decode_argmax_ws_f16(const void *d_logits, int n, void *d_t
     if (n < 1) return ELUTQ_ERR_SHAPE;
     const size_t need = (size_t)HLQ_WS_COUNTER_BYTES + (size_t)ARGMAX_WGS * (sizeof(float) + sizeof(int));
     // short or unaligned vectors, or no workspace: the single-workgroup kernel
-    if (!d_workspace || n < 16384 || ((uintptr_t)d_logits & 15) != 0)
+    if (!d_workspace || n < 65536 || ((uintptr_t)d_logits & 15) != 0)
         return elutq_decode_argmax_f16(d_logits, n, d_token, d_pos, stream);
     if (workspace_bytes < need) return ELUTQ_ERR_WORKSPACE;
     float *pval = (float *)((unsigned char *)d_workspace + HLQ_WS_COUNTER_BYTES);

@@ -176,7 +176,7 @@ def test_rope_attn_rejects_bad_arguments(cuda):
 
 
 @pytest.mark.parametrize("split", [False, True])
-@pytest.mark.parametrize("n", [1, 7, 8, 4096, 16384, 128256, 128259])
+@pytest.mark.parametrize("n", [1, 7, 8, 4096, 65536, 128256, 128259])
 def test_argmax_kernel(cuda, n, split):
     """elutq_decode_argmax_f16 / _ws_f16 (64 workgroups that meet in a workspace; two calls in a row must
     find its counter at zero): first index of the strict maximum (arm_argmax.cpp:3-30), also
@@ -222,7 +222,7 @@ def test_argmax_kernel(cuda, n, split):
     assert L.elutq_decode_argmax_f16(cases[0].data_ptr(), 0, tok.data_ptr(), None, stream) == -2
     if split:
         assert not bool(ws[:4].any())                    # the arrival counter is back at zero
-        if n >= 16384:
+        if n >= 65536:
             small = torch.zeros(1024, dtype=torch.uint8, device=cuda)
             assert _lib.lib().elutq_decode_argmax_ws_f16(cases[0].data_ptr(), n, tok.data_ptr(), None, small.data_ptr(),
                                                          small.numel(), stream) == -5
