@@ -878,7 +878,10 @@ void choose_shape(const HlqGeo &g, int &ksplit, int &waves)
             if (ksplit < fill) ksplit = fill;
         }
         if (ksplit > 4) ksplit = 4;
-        const int by_len = (g.U + 31) / 32;
+        // slices of at most 32 units (one table-build pass of 1024 lanes); with workgroups to spare anyway
+        // a slice of up to 48 units in two passes beats a second slice and its exchange (K = 5120: 9.5 -> 8.9 us)
+        const int max_ups = g.ncb >= 128 ? 48 : 32;
+        const int by_len = (g.U + max_ups - 1) / max_ups;
         if (ksplit < by_len) ksplit = by_len;
         if (ksplit > g.U) ksplit = g.U;
     }
