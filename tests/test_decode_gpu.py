@@ -110,10 +110,21 @@ def test_rope_cache_attention_kernel(cuda, d, nq, nkv, splits, pos):
     workgroups per head, 0 = default) against the PyTorch restatement of the reference ops
     (half-split RoPE, cache append, fp32-softmax GQA attention); two calls in a row on one
     workspace (the second must find the arrival counters at zero)."""
+    check_rope_cache_attention(cuda, d, nq, nkv, splits, pos, max_seq=1100)
+
+
+@pytest.mark.parametrize("d,nq,nkv,splits", [(128, 32, 8, 0), (128, 8, 2, 1), (128, 8, 2, 8), (128, 4, 4, 3), (64, 8, 2, 4)])
+@pytest.mark.parametrize("pos", [2047, 4096, 8191])
+def test_rope_cache_attention_kernel_long_context(cuda, d, nq, nkv, splits, pos):
+    """The same check at the context lengths of a LLaMA-3 model (cache of 8192 positions)."""
+    check_rope_cache_attention(cuda, d, nq, nkv, splits, pos, max_seq=8192)
+
+
+def check_rope_cache_attention(cuda, d, nq, nkv, splits, pos, max_seq):
     from elutq_amd import _lib
     from elutq_amd.llama_decode import rope
     g = torch.Generator(device=cuda).manual_seed(pos * 7 + d)
-    max_seq, base = 1100, 10000.0
+    base = 10000.0
     L = _lib.lib()
     qkv = torch.randn(1, (nq + 2 * nkv) * d, generator=g, device=cuda).half()
     kc = torch.randn(max_seq, nkv, d, generator=g, device=cuda).half()
