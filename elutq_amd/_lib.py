@@ -27,6 +27,7 @@ SIGNATURES = {
     "elutq_hlq_gemv_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp]),
     "elutq_hlq_gemv_f16_tuned": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _ci, _ci]),
     "elutq_hlq_gemv_fused_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
+    "elutq_hlq_gemv_slices": (_ci, [_ci] * 6),
     "elutq_decode_rope_attn_f16": (_ci, [_vp] * 5 + [_ci] * 4 + [ctypes.c_float, _vp]),
     "elutq_decode_rope_attn_split_f16": (_ci, [_vp] * 5 + [_ci] * 4 + [ctypes.c_float, _ci, _vp, _sz, _vp]),
     "elutq_decode_attn_workspace_bytes": (_sz, [_ci] * 3),
@@ -53,7 +54,9 @@ SIGNATURES = {
 class GemvFusion(ctypes.Structure):
     """struct elutq_gemv_fusion of include/elutq_hip.h."""
     _fields_ = [("prologue", ctypes.c_int), ("eps", ctypes.c_float),
-                ("d_norm_weight", ctypes.c_void_p), ("d_residual", ctypes.c_void_p)]
+                ("d_norm_weight", ctypes.c_void_p), ("d_residual", ctypes.c_void_p),
+                ("d_slices_out", ctypes.c_void_p), ("d_slices_in", ctypes.c_void_p),
+                ("n_slices_in", ctypes.c_int), ("d_x_out", ctypes.c_void_p)]
 
 
 class GemvProblem(ctypes.Structure):

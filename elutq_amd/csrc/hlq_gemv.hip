@@ -67,6 +67,11 @@ struct GemvArgs {
     const HLQ_GLOBAL uint16_t *norm_w;  // fp16 [K]      (prologue 1)
     const HLQ_GLOBAL uint16_t *residual;  // fp16 [N] added to the output, or null
     const HLQ_GLOBAL float *extra;        // fp32 [N] added to the output before it is rounded, or null
+    // K slices handed to the next launch instead of being summed here, and the consuming side
+    int defer;                            // 1: write the slices' partial sums to `partial` and nothing else
+    int n_slices_in;                      // > 0: x = fp16(sum of slices_in in order + x), prologue 1 only
+    const HLQ_GLOBAL float *slices_in;    // fp32 [n_slices_in][K]
+    HLQ_GLOBAL uint16_t *x_out;           // fp16 [K] or null: the combined x, written by workgroup (0, 0)
 };
 
 #ifdef HLQ_TIMING
@@ -327,6 +332,35 @@ __device__ __forceinline__ void lds_barrier()
 // RSTD_SCRATCH floats.  Every workgroup does this for itself (2K bytes from cache).
 constexpr int RSTD_SCRATCH = 80;
 
+// Activations that arrive as a base vector plus the unsummed K slices of the launch that
+// produced them (its `defer` mode): element k is fp16(((s0[k] + s1[k]) + ...) + x[k]), the same
+// operations in the same order as that launch's own output stage would have used.
+constexpr int GEMV_MAX_SLICES_IN = 4;
+
+struct SliceChunk {
+    float4 p[GEMV_MAX_SLICES_IN];
+};
+
+__device__ __forceinline__ void load_slice_chunk(const GemvArgs &a, int K, int chunk, SliceChunk &c)
+{
+#pragma unroll
+    for (int s = 0; s < GEMV_MAX_SLICES_IN; s++)     // always GEMV_MAX_SLICES_IN loads: a fixed count
+        c.p[s] = *(const HLQ_GLOBAL float4 *)(a.slices_in + (size_t)min(s, a.n_slices_in - 1) * K + (size_t)chunk * 4);
+}
+
+__device__ __forceinline__ uint2 combine_chunk(const GemvArgs &a, uint2 base, const SliceChunk &c)
+{
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < GEMV_MAX_SLICES_IN; s++)
+        if (s < a.n_slices_in) { v[0] += c.p[s].x; v[1] += c.p[s].y; v[2] += c.p[s].z; v[3] += c.p[s].w; }
+    v[0] += h2f_lo(base.x); v[1] += h2f_hi(base.x); v[2] += h2f_lo(base.y); v[3] += h2f_hi(base.y);
+    auto pack = [](float lo, float hi) __attribute__((always_inline)) {
+        return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+    };
+    return make_uint2(pack(v[0], v[1]), pack(v[2], v[3]));
+}
+
 // The chunk of x this thread squares first; issued ahead of the other loads of the tile so that
 // the reduction below overlaps with them.
 __device__ __forceinline__ uint2 rstd_first_load(const GemvArgs &a, int K, int tid)
@@ -334,14 +368,33 @@ __device__ __forceinline__ uint2 rstd_first_load(const GemvArgs &a, int K, int t
     return *(const HLQ_GLOBAL uint2 *)(a.x + (size_t)min(tid, K / 4 - 1) * 4);
 }
 
-__device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scratch, int tid, int nthreads, uint2 first)
+// With slices (`stage` non-null) every chunk of the combined x is formed here once, kept in
+// `stage` (LDS, fp16 [K]) for the table builds and, by the first workgroup, written to a.x_out.
+__device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scratch, int tid, int nthreads, uint2 first,
+                                            const SliceChunk &sfirst, uint2 *stage, bool write_out)
 {
     auto sq4 = [](uint2 r) __attribute__((always_inline)) {
         const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
         return (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
     };
-    float ssq = tid < K / 4 ? sq4(first) : 0.f;
-    for (int i = tid + nthreads; i < K / 4; i += nthreads) ssq += sq4(*(const HLQ_GLOBAL uint2 *)(a.x + (size_t)i * 4));
+    float ssq = 0.f;
+    if (stage) {
+        for (int i = tid; i < K / 4; i += nthreads) {
+            uint2 r;
+            if (i == tid) r = combine_chunk(a, first, sfirst);
+            else {
+                SliceChunk c;
+                load_slice_chunk(a, K, i, c);
+                r = combine_chunk(a, *(const HLQ_GLOBAL uint2 *)(a.x + (size_t)i * 4), c);
+            }
+            stage[i] = r;
+            if (write_out) *(HLQ_GLOBAL uint2 *)(a.x_out + (size_t)i * 4) = r;
+            ssq += sq4(r);
+        }
+    } else {
+        ssq = tid < K / 4 ? sq4(first) : 0.f;
+        for (int i = tid + nthreads; i < K / 4; i += nthreads) ssq += sq4(*(const HLQ_GLOBAL uint2 *)(a.x + (size_t)i * 4));
+    }
     HLQ_ROW_REDUCE(ssq, op_add);
     if ((tid & 15) == 0) scratch[tid >> 4] = ssq;
     lds_barrier();
@@ -450,6 +503,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     }
     uint2 rfirst = make_uint2(0, 0);
     if (prologue == 1) rfirst = rstd_first_load(a, K, tid);
+    const bool sliced = !PLAIN && a.n_slices_in > 0;                       // host: only with prologue 1
+    SliceChunk sfirst = {};
+    uint2 *stage = sliced ? (uint2 *)(rstd_scratch + RSTD_SCRATCH + 4) : nullptr;   // fp16 [K]
+    if (sliced) load_slice_chunk(a, K, min(tid, K / 4 - 1), sfirst);
     uint2 raw, raw2;
     // lanes past the run (and waves without one, whose k0 is the end of the slice) re-read a valid chunk
     load_chunk<PLAIN>(a, prologue, K, nchunks ? k0 + (size_t)min(lane, nchunks - 1) * 4 : 0, raw, raw2);
@@ -462,7 +519,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         load_slot<BITS, G64, PAIRED, 0>(slot[0], here, u0, min(s_begin, s_last), lane);
     }
     asm volatile("" ::: "memory");
-    if (prologue == 1) rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst);
+    if (prologue == 1)
+        rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst, sfirst, stage,
+                          sliced && a.x_out && blockIdx.x == 0 && blockIdx.y == 0);
+    if (sliced) raw = stage[(k0 >> 2) + (nchunks ? min(lane, nchunks - 1) : 0)];   // the combined chunk replaces the base's
 
     // ... the tables are built as soon as the activations are in (a wave that first queued all
     // its weight loads would sit in the memory pipeline's back-pressure instead) ...
@@ -477,6 +537,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     });
     for (int ci = lane + 64; ci < nchunks; ci += 64) {      // runs of more than two units (not the common case)
         load_chunk<PLAIN>(a, prologue, K, k0 + (size_t)ci * 4, raw, raw2);
+        if (sliced) raw = stage[(k0 >> 2) + ci];
         build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0);
     }
     HLQ_STAMP(1);
@@ -520,6 +581,11 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         // waits for its stores to be acknowledged before it takes a ticket, and the reader's
         // loads depend on the ticket it drew -- so no cache write-back / invalidate is needed.
         const size_t npad = (size_t)a.ncb * HLQ_CB;
+        if (!PLAIN && a.defer) {
+            // the consumer is a later launch on the same stream: an ordinary store, no meeting
+            if (wave == fin) a.partial[(size_t)slice * npad + n] = total;
+            return;
+        }
         if (wave == fin) {
             __hip_atomic_store(&a.partial[(size_t)slice * npad + n], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -733,7 +799,8 @@ int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
         if (a.prologue != 0 || a.residual) return ELUTQ_ERR_TUNING;     // no instance reads both
         return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_EXTRA>(a, waves, lds, stream);
     }
-    if (a.prologue == 0 && !a.residual) return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_PLAIN>(a, waves, lds, stream);
+    if (a.prologue == 0 && !a.residual && !a.defer && a.n_slices_in == 0)      // the plain instances read none of these fields
+        return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_PLAIN>(a, waves, lds, stream);
     return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_FUSED>(a, waves, lds, stream);
 }
 
@@ -961,6 +1028,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     a.spw = wp.spw; a.nuw_max = wp.nuw_max; a.wave_lds = wp.wave_lds;
     a.partial = nullptr; a.counters = nullptr;
     a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
+    a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr;
     if (fusion) {
         if (fusion->prologue < 0 || fusion->prologue > 2) return ELUTQ_ERR_TUNING;
         if (fusion->prologue == 1 && !fusion->d_norm_weight) return ELUTQ_ERR_NULL;
@@ -970,7 +1038,24 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         a.residual = (const HLQ_GLOBAL uint16_t *)fusion->d_residual;
     }
     a.extra = (const HLQ_GLOBAL float *)d_extra;
-    if (ksplit > 1) {
+    size_t stage_bytes = 0;
+    if (fusion && fusion->n_slices_in != 0) {
+        // x arrives as a base vector plus the unsummed K slices of the launch that produced it
+        if (fusion->n_slices_in < 0 || fusion->n_slices_in > GEMV_MAX_SLICES_IN || fusion->prologue != 1) return ELUTQ_ERR_TUNING;
+        if (!fusion->d_slices_in) return ELUTQ_ERR_NULL;
+        a.n_slices_in = fusion->n_slices_in;
+        a.slices_in = (const HLQ_GLOBAL float *)fusion->d_slices_in;
+        if (fusion->d_x_out == d_x) return ELUTQ_ERR_TUNING;       // other workgroups still read the base
+        a.x_out = (HLQ_GLOBAL uint16_t *)fusion->d_x_out;
+        stage_bytes = (size_t)K * sizeof(uint16_t);
+        if (gemv_lds_bytes(ups, bits, waves) + stage_bytes > (size_t)MAX_LDS) return ELUTQ_ERR_SHAPE;
+    }
+    if (fusion && fusion->d_slices_out) {
+        // the K slices stay unsummed for the next launch: nothing else may be due in the output stage
+        if (ksplit < 2 || d_bias || a.residual || d_extra || N % HLQ_CB != 0) return ELUTQ_ERR_TUNING;
+        a.defer = 1;
+        a.partial = (HLQ_GLOBAL float *)fusion->d_slices_out;
+    } else if (ksplit > 1) {
         if (!d_workspace) return ELUTQ_ERR_NULL;
         if ((size_t)g.ncb * sizeof(unsigned) > (size_t)WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
         if (workspace_bytes < (size_t)WS_COUNTER_BYTES + (size_t)ksplit * g.ncb * HLQ_CB * sizeof(float))
@@ -978,7 +1063,18 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         a.counters = (HLQ_GLOBAL unsigned *)d_workspace;
         a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
-    return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves), (hipStream_t)stream);
+    return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves) + stage_bytes, (hipStream_t)stream);
+}
+
+extern "C" int elutq_hlq_gemv_slices(int K, int N, int bits, int group, int ksplit, int waves)
+{
+    if (check_shape(K, N, bits, group) != ELUTQ_OK) return 0;
+    const HlqGeo g = hlq_geo(K, N, bits, group);
+    if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return 0;
+    choose_shape(g, ksplit, waves);                      // the same steps as the launch itself
+    int ups = (g.U + ksplit - 1) / ksplit;
+    while (gemv_lds_bytes(ups, bits, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
+    return (g.U + ups - 1) / ups;
 }
 
 extern "C" {
@@ -1095,6 +1191,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
             a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + poff[i]);
         }
         a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
+        a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr;
         const int ns = a.spw < depth_of(bits) ? a.spw : depth_of(bits);
         if (ns > nslot) nslot = ns;
         const size_t l = gemv_lds_bytes(sh.ups, bits, 16);

@@ -264,17 +264,31 @@ class HLQLinear(nn.Module):
 
     def gemv_fused(self, x: torch.Tensor, out: torch.Tensor, ws: torch.Tensor, prologue: int = 0,
                    norm_weight: torch.Tensor | None = None, eps: float = 0.0,
-                   residual: torch.Tensor | None = None) -> torch.Tensor:
+                   residual: torch.Tensor | None = None, slices_out: torch.Tensor | None = None,
+                   slices_in: torch.Tensor | None = None, x_out: torch.Tensor | None = None) -> torch.Tensor:
         """Batch-1 GEMV into a caller-owned `out`, optionally fused with the RMSNorm in front of
         the projection (prologue 1), the SiLU(gate)*up in front of it (prologue 2; x holds 2K
         values) and a residual added to the result.  No allocation: `ws` is the caller's
         zero-initialised workspace.  See elutq_hlq_gemv_fused_f16 in include/elutq_hip.h.
+        `slices_out` (fp32 [self.slices, N]): the K slices are left unsummed there and `out` is
+        not written; `slices_in` (fp32 [S, K], prologue 1): x is the sum of those slices plus `x`,
+        rounded to fp16 (what the producer would have written with residual = x), and `x_out`
+        receives it.
         A layer with a sparse extra plane cannot be fused (the plane reads the projection's own
         input, which a prologue only forms inside the kernel): use forward()."""
         if self.sparse_count:
             raise NotImplementedError("a layer with a sparse extra plane has no fused GEMV; call forward()")
         f = _lib.GemvFusion(prologue, eps, norm_weight.data_ptr() if norm_weight is not None else None,
-                            residual.data_ptr() if residual is not None else None)
+                            residual.data_ptr() if residual is not None else None,
+                            slices_out.data_ptr() if slices_out is not None else None,
+                            slices_in.data_ptr() if slices_in is not None else None,
+                            slices_in.shape[0] if slices_in is not None else 0,
+                            x_out.data_ptr() if x_out is not None else None)
+        if slices_out is not None and (slices_out.dtype != torch.float32 or slices_out.numel() < self.slices * self.out_features):
+            raise ValueError("slices_out must be fp32 [slices, out_features]")
+        if slices_in is not None and (slices_in.dtype != torch.float32 or slices_in.dim() != 2
+                                      or slices_in.shape[1] != self.in_features or not slices_in.is_contiguous()):
+            raise ValueError("slices_in must be contiguous fp32 [S, in_features]")
         rc = _lib.lib().elutq_hlq_gemv_fused_f16(
             self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
             self.bias.data_ptr() if self.bias is not None else None, x.data_ptr(), out.data_ptr(),
@@ -286,6 +300,12 @@ class HLQLinear(nn.Module):
     @property
     def workspace_bytes(self) -> int:
         return self._ws_bytes
+
+    @property
+    def slices(self) -> int:
+        """K slices across workgroups of this layer's batch-1 launch (1 = none)."""
+        return _lib.lib().elutq_hlq_gemv_slices(self.in_features, self.out_features, self.bits, self.group_size,
+                                                self.ksplit, self.waves)
 
     def dequantize(self) -> torch.Tensor:
         """Dense fp16 W [N, K] (``dequantize_with_scales``, GPTQ/quant.py:176-183)."""

@@ -141,6 +141,41 @@ class FusedBuffers:
         self.gu = torch.zeros(1, 2 * s.ffn, **f16)
         self.ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=device)
         self.logits = torch.zeros(1, s.vocab, **f16)
+        # unsummed K slices of a down projection, read by the next layer's first launch
+        self.sd = torch.zeros(MAX_DEFERRED_SLICES, s.hidden, dtype=torch.float32, device=device)
+
+
+MAX_DEFERRED_SLICES = 4        # what a consuming launch accepts (elutq_gemv_fusion.n_slices_in)
+
+
+def deferred_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tensor, cur: torch.Tensor,
+                        other: torch.Tensor, pending: int, last: bool):
+    """The same five launches with the K slices of the down projection left unsummed for the launch
+    that reads them (the next layer's q|k|v), which forms fp16(slices + residual) itself, bit for
+    bit what the producer's own output stage writes, and stores it for the later residual add.
+    `cur` holds the residual stream, `other` is free; `pending` = slices of the previous layer's
+    down waiting in b.sd (0 = none).  Returns (cur, other, pending)."""
+    s = layer.s
+    if pending:
+        layer.qkv.gemv_fused(cur, b.qkv, b.ws, prologue=1, norm_weight=layer.ln1, eps=s.rms_eps,
+                             slices_in=b.sd[:pending], x_out=other)
+        cur, other = other, cur
+    else:
+        layer.qkv.gemv_fused(cur, b.qkv, b.ws, prologue=1, norm_weight=layer.ln1, eps=s.rms_eps)
+    rc = _lib.lib().elutq_decode_rope_attn_split_f16(
+        b.qkv.data_ptr(), layer.k_cache.data_ptr(), layer.v_cache.data_ptr(), pos.data_ptr(), b.attn.data_ptr(),
+        s.n_heads, s.n_kv_heads, s.head_dim, s.max_seq, s.rope_base, 0, b.ws.data_ptr(), b.ws.numel(),
+        torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "elutq_decode_rope_attn_split_f16")
+    layer.o_proj.gemv_fused(b.attn, other, b.ws, residual=cur)
+    layer.gate_up.gemv_fused(other, b.gu, b.ws, prologue=1, norm_weight=layer.ln2, eps=s.rms_eps)
+    cur, other = other, cur
+    n_d = layer.down_proj.slices
+    if not last and 2 <= n_d <= MAX_DEFERRED_SLICES and layer.down_proj.bias is None:
+        layer.down_proj.gemv_fused(b.gu, other, b.ws, prologue=2, slices_out=b.sd)
+        return cur, other, n_d
+    layer.down_proj.gemv_fused(b.gu, other, b.ws, prologue=2, residual=cur)
+    return other, cur, 0
 
 
 def fused_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tensor) -> None:
@@ -267,6 +302,9 @@ class LlamaDecoder(nn.Module):
         self.register_buffer("pos", torch.zeros(1, dtype=torch.long, device=dev))
         self._graph = None
         self._buf = None
+        # leave the K slices of down to the launch that reads them (deferred_layer_step); the
+        # logits are bit for bit those of fused_layer_step.  Set before capture().
+        self.defer_slices = True
         if impl == "hip":
             if any(m.sparse_count for m in self.modules() if isinstance(m, HLQLinear)):
                 raise NotImplementedError("the fused decode step takes no sparse extra plane held as blocks: load the "
@@ -301,9 +339,15 @@ class LlamaDecoder(nn.Module):
         if self.impl == "hip":
             b = self._buf
             torch.index_select(self.embed, 0, self.token, out=b.xa)
-            for layer in self.layers:
-                fused_layer_step(layer, b, self.pos)
-            x = b.xa
+            if self.defer_slices:
+                x, free, pending = b.xa, b.xb, 0
+                for i, layer in enumerate(self.layers):
+                    x, free, pending = deferred_layer_step(layer, b, self.pos, x, free, pending,
+                                                           last=i == len(self.layers) - 1)
+            else:
+                for layer in self.layers:
+                    fused_layer_step(layer, b, self.pos)
+                x, free = b.xa, b.xb
         else:
             x = self.embed.index_select(0, self.token)
             cos = self.cos_t.index_select(0, self.pos)
@@ -317,9 +361,9 @@ class LlamaDecoder(nn.Module):
                 logits = self.lm_head_q.gemv_fused(x, b.logits, b.ws, prologue=1, norm_weight=self.norm,
                                                    eps=self.s.rms_eps)
             else:
-                _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), b.xb.data_ptr(),
+                _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), free.data_ptr(),
                                                       self.s.hidden, self.s.rms_eps, stream), "elutq_decode_rmsnorm_f16")
-                logits = torch.mm(b.xb, self.lm_head.t(), out=b.logits)
+                logits = torch.mm(free, self.lm_head.t(), out=b.logits)
             _lib.check(L.elutq_decode_argmax_ws_f16(logits.data_ptr(), self.s.vocab, self.token.data_ptr(),
                                                     self.pos.data_ptr(), b.ws.data_ptr(), b.ws.numel(), stream),
                        "elutq_decode_argmax_ws_f16")

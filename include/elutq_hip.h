@@ -120,13 +120,33 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
  *                                                       norm in the reference (arm_rmsnorm.cpp:43-85)
  * `fusion` is a HOST pointer (read before the call returns) or NULL for a plain GEMV.
  * ksplit / waves as in elutq_hlq_gemv_f16_tuned.
+ *
+ * A projection whose K is divided among workgroups can leave the sum of its K slices to the
+ * projection that reads its output (in a decoder layer: o -> gate|up, down -> the next
+ * layer's q|k|v), which saves the producing launch the meeting of its slices in device memory:
+ *   producer  d_slices_out = fp32 [S][N], S = elutq_hlq_gemv_slices(K, N, bits, group, ksplit, waves) >= 2,
+ *             N % 64 == 0: every slice's partial sums are stored there and d_y is NOT written;
+ *             no bias and no d_residual (the consumer adds the residual)
+ *   consumer  prologue 1 with n_slices_in = S (at most 4), d_slices_in = that buffer (row stride K),
+ *             d_x = the residual: x <- fp16(((s0 + s1) + ...) + d_x) element by element, i.e. what
+ *             the producer would have written with d_residual = d_x, bit for bit; the RMSNorm
+ *             follows.  d_x_out (fp16 [K], or NULL; not d_x) receives that x for later readers.
+ * No counterpart in the reference, whose operators run one after the other on whole vectors.
  */
 typedef struct elutq_gemv_fusion {
     int prologue;               /* 0, 1 or 2 */
     float eps;                  /* RMSNorm epsilon (prologue 1) */
     const void *d_norm_weight;  /* fp16 [K] (prologue 1) */
     const void *d_residual;     /* fp16 [N] or NULL */
+    void *d_slices_out;         /* producer of deferred K slices, or NULL */
+    const void *d_slices_in;    /* consumer of deferred K slices (n_slices_in > 0) */
+    int n_slices_in;            /* 0 = none */
+    void *d_x_out;              /* fp16 [K] or NULL (consumer only) */
 } elutq_gemv_fusion;
+
+/* K slices the GEMV launch of this shape is divided into (ksplit / waves as in
+ * elutq_hlq_gemv_f16_tuned, 0 = default); 0 for an unsupported shape or tuning. */
+int elutq_hlq_gemv_slices(int K, int N, int bits, int group, int ksplit, int waves);
 
 int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
                              const void *d_bias, const void *d_x, void *d_y,
