@@ -368,17 +368,17 @@ __device__ __forceinline__ uint2 rstd_first_load(const GemvArgs &a, int K, int t
     return *(const HLQ_GLOBAL uint2 *)(a.x + (size_t)min(tid, K / 4 - 1) * 4);
 }
 
-// With slices (`stage` non-null) every chunk of the combined x is formed here once, kept in
+// With slices (`sliced`) every chunk of the combined x is formed here once, kept in
 // `stage` (LDS, fp16 [K]) for the table builds and, by the first workgroup, written to a.x_out.
 __device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scratch, int tid, int nthreads, uint2 first,
-                                            const SliceChunk &sfirst, uint2 *stage, bool write_out)
+                                            const SliceChunk &sfirst, bool sliced, uint2 *stage, bool write_out)
 {
     auto sq4 = [](uint2 r) __attribute__((always_inline)) {
         const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
         return (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
     };
     float ssq = 0.f;
-    if (stage) {
+    if (sliced) {
         for (int i = tid; i < K / 4; i += nthreads) {
             uint2 r;
             if (i == tid) r = combine_chunk(a, first, sfirst);
@@ -505,7 +505,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     if (prologue == 1) rfirst = rstd_first_load(a, K, tid);
     const bool sliced = !PLAIN && a.n_slices_in > 0;                       // host: only with prologue 1
     SliceChunk sfirst = {};
-    uint2 *stage = sliced ? (uint2 *)(rstd_scratch + RSTD_SCRATCH + 4) : nullptr;   // fp16 [K]
+    // fp16 [K] behind the reduction scratch when `sliced` (not selected against a null pointer: the
+    // accesses must stay LDS instructions, a generic access would also count as a vector-memory one
+    // and wait behind the weight loads in flight)
+    uint2 *stage = (uint2 *)(rstd_scratch + RSTD_SCRATCH + 4);
     if (sliced) load_slice_chunk(a, K, min(tid, K / 4 - 1), sfirst);
     uint2 raw, raw2;
     // lanes past the run (and waves without one, whose k0 is the end of the slice) re-read a valid chunk
@@ -520,7 +523,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     }
     asm volatile("" ::: "memory");
     if (prologue == 1)
-        rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst, sfirst, stage,
+        rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst, sfirst, sliced, stage,
                           sliced && a.x_out && blockIdx.x == 0 && blockIdx.y == 0);
     if (sliced) raw = stage[(k0 >> 2) + (nchunks ? min(lane, nchunks - 1) : 0)];   // the combined chunk replaces the base's
 
