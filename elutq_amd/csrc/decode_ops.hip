@@ -23,9 +23,40 @@ struct AttnArgs {
     int splits;              // workgroups per query head (head_dim 128 only)
     float *partial;          // [nq][splits][d + 2] unnormalised output, running max, running sum
     unsigned *counters;      // [nq] arrival counters, zero between launches
+    const float *qkv_slices; // fp32 [n_qkv_slices][qkv_stride]: the q|k|v projection's K slices, unsummed, or null
+    int n_qkv_slices, qkv_stride;
 };
 
 constexpr int ATTN_MAX_SPLITS = 8;
+constexpr int ATTN_MAX_QKV_SLICES = 4;
+
+// The six q|k|v elements a lane needs (indices idx[]): as stored (fp16), or fp16(((s0[i] + s1[i]) + ...))
+// where the projection left its K slices unsummed -- the value its own output stage would have stored.
+// One branch, then all loads of the taken side before the first use (ATTN_MAX_QKV_SLICES per element in
+// the second case, the last slice repeated, none of them conditional).
+__device__ __forceinline__ void qkv_elems(const AttnArgs &a, const int (&idx)[6], uint16_t (&out)[6])
+{
+    if (a.n_qkv_slices == 0) {
+#pragma unroll
+        for (int e = 0; e < 6; e++) out[e] = a.qkv[idx[e]];
+        return;
+    }
+    float v[6][ATTN_MAX_QKV_SLICES];
+#pragma unroll
+    for (int s = 0; s < ATTN_MAX_QKV_SLICES; s++) {
+        const float *row = a.qkv_slices + (size_t)min(s, a.n_qkv_slices - 1) * a.qkv_stride;
+#pragma unroll
+        for (int e = 0; e < 6; e++) v[e][s] = row[idx[e]];
+    }
+#pragma unroll
+    for (int e = 0; e < 6; e++) {
+        float sum = v[e][0];
+#pragma unroll
+        for (int s = 1; s < ATTN_MAX_QKV_SLICES; s++)
+            if (s < a.n_qkv_slices) sum += v[e][s];
+        out[e] = __builtin_bit_cast(uint16_t, (_Float16)sum);
+    }
+}
 
 __device__ __forceinline__ float h2f(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
 __device__ __forceinline__ uint16_t f2h(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
@@ -222,10 +253,11 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     }
     // every wave loads the rotary pair (lane, lane + 64) of q, k and v (only wave 0 uses it):
     // unconditional, so that nothing is converted -- and therefore waited for -- in between
-    const uint16_t *qp = a.qkv + (size_t)h * D, *kp = a.qkv + (size_t)a.nq * D + (size_t)g * D;
-    const uint16_t *vp = a.qkv + (size_t)(a.nq + a.nkv) * D + (size_t)g * D;
-    const uint16_t qa16 = qp[lane], qb16 = qp[lane + HALF], ka16 = kp[lane], kb16 = kp[lane + HALF];
-    const uint16_t va16 = vp[lane], vb16 = vp[lane + HALF];
+    const int qi = h * D, ki = a.nq * D + g * D, vi = (a.nq + a.nkv) * D + g * D;
+    const int idx[6] = {qi + lane, qi + lane + HALF, ki + lane, ki + lane + HALF, vi + lane, vi + lane + HALF};
+    uint16_t el[6];
+    qkv_elems(a, idx, el);
+    const uint16_t qa16 = el[0], qb16 = el[1], ka16 = el[2], kb16 = el[3], va16 = el[4], vb16 = el[5];
     asm volatile("" ::: "memory");
     const int pos = (int)pos64;
     if (pos64 < 0 || pos64 >= a.max_seq) return;
@@ -537,11 +569,19 @@ extern "C" int elutq_debug_set_attn_stamps(void *d_buf)
 }
 #endif
 
-extern "C" int elutq_decode_rope_attn_split_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,
-                                                void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,
-                                                float rope_base, int splits, void *d_workspace, size_t workspace_bytes,
-                                                void *stream)
+// d_qkv_slices non-null: q|k|v arrives as n_qkv_slices unsummed K slices (fp32 rows of qkv_stride floats)
+static int launch_rope_attn(const void *d_qkv, const void *d_qkv_slices, int n_qkv_slices, int qkv_stride,
+                            void *d_k_cache, void *d_v_cache, const void *d_pos,
+                            void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                            float rope_base, int splits, void *d_workspace, size_t workspace_bytes,
+                            void *stream)
 {
+    if (d_qkv_slices) {
+        if (head_dim != FAST_D || n_qkv_slices < 1 || n_qkv_slices > ATTN_MAX_QKV_SLICES ||
+            qkv_stride < (n_heads + 2 * n_kv_heads) * head_dim)
+            return ELUTQ_ERR_TUNING;
+        d_qkv = d_qkv_slices;                            // (only checked against null below)
+    }
     if (!d_qkv || !d_k_cache || !d_v_cache || !d_pos || !d_out) return ELUTQ_ERR_NULL;
     if (n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads != 0 || head_dim < 2 || head_dim > 128 ||
         head_dim % 2 != 0 || max_seq < 1 || !(rope_base > 1.f))
@@ -561,6 +601,7 @@ extern "C" int elutq_decode_rope_attn_split_f16(const void *d_qkv, void *d_k_cac
     a.out = (uint16_t *)d_out;
     a.nq = n_heads; a.nkv = n_kv_heads; a.d = head_dim; a.max_seq = max_seq;
     a.log2_base = log2f(rope_base);
+    a.qkv_slices = (const float *)d_qkv_slices; a.n_qkv_slices = d_qkv_slices ? n_qkv_slices : 0; a.qkv_stride = qkv_stride;
     a.splits = splits; a.partial = nullptr; a.counters = nullptr;
     if (splits > 1) {
         if (!d_workspace) return ELUTQ_ERR_NULL;
@@ -576,6 +617,25 @@ extern "C" int elutq_decode_rope_attn_split_f16(const void *d_qkv, void *d_k_cac
     else
         hipLaunchKernelGGL((rope_attn_d128_kernel<4, 4>), dim3(n_heads * splits), dim3(4 * 64), 0, (hipStream_t)stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
+}
+
+extern "C" int elutq_decode_rope_attn_split_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,
+                                                void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,
+                                                float rope_base, int splits, void *d_workspace, size_t workspace_bytes,
+                                                void *stream)
+{
+    return launch_rope_attn(d_qkv, nullptr, 0, 0, d_k_cache, d_v_cache, d_pos, d_out, n_heads, n_kv_heads, head_dim, max_seq,
+                            rope_base, splits, d_workspace, workspace_bytes, stream);
+}
+
+extern "C" int elutq_decode_rope_attn_sliced_f16(const void *d_qkv_slices, int n_slices, int slice_stride, void *d_k_cache,
+                                                 void *d_v_cache, const void *d_pos, void *d_out, int n_heads,
+                                                 int n_kv_heads, int head_dim, int max_seq, float rope_base, int splits,
+                                                 void *d_workspace, size_t workspace_bytes, void *stream)
+{
+    if (!d_qkv_slices) return ELUTQ_ERR_NULL;
+    return launch_rope_attn(nullptr, d_qkv_slices, n_slices, slice_stride, d_k_cache, d_v_cache, d_pos, d_out, n_heads,
+                            n_kv_heads, head_dim, max_seq, rope_base, splits, d_workspace, workspace_bytes, stream);
 }
 
 extern "C" int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,

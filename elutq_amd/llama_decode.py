@@ -141,6 +141,8 @@ class FusedBuffers:
         self.gu = torch.zeros(1, 2 * s.ffn, **f16)
         self.ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=device)
         self.logits = torch.zeros(1, s.vocab, **f16)
+        # unsummed K slices of a q|k|v projection, read by the attention launch
+        self.sq = torch.zeros(MAX_DEFERRED_SLICES, self.qkv.shape[1], dtype=torch.float32, device=device)
         # unsummed K slices of a down projection, read by the next layer's first launch
         self.sd = torch.zeros(MAX_DEFERRED_SLICES, s.hidden, dtype=torch.float32, device=device)
 
@@ -149,24 +151,34 @@ MAX_DEFERRED_SLICES = 4        # what a consuming launch accepts (elutq_gemv_fus
 
 
 def deferred_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tensor, cur: torch.Tensor,
-                        other: torch.Tensor, pending: int, last: bool):
+                        other: torch.Tensor, pending: int, last: bool, defer_qkv: bool = True):
     """The same five launches with the K slices of the down projection left unsummed for the launch
     that reads them (the next layer's q|k|v), which forms fp16(slices + residual) itself, bit for
     bit what the producer's own output stage writes, and stores it for the later residual add.
     `cur` holds the residual stream, `other` is free; `pending` = slices of the previous layer's
-    down waiting in b.sd (0 = none).  Returns (cur, other, pending)."""
+    down waiting in b.sd (0 = none).  Returns (cur, other, pending).  `defer_qkv`: the q|k|v
+    projection's K slices go to the attention launch the same way (head_dim 128), where a
+    workgroup only sums the 3 x 128 elements of its own head."""
     s = layer.s
+    n_q = layer.qkv.slices
+    defer_qkv = defer_qkv and s.head_dim == 128 and 2 <= n_q <= MAX_DEFERRED_SLICES and layer.qkv.bias is None
+    layer.qkv.gemv_fused(cur, b.qkv, b.ws, prologue=1, norm_weight=layer.ln1, eps=s.rms_eps,
+                         slices_in=b.sd[:pending] if pending else None, x_out=other if pending else None,
+                         slices_out=b.sq if defer_qkv else None)
     if pending:
-        layer.qkv.gemv_fused(cur, b.qkv, b.ws, prologue=1, norm_weight=layer.ln1, eps=s.rms_eps,
-                             slices_in=b.sd[:pending], x_out=other)
         cur, other = other, cur
+    L, stream = _lib.lib(), torch.cuda.current_stream().cuda_stream
+    if defer_qkv:
+        rc = L.elutq_decode_rope_attn_sliced_f16(
+            b.sq.data_ptr(), n_q, b.sq.shape[1], layer.k_cache.data_ptr(), layer.v_cache.data_ptr(), pos.data_ptr(),
+            b.attn.data_ptr(), s.n_heads, s.n_kv_heads, s.head_dim, s.max_seq, s.rope_base, 0, b.ws.data_ptr(),
+            b.ws.numel(), stream)
+        _lib.check(rc, "elutq_decode_rope_attn_sliced_f16")
     else:
-        layer.qkv.gemv_fused(cur, b.qkv, b.ws, prologue=1, norm_weight=layer.ln1, eps=s.rms_eps)
-    rc = _lib.lib().elutq_decode_rope_attn_split_f16(
-        b.qkv.data_ptr(), layer.k_cache.data_ptr(), layer.v_cache.data_ptr(), pos.data_ptr(), b.attn.data_ptr(),
-        s.n_heads, s.n_kv_heads, s.head_dim, s.max_seq, s.rope_base, 0, b.ws.data_ptr(), b.ws.numel(),
-        torch.cuda.current_stream().cuda_stream)
-    _lib.check(rc, "elutq_decode_rope_attn_split_f16")
+        rc = L.elutq_decode_rope_attn_split_f16(
+            b.qkv.data_ptr(), layer.k_cache.data_ptr(), layer.v_cache.data_ptr(), pos.data_ptr(), b.attn.data_ptr(),
+            s.n_heads, s.n_kv_heads, s.head_dim, s.max_seq, s.rope_base, 0, b.ws.data_ptr(), b.ws.numel(), stream)
+        _lib.check(rc, "elutq_decode_rope_attn_split_f16")
     layer.o_proj.gemv_fused(b.attn, other, b.ws, residual=cur)
     layer.gate_up.gemv_fused(other, b.gu, b.ws, prologue=1, norm_weight=layer.ln2, eps=s.rms_eps)
     cur, other = other, cur
@@ -305,6 +317,7 @@ class LlamaDecoder(nn.Module):
         # leave the K slices of down to the launch that reads them (deferred_layer_step); the
         # logits are bit for bit those of fused_layer_step.  Set before capture().
         self.defer_slices = True
+        self.defer_qkv = True              # likewise q|k|v -> attention (takes effect where q|k|v is K-sliced)
         if impl == "hip":
             if any(m.sparse_count for m in self.modules() if isinstance(m, HLQLinear)):
                 raise NotImplementedError("the fused decode step takes no sparse extra plane held as blocks: load the "
@@ -313,6 +326,14 @@ class LlamaDecoder(nn.Module):
             ws = max(m.workspace_bytes for m in self.modules() if isinstance(m, HLQLinear))
             ws = max(ws, _lib.lib().elutq_decode_attn_workspace_bytes(s.n_heads, s.head_dim, 0))
             self._buf = FusedBuffers(s, ws, dev)
+            # q|k|v in two K slices where that still leaves at most one workgroup per compute unit: the
+            # attention launch sums the slices of its own head for free, so the projection gets twice
+            # the workgroups without the meeting that otherwise makes the split a loss
+            # (LLaMA-3-8B: 96 -> 192 workgroups, 6.7 -> 5.7 us)
+            for layer in self.layers:
+                q = layer.qkv
+                if d == 128 and q.bias is None and q.slices == 1 and 2 * ((q.out_features + 63) // 64) <= 256:
+                    q.ksplit, q.waves = 2, 16
 
     @classmethod
     def from_export(cls, root: str, s: LlamaShape, device="cuda", fuse: bool = True, impl: str = "hip",
@@ -343,7 +364,7 @@ class LlamaDecoder(nn.Module):
                 x, free, pending = b.xa, b.xb, 0
                 for i, layer in enumerate(self.layers):
                     x, free, pending = deferred_layer_step(layer, b, self.pos, x, free, pending,
-                                                           last=i == len(self.layers) - 1)
+                                                           last=i == len(self.layers) - 1, defer_qkv=self.defer_qkv)
             else:
                 for layer in self.layers:
                     fused_layer_step(layer, b, self.pos)

@@ -235,6 +235,19 @@ int elutq_decode_rope_attn_split_f16(const void *d_qkv, void *d_k_cache, void *d
                                      void *stream);
 
 /*
+ * The same operator reading q|k|v as the unsummed K slices of the projection that produced it
+ * (elutq_gemv_fusion.d_slices_out of that launch: fp32 rows of slice_stride floats, n_slices 1..4):
+ * every element is fp16(((s0 + s1) + ...)), bit for bit what the projection would have stored.  A
+ * workgroup reads only its own head's 3 x 128 elements, so the sum costs it next to nothing, while
+ * the projection is spared the meeting of its slices in device memory.  head_dim 128 only.
+ * No counterpart in the reference.
+ */
+int elutq_decode_rope_attn_sliced_f16(const void *d_qkv_slices, int n_slices, int slice_stride, void *d_k_cache,
+                                      void *d_v_cache, const void *d_pos, void *d_out, int n_heads,
+                                      int n_kv_heads, int head_dim, int max_seq, float rope_base, int splits,
+                                      void *d_workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Tail of a decode step.  elutq_decode_rmsnorm_f16: out[i] = fp16(x[i] * rsqrt(mean(x^2) + eps)
  * * weight[i]), statistics in fp32 (launch_pre_rms_norm, C++/ops/src/arm/arm_rmsnorm.cpp:25-84).
  * elutq_decode_argmax_f16: *d_token (DEVICE int64) = first index of the strict maximum of the

@@ -102,3 +102,92 @@ def test_decode_step_is_bit_identical_with_deferred_slices(cuda, graph):
     assert runs[False][1] == runs[True][1]
     assert all(torch.equal(a, b) for a, b in zip(runs[False][0], runs[True][0]))
     assert torch.equal(runs[False][2], runs[True][2])
+
+
+@pytest.mark.parametrize("n_slices", [1, 2, 4])
+@pytest.mark.parametrize("pos,splits", [(0, 0), (37, 0), (250, 0), (900, 0), (250, 1), (600, 3)])
+def test_attention_reads_unsummed_qkv_slices(cuda, n_slices, pos, splits):
+    """elutq_decode_rope_attn_sliced_f16 on fp32 slices == elutq_decode_rope_attn_split_f16 on the fp16
+    vector a projection would have stored (slices summed in order, rounded once): output and appended
+    cache rows bit for bit."""
+    L = _lib.lib()
+    nq, nkv, d, max_seq, base = 8, 2, 128, 1024, 500000.0
+    g = torch.Generator(device=cuda).manual_seed(pos + n_slices)
+    width = (nq + 2 * nkv) * d
+    stride = width + 64                                   # rows may be longer than the vector
+    slices = torch.randn(n_slices, stride, generator=g, device=cuda)
+    tot = slices[0, :width].clone()
+    for s in range(1, n_slices):
+        tot += slices[s, :width]
+    qkv = tot.half().view(1, width)
+    kc0 = torch.randn(max_seq, nkv, d, generator=g, device=cuda).half()
+    vc0 = torch.randn(max_seq, nkv, d, generator=g, device=cuda).half()
+    pos_t = torch.tensor([pos], dtype=torch.long, device=cuda)
+    ws = torch.zeros(L.elutq_decode_attn_workspace_bytes(nq, d, 0), dtype=torch.uint8, device=cuda)
+    stream = torch.cuda.current_stream().cuda_stream
+    res = []
+    for sliced in (False, True):
+        kc, vc = kc0.clone(), vc0.clone()
+        out = torch.zeros(1, nq * d, dtype=torch.float16, device=cuda)
+        if sliced:
+            rc = L.elutq_decode_rope_attn_sliced_f16(slices.data_ptr(), n_slices, stride, kc.data_ptr(), vc.data_ptr(),
+                                                     pos_t.data_ptr(), out.data_ptr(), nq, nkv, d, max_seq, base, splits,
+                                                     ws.data_ptr(), ws.numel(), stream)
+        else:
+            rc = L.elutq_decode_rope_attn_split_f16(qkv.data_ptr(), kc.data_ptr(), vc.data_ptr(), pos_t.data_ptr(),
+                                                    out.data_ptr(), nq, nkv, d, max_seq, base, splits, ws.data_ptr(),
+                                                    ws.numel(), stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        res.append((out, kc, vc))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1]) and torch.equal(res[0][2], res[1][2])
+    assert not ws[:64 * 1024].any()
+
+
+def test_sliced_attention_argument_errors(cuda):
+    L = _lib.lib()
+    nq, nkv, max_seq = 4, 2, 64
+    buf = torch.zeros(8, 2048, device=cuda)
+    kc = torch.zeros(max_seq, nkv, 128, dtype=torch.float16, device=cuda)
+    pos_t = torch.zeros(1, dtype=torch.long, device=cuda)
+    out = torch.zeros(1, nq * 128, dtype=torch.float16, device=cuda)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call(n_slices, stride, d=128, slices=buf):
+        return L.elutq_decode_rope_attn_sliced_f16(slices.data_ptr() if slices is not None else None, n_slices, stride,
+                                                   kc.data_ptr(), kc.data_ptr(), pos_t.data_ptr(), out.data_ptr(), nq, nkv, d,
+                                                   max_seq, 10000.0, 1, None, 0, stream)
+    assert call(2, 2048) == 0
+    assert call(0, 2048) != 0 and call(5, 2048) != 0      # 1..4 slices
+    assert call(2, 1000) != 0                             # rows shorter than q|k|v
+    assert call(2, 2048, d=64) != 0                       # head_dim 128 only
+    assert call(2, 2048, slices=None) != 0
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("graph", [False, True])
+def test_decode_step_is_bit_identical_with_qkv_slices_left_to_attention(cuda, graph):
+    """head_dim 128, a context long enough for several attention splits; the q|k|v projection keeps
+    its K slices either way, so only where they are summed differs."""
+    shape = LlamaShape(n_layers=2, hidden=1024, n_heads=8, n_kv_heads=2, ffn=2048, vocab=2000, max_seq=320)
+    runs = {}
+    for defer in (False, True):
+        m = LlamaDecoder(shape, device=cuda, seed=3)
+        m.defer_qkv = defer
+        assert 2 <= m.layers[0].qkv.slices <= 4
+        m.fill_cache(250)
+        m.token.fill_(5)
+        if graph:
+            m.capture()
+        logits, toks = [], []
+        for _ in range(4):
+            if graph:
+                m.replay()
+                logits.append(m._buf.logits.clone())
+            else:
+                logits.append(m.step().clone())
+            toks.append(int(m.token))
+        runs[defer] = (logits, toks, m.layers[1].k_cache[250:254].clone())
+    assert runs[False][1] == runs[True][1]
+    assert all(torch.equal(a, b) for a, b in zip(runs[False][0], runs[True][0]))
+    assert torch.equal(runs[False][2], runs[True][2])
