@@ -34,11 +34,16 @@ constexpr int ATTN_MAX_QKV_SLICES = 4;
 // where the projection left its K slices unsummed -- the value its own output stage would have stored.
 // One branch, then all loads of the taken side before the first use (ATTN_MAX_QKV_SLICES per element in
 // the second case, the last slice repeated, none of them conditional).
-__device__ __forceinline__ void qkv_elems(const AttnArgs &a, const int (&idx)[6], uint16_t (&out)[6])
+__device__ __forceinline__ void qkv_elems(const AttnArgs &a, const int (&idx)[6], bool needed, uint16_t (&out)[6])
 {
     if (a.n_qkv_slices == 0) {
 #pragma unroll
         for (int e = 0; e < 6; e++) out[e] = a.qkv[idx[e]];
+        return;
+    }
+    if (!needed) {                                       // wave-uniform: only the wave that rotates q and k sums slices
+#pragma unroll
+        for (int e = 0; e < 6; e++) out[e] = 0;
         return;
     }
     float v[6][ATTN_MAX_QKV_SLICES];
@@ -256,7 +261,7 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     const int qi = h * D, ki = a.nq * D + g * D, vi = (a.nq + a.nkv) * D + g * D;
     const int idx[6] = {qi + lane, qi + lane + HALF, ki + lane, ki + lane + HALF, vi + lane, vi + lane + HALF};
     uint16_t el[6];
-    qkv_elems(a, idx, el);
+    qkv_elems(a, idx, wave == 0, el);
     const uint16_t qa16 = el[0], qb16 = el[1], ka16 = el[2], kb16 = el[3], va16 = el[4], vb16 = el[5];
     asm volatile("" ::: "memory");
     const int pos = (int)pos64;
