@@ -58,6 +58,29 @@ def test_size_queries_and_argument_errors():
     assert L.elutq_hlq_repack_host(None, None, None, 128, 64, 2, 128, None, None, None) == -1
     with pytest.raises(_lib.ElutqError, match="group must be 64 or 128"):
         _lib.check(-4, "t")
+    # K slices of a batch-1 launch: none where the column blocks fill the chip, up to four where they do not,
+    # the caller's count when given, 0 for what no launch accepts
+    assert L.elutq_hlq_gemv_slices(4096, 14336, 2, 128, 0, 0) == 1
+    assert L.elutq_hlq_gemv_slices(4096, 4096, 2, 128, 0, 0) == 1
+    assert L.elutq_hlq_gemv_slices(14336, 4096, 2, 128, 0, 0) == 4
+    assert L.elutq_hlq_gemv_slices(4096, 1024, 2, 128, 0, 0) == 4
+    assert L.elutq_hlq_gemv_slices(4096, 6144, 2, 128, 2, 16) == 2
+    assert L.elutq_hlq_gemv_slices(256, 64, 2, 128, 0, 0) == 2          # never more slices than units
+    assert L.elutq_hlq_gemv_slices(4096, 4096, 2, 128, 33, 0) == 0
+    assert L.elutq_hlq_gemv_slices(4000, 4096, 2, 128, 0, 0) == 0
+    # entry points that take handed-over slices check their arguments before any launch
+    assert L.elutq_decode_rope_attn_sliced_f16(None, 2, 2048, one, one, one, one, 4, 2, 128, 64, 10000.0, 1, None, 0, None) == -1
+    assert L.elutq_decode_rope_attn_sliced_f16(one, 5, 2048, one, one, one, one, 4, 2, 128, 64, 10000.0, 1, None, 0, None) == -7
+    assert L.elutq_decode_rope_attn_sliced_f16(one, 2, 100, one, one, one, one, 4, 2, 128, 64, 10000.0, 1, None, 0, None) == -7
+    assert L.elutq_decode_rope_attn_sliced_f16(one, 2, 2048, one, one, one, one, 4, 2, 64, 64, 10000.0, 1, None, 0, None) == -7
+    f = _lib.GemvFusion(0, 0.0, None, None, None, ctypes.c_void_p(1), 2, None)
+    fused = lambda fus, ks=0: L.elutq_hlq_gemv_fused_f16(one, one, one, None, one, one, 4096, 64, 2, 128, one, 1 << 20, None,
+                                                         ctypes.byref(fus), ks, 0)
+    assert fused(f) == -7                                               # slices come with the RMSNorm prologue only
+    assert fused(_lib.GemvFusion(1, 1e-5, one, None, None, one, 5, None)) == -7      # at most four
+    assert fused(_lib.GemvFusion(1, 1e-5, one, None, None, one, 2, one)) == -7       # x_out may not be x itself
+    assert fused(_lib.GemvFusion(0, 0.0, None, one, one, None, 0, None), 4) == -7    # the consumer adds the residual
+    assert fused(_lib.GemvFusion(0, 0.0, None, None, one, None, 0, None), 1) == -7   # one slice: nothing to hand over
 
 
 @pytest.mark.parametrize("k,n,bits,group", [(256, 64, 2, 128), (384, 70, 3, 128), (128, 1, 1, 64),
