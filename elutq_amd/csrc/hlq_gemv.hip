@@ -1049,6 +1049,9 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         a.n_slices_in = fusion->n_slices_in;
         a.slices_in = (const HLQ_GLOBAL float *)fusion->d_slices_in;
         if (fusion->d_x_out == d_x) return ELUTQ_ERR_TUNING;       // other workgroups still read the base
+        // only launches of one tile per workgroup take slices: the instances that walk a run of column
+        // blocks (more tiles than compute units) have not been validated as consumers
+        if ((long long)g.ncb * ksplit > NUM_CU) return ELUTQ_ERR_TUNING;
         a.x_out = (HLQ_GLOBAL uint16_t *)fusion->d_x_out;
         stage_bytes = (size_t)K * sizeof(uint16_t);
         if (gemv_lds_bytes(ups, bits, waves) + stage_bytes > (size_t)MAX_LDS) return ELUTQ_ERR_SHAPE;

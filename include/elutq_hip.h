@@ -131,6 +131,8 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
  *             d_x = the residual: x <- fp16(((s0 + s1) + ...) + d_x) element by element, i.e. what
  *             the producer would have written with d_residual = d_x, bit for bit; the RMSNorm
  *             follows.  d_x_out (fp16 [K], or NULL; not d_x) receives that x for later readers.
+ *             The consuming launch must have at most one tile per compute unit
+ *             (ceil(N/64) * slices <= 256); wider projections return ELUTQ_ERR_TUNING.
  * No counterpart in the reference, whose operators run one after the other on whole vectors.
  */
 typedef struct elutq_gemv_fusion {

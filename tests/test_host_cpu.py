@@ -79,6 +79,9 @@ def test_size_queries_and_argument_errors():
     assert fused(f) == -7                                               # slices come with the RMSNorm prologue only
     assert fused(_lib.GemvFusion(1, 1e-5, one, None, None, one, 5, None)) == -7      # at most four
     assert fused(_lib.GemvFusion(1, 1e-5, one, None, None, one, 2, one)) == -7       # x_out may not be x itself
+    wide = L.elutq_hlq_gemv_fused_f16(one, one, one, None, one, one, 4096, 28672, 2, 128, one, 1 << 20, None,
+                                      ctypes.byref(_lib.GemvFusion(1, 1e-5, one, None, None, one, 2, None)), 0, 0)
+    assert wide == -7                                                   # a consumer has one tile per compute unit at most
     assert fused(_lib.GemvFusion(0, 0.0, None, one, one, None, 0, None), 4) == -7    # the consumer adds the residual
     assert fused(_lib.GemvFusion(0, 0.0, None, None, one, None, 0, None), 1) == -7   # one slice: nothing to hand over
 
