@@ -447,7 +447,8 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
             "model": f"LLaMA-3-8B-shaped random init, {s.n_layers} layers, HLQ w{s.bits}g{s.group}, "
                      + (f"HLQ w{s.bits}g{s.group} lm_head" if hlq_lm_head else "fp16 lm_head"),
             "glue": ("5 launches per layer (rmsnorm+qkv | rope+cache+attention | o+residual | rmsnorm+gate|up | "
-                     "silu*up+down+residual), " if impl == "hip" else "PyTorch-ROCm ops around the HLQ GEMVs, ")
+                     "silu*up+down+residual; the K slices of q|k|v and of down are summed by the launch that reads "
+                     "them), " if impl == "hip" else "PyTorch-ROCm ops around the HLQ GEMVs, ")
                     + ("own final norm and argmax kernels, torch embedding gather, "
                        + ("HLQ GEMV lm_head, " if hlq_lm_head else "hipBLASLt fp16 lm_head, ")
                        if impl == "hip" else "torch embedding / final norm / hipBLASLt fp16 lm_head / argmax, ")
