@@ -13,16 +13,18 @@ from elutq_amd.synth import make_layer
 pytestmark = pytest.mark.gpu
 
 
-def build(k, n, seed, dev):
-    L = make_layer(k, n, bits=2, group=128, seed=seed, bias=False)
-    return HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, 128, None, dev)
+def build(k, n, seed, dev, bits=2, group=128):
+    L = make_layer(k, n, bits=bits, group=group, seed=seed, bias=False)
+    return HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, group, None, dev)
 
 
-@pytest.mark.parametrize("ffn,hidden,n_next", [(1024, 512, 768), (14336, 4096, 6144)])
-def test_consumer_sees_what_the_producer_would_have_written(cuda, ffn, hidden, n_next):
+@pytest.mark.parametrize("ffn,hidden,n_next,bits,group", [(1024, 512, 768, 2, 128), (14336, 4096, 6144, 2, 128),
+                                                          (1024, 512, 768, 3, 64), (1024, 512, 768, 4, 128),
+                                                          (2048, 1024, 1536, 2, 64)])
+def test_consumer_sees_what_the_producer_would_have_written(cuda, ffn, hidden, n_next, bits, group):
     """down (SiLU*up prologue, K slices) -> next q|k|v (RMSNorm prologue), at the shapes of the small test
-    model and of LLaMA-3-8B."""
-    down, qkv = build(ffn, hidden, 1, cuda), build(hidden, n_next, 2, cuda)
+    model and of LLaMA-3-8B, and at the other plane counts / group size."""
+    down, qkv = build(ffn, hidden, 1, cuda, bits, group), build(hidden, n_next, 2, cuda, bits, group)
     S = down.slices
     assert 2 <= S <= 4
     g = torch.Generator(device=cuda).manual_seed(3)
