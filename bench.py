@@ -482,6 +482,14 @@ def main():
             # the workload of the headline decode figure keeps the fp16 lm_head)
             torch.cuda.empty_cache()
             out["decode_hlq_lm_head"] = bench_decode(dev, hlq_lm_head=True)
+            # the same step (fp16 lm_head) at the other formats of the GEMV sweep
+            from elutq_amd.llama_decode import LlamaShape
+            out["decode_other_formats"] = {}
+            for bits, group in ((3, 128), (2, 64)):
+                torch.cuda.empty_cache()
+                r = bench_decode(dev, shape=LlamaShape(bits=bits, group=group))
+                out["decode_other_formats"][f"w{bits}g{group}"] = {k: r[k] for k in ("tokens_per_s", "ms_per_token",
+                                                                                     "bytes_per_token", "GBps")}
         except ImportError:
             out["decode"] = None
 
