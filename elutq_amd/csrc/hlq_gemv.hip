@@ -525,7 +525,8 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     if (prologue == 1)
         rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst, sfirst, sliced, stage,
                           sliced && a.x_out && blockIdx.x == 0 && blockIdx.y == 0);
-    if (sliced) raw = stage[(k0 >> 2) + (nchunks ? min(lane, nchunks - 1) : 0)];   // the combined chunk replaces the base's
+    // the combined chunk replaces the base's (a wave without a run sits at the end of the slice: clamped)
+    if (sliced) raw = stage[min((int)(k0 >> 2) + (nchunks ? min(lane, nchunks - 1) : 0), K / 4 - 1)];
 
     // ... the tables are built as soon as the activations are in (a wave that first queued all
     // its weight loads would sit in the memory pipeline's back-pressure instead) ...
