@@ -62,7 +62,7 @@ def test_gemm_exact_on_integer_inputs(cuda):
     assert np.array_equal(y.astype(np.float64), O.gemm_f64(x, wq, ws, wz, group))
 
 
-@pytest.mark.parametrize("m", [16, 64])
+@pytest.mark.parametrize("m", [16, 32, 64])
 @pytest.mark.parametrize("k,n", LLAMA2_13B_PREFILL_SHAPES)
 def test_llama2_13b_prefill_shapes(cuda, m, k, n):
     L = make_layer(k, n, bits=2, group=128, m=m, seed=11)

@@ -213,6 +213,31 @@ def test_fp16_chain_close_to_f64_and_gemm_is_row_loop(lutref):
     assert np.max(np.abs(ym.astype(np.float64) - y64)) / np.sqrt(np.mean(y64 ** 2)) < 2e-2
     fast = np.stack([rw.gemv_fast(r) for r in L.x])
     assert O.rel_err(fast, y64) < 5e-2
+    # the NumPy row loop is the C one bit for bit (two implementations, 1 and 4 threads, both mac forms)
+    for fused in (True, False):
+        yr = O.gemm_rows(L.x, L.w_quant, L.w_scale, L.w_zero, 128, fused=fused)
+        assert yr.shape == (3, 128) and yr.dtype == np.float16
+        for threads in (1, 4):
+            yc = lutref.RefWeight(L.w_quant, L.w_scale, L.w_zero, 128, threads).gemm(L.x, fused)
+            assert np.array_equal(yr.view(np.uint16), yc.view(np.uint16))
+
+
+def test_gemm_rows_exact_on_integer_inputs():
+    """Rows of small integers against power-of-two scales: every fp16 operation of the row loop is
+    exact, so it equals the float64 dequantize-then-matmul bit for bit, row by row, bias included."""
+    r = rng(21)
+    m, k, n, bits, g = 5, 256, 96, 3, 64
+    x = r.integers(-2, 3, (m, k)).astype(np.float16)
+    wq = O.pack_planes(r.integers(0, 2, (bits, n, k), dtype=np.uint8))
+    ws = np.stack([np.full((n, k // g), 2.0 ** (b - 3), np.float16) for b in range(bits)])
+    wz = (r.integers(-3, 1, (n, k // g)) / 4).astype(np.float16)
+    bias = r.integers(-4, 5, n).astype(np.float16)
+    y64 = O.gemm_f64(x, wq, ws, wz, g, bias)
+    assert np.all(np.abs(y64) < 1024)
+    assert np.array_equal(O.gemm_rows(x, wq, ws, wz, g, bias).astype(np.float64), y64)
+    # a permutation of the rows permutes the result: rows do not see each other
+    perm = r.permutation(m)
+    assert np.array_equal(O.gemm_rows(x[perm], wq, ws, wz, g, bias), O.gemm_rows(x, wq, ws, wz, g, bias)[perm])
 
 
 def test_rel_err_metric():

@@ -1,5 +1,7 @@
 """Quantize on the device, export, load, run: the whole chain from an fp16 weight to the HIP
 kernels without the reference (HLQ.fasterquant -> export files -> load_Parameter -> arm_gemm)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -9,6 +11,43 @@ from elutq_amd import hlq_quantize as HQ
 from elutq_amd.hlq_linear import HLQLinear
 
 pytestmark = pytest.mark.gpu
+
+GOLD = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "hlq_quantizer_vectors.npz"))
+
+
+@pytest.mark.parametrize("name,bits", [("b2_g128", 2), ("b3_g128", 3), ("b2_g64", 2), ("b4_g128", 4), ("b1_g64", 1)])
+def test_fit_and_assignment_on_the_device_match_reference_vectors(cuda, name, bits):
+    """The alternating fit and the nearest-level assignment run on device tensors against the vectors the
+    reference's own GPTQ/quant.py wrote (tests/golden/make_quantizer_goldens.py): same bars as on the CPU."""
+    w = torch.from_numpy(GOLD[f"{name}_w"]).to(cuda)
+    scales, zeros = HQ.fit_alternating(w, bits)
+    assert scales.is_cuda and zeros.is_cuda
+    np.testing.assert_allclose(scales.cpu().numpy(), GOLD[f"{name}_scales"], rtol=2e-4, atol=1e-7)
+    np.testing.assert_allclose(zeros.cpu().numpy(), GOLD[f"{name}_zeros"], rtol=2e-4, atol=1e-6)
+    gs, gz = torch.from_numpy(GOLD[f"{name}_scales"]).to(cuda), torch.from_numpy(GOLD[f"{name}_zeros"]).to(cuda)
+    codes = HQ.assign_codes(w, gs, gz, bits)
+    assert codes.is_cuda and codes.dtype == torch.uint8
+    # the device forms the levels with a library matrix product whose summation order is its own: an
+    # element that sits within an ulp of the midpoint of two levels may land on the other one
+    same = codes.cpu().numpy() == GOLD[f"{name}_codes"]
+    assert (~same).mean() <= 1e-3
+    deq = HQ.dequantize_codes(codes, gs, gz).cpu().numpy()
+    keep = same.all(axis=-1)
+    np.testing.assert_allclose(deq[keep], GOLD[f"{name}_deq"][keep], rtol=1e-6, atol=1e-8)
+    own = HQ.assign_codes(w, scales, zeros, bits)
+    assert (own.cpu().numpy() != GOLD[f"{name}_codes"]).mean() < 0.01
+    mse = float(((HQ.dequantize_codes(own, scales, zeros) - w) ** 2).mean())
+    assert mse == pytest.approx(float(((GOLD[f"{name}_deq"] - GOLD[f"{name}_w"]) ** 2).mean()), rel=1e-3)
+
+
+def test_quantize_groups_on_the_device_matches_reference_slab(cuda):
+    w = torch.from_numpy(GOLD["slab_w"]).to(cuda)
+    wq, codes, scales, zeros = HQ.quantize_groups(w, 2, 128)
+    assert wq.is_cuda and codes.shape == GOLD["slab_codes"].shape
+    np.testing.assert_allclose(scales.cpu().numpy(), GOLD["slab_scales"], rtol=2e-4, atol=1e-7)
+    np.testing.assert_allclose(zeros.cpu().numpy(), GOLD["slab_zeros"], rtol=2e-4, atol=1e-6)
+    assert (codes.cpu().numpy() != GOLD["slab_codes"]).mean() < 0.01
+    np.testing.assert_allclose(wq.cpu().numpy(), GOLD["slab_deq"], atol=2e-3 * np.abs(GOLD["slab_w"]).max())
 
 
 @pytest.mark.parametrize("bits,group", [(2, 128), (3, 128), (2, 64), (4, 128)])
