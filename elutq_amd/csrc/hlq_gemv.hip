@@ -1073,6 +1073,22 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves) + stage_bytes, (hipStream_t)stream);
 }
 
+// Whether a launch of this shape (ksplit / waves as the call would pass them) takes `n_slices` handed-over
+// K slices in its RMSNorm prologue: the same steps and limits as the launch itself.
+extern "C" int elutq_hlq_gemv_accepts_slices(int K, int N, int bits, int group, int ksplit, int waves, int n_slices)
+{
+    if (check_shape(K, N, bits, group) != ELUTQ_OK) return 0;
+    if (n_slices < 1 || n_slices > GEMV_MAX_SLICES_IN) return 0;
+    const HlqGeo g = hlq_geo(K, N, bits, group);
+    if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return 0;
+    choose_shape(g, ksplit, waves);
+    int ups = (g.U + ksplit - 1) / ksplit;
+    while (gemv_lds_bytes(ups, bits, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
+    ksplit = (g.U + ups - 1) / ups;
+    if ((long long)g.ncb * ksplit > NUM_CU) return 0;
+    return gemv_lds_bytes(ups, bits, waves) + (size_t)K * sizeof(uint16_t) <= (size_t)MAX_LDS ? 1 : 0;
+}
+
 extern "C" int elutq_hlq_gemv_slices(int K, int N, int bits, int group, int ksplit, int waves)
 {
     if (check_shape(K, N, bits, group) != ELUTQ_OK) return 0;

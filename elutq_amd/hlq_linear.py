@@ -307,6 +307,12 @@ class HLQLinear(nn.Module):
         return _lib.lib().elutq_hlq_gemv_slices(self.in_features, self.out_features, self.bits, self.group_size,
                                                 self.ksplit, self.waves)
 
+    def accepts_slices(self, n_slices: int) -> bool:
+        """Whether this layer's batch-1 launch takes `n_slices` handed-over K slices in its RMSNorm prologue
+        (gemv_fused(..., slices_in=...)); a producer may leave its slices unsummed only then."""
+        return bool(_lib.lib().elutq_hlq_gemv_accepts_slices(self.in_features, self.out_features, self.bits,
+                                                             self.group_size, self.ksplit, self.waves, n_slices))
+
     def dequantize(self) -> torch.Tensor:
         """Dense fp16 W [N, K] (``dequantize_with_scales``, GPTQ/quant.py:176-183)."""
         w = torch.empty((self.out_features, self.in_features), dtype=torch.float16, device=self.planes.device)

@@ -151,14 +151,17 @@ MAX_DEFERRED_SLICES = 4        # what a consuming launch accepts (elutq_gemv_fus
 
 
 def deferred_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tensor, cur: torch.Tensor,
-                        other: torch.Tensor, pending: int, last: bool, defer_qkv: bool = True):
+                        other: torch.Tensor, pending: int, last: bool, defer_qkv: bool = True,
+                        defer_down: bool = True):
     """The same five launches with the K slices of the down projection left unsummed for the launch
     that reads them (the next layer's q|k|v), which forms fp16(slices + residual) itself, bit for
     bit what the producer's own output stage writes, and stores it for the later residual add.
     `cur` holds the residual stream, `other` is free; `pending` = slices of the previous layer's
     down waiting in b.sd (0 = none).  Returns (cur, other, pending).  `defer_qkv`: the q|k|v
     projection's K slices go to the attention launch the same way (head_dim 128), where a
-    workgroup only sums the 3 x 128 elements of its own head."""
+    workgroup only sums the 3 x 128 elements of its own head.  `defer_down` = False: the launch that
+    would read down's slices cannot take them (LlamaDecoder decides that per layer when it is built), so
+    down sums them itself."""
     s = layer.s
     n_q = layer.qkv.slices
     defer_qkv = defer_qkv and s.head_dim == 128 and 2 <= n_q <= MAX_DEFERRED_SLICES and layer.qkv.bias is None
@@ -183,7 +186,7 @@ def deferred_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tenso
     layer.gate_up.gemv_fused(other, b.gu, b.ws, prologue=1, norm_weight=layer.ln2, eps=s.rms_eps)
     cur, other = other, cur
     n_d = layer.down_proj.slices
-    if not last and 2 <= n_d <= MAX_DEFERRED_SLICES and layer.down_proj.bias is None:
+    if not last and defer_down and 2 <= n_d <= MAX_DEFERRED_SLICES and layer.down_proj.bias is None:
         layer.down_proj.gemv_fused(b.gu, other, b.ws, prologue=2, slices_out=b.sd)
         return cur, other, n_d
     layer.down_proj.gemv_fused(b.gu, other, b.ws, prologue=2, residual=cur)
@@ -334,6 +337,12 @@ class LlamaDecoder(nn.Module):
                 q = layer.qkv
                 if d == 128 and q.bias is None and q.slices == 1 and 2 * ((q.out_features + 63) // 64) <= 256:
                     q.ksplit, q.waves = 2, 16
+            # down leaves its K slices unsummed only where the next layer's q|k|v launch takes them (a q|k|v
+            # with more tiles than compute units, or tables that leave no room for the staged activations,
+            # does not): decided here, once, so that a step never meets a refusing launch
+            self._defer_down = [i + 1 < len(self.layers) and 2 <= layer.down_proj.slices <= MAX_DEFERRED_SLICES
+                                and self.layers[i + 1].qkv.accepts_slices(layer.down_proj.slices)
+                                for i, layer in enumerate(self.layers)]
 
     @classmethod
     def from_export(cls, root: str, s: LlamaShape, device="cuda", fuse: bool = True, impl: str = "hip",
@@ -364,7 +373,8 @@ class LlamaDecoder(nn.Module):
                 x, free, pending = b.xa, b.xb, 0
                 for i, layer in enumerate(self.layers):
                     x, free, pending = deferred_layer_step(layer, b, self.pos, x, free, pending,
-                                                           last=i == len(self.layers) - 1, defer_qkv=self.defer_qkv)
+                                                           last=i == len(self.layers) - 1, defer_qkv=self.defer_qkv,
+                                                           defer_down=self._defer_down[i])
             else:
                 for layer in self.layers:
                     fused_layer_step(layer, b, self.pos)

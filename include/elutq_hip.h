@@ -150,6 +150,13 @@ typedef struct elutq_gemv_fusion {
  * elutq_hlq_gemv_f16_tuned, 0 = default); 0 for an unsupported shape or tuning. */
 int elutq_hlq_gemv_slices(int K, int N, int bits, int group, int ksplit, int waves);
 
+/* 1 if a launch of this shape (ksplit / waves as the call would pass them) accepts `n_slices`
+ * handed-over K slices (elutq_gemv_fusion.n_slices_in) in its RMSNorm prologue, else 0: the limits the
+ * launch itself applies (1..4 slices, at most one tile per compute unit, tables plus the fp16 [K]
+ * staging area within the LDS).  A caller decides with it, before it lets a producer leave its slices
+ * unsummed, whether the consumer can take them. */
+int elutq_hlq_gemv_accepts_slices(int K, int N, int bits, int group, int ksplit, int waves, int n_slices);
+
 int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const void *d_zeros,
                              const void *d_bias, const void *d_x, void *d_y,
                              int K, int N, int bits, int group,

@@ -206,3 +206,25 @@ def test_two_streams_with_their_own_workspaces(cuda):
             outs_b.append(mb(xb))
     torch.cuda.synchronize()
     assert all(torch.equal(o, ya0) for o in outs_a) and all(torch.equal(o, yb0) for o in outs_b)
+
+
+@pytest.mark.parametrize("bad", [float("nan"), float("inf"), float("-inf")])
+@pytest.mark.parametrize("ksplit,waves", [(0, 0), (2, 8)])
+def test_non_finite_activations_reach_the_output(cuda, bad, ksplit, waves):
+    """The reference's fp16 table entries and sums carry a NaN or an infinity in x into every output it
+    touches (arm_t_mac_kernal.cpp:111-126, arm_gemm.cpp:250-279).  The integer tables here cannot hold
+    one, but the fp32 sum of each 64-k half is non-finite exactly when one of its activations is, and the
+    zero-point fold multiplies it into every column: a numerical blow-up upstream stays visible.  Columns
+    whose activations are all finite elsewhere keep their finite value only if the bad element is absent."""
+    L = make_layer(1024, 192, bits=2, group=128, seed=41)
+    m = to_mod(L, cuda, ksplit, waves)
+    x = L.x.copy()
+    y_ok = run(m, x, cuda)[0]
+    assert np.all(np.isfinite(y_ok))
+    x[0, 517] = bad
+    y = run(m, x, cuda)[0]
+    w = O.dequantize(L.w_quant, L.w_scale, L.w_zero, 128, np.float64)
+    with np.errstate(invalid="ignore", over="ignore"):
+        ref = w @ x[0].astype(np.float64)
+    assert not np.any(np.isfinite(ref))              # every weight of the synthetic layer is non-zero
+    assert not np.any(np.isfinite(y.astype(np.float32)))

@@ -84,6 +84,30 @@ def test_size_queries_and_argument_errors():
     assert wide == -7                                                   # a consumer has one tile per compute unit at most
     assert fused(_lib.GemvFusion(0, 0.0, None, one, one, None, 0, None), 4) == -7    # the consumer adds the residual
     assert fused(_lib.GemvFusion(0, 0.0, None, None, one, None, 0, None), 1) == -7   # one slice: nothing to hand over
+    # the query a caller decides with before it lets a producer leave its slices unsummed: the launch's own limits
+    acc = L.elutq_hlq_gemv_accepts_slices
+    assert acc(4096, 6144, 2, 128, 2, 16, 4) == 1                       # LLaMA-3-8B q|k|v in two K slices: 192 tiles
+    assert acc(4096, 6144, 2, 128, 0, 0, 4) == 1
+    assert acc(4096, 28672, 2, 128, 0, 0, 2) == 0                       # more tiles than compute units (what `wide` is refused for)
+    assert acc(8192, 10240, 2, 128, 2, 16, 4) == 0                      # a q|k|v of 160 column blocks in two slices: 320 tiles
+    assert acc(8192, 10240, 2, 128, 1, 16, 4) == 1
+    assert acc(4096, 6144, 2, 128, 2, 16, 5) == 0 and acc(4096, 6144, 2, 128, 2, 16, 0) == 0
+    assert acc(4000, 6144, 2, 128, 0, 0, 2) == 0
+
+
+def test_decoder_defers_down_only_where_the_next_qkv_takes_the_slices():
+    """A decode step must never meet a launch that refuses handed-over slices: the decision is the library's
+    query, taken per layer when the decoder is built (here replayed on shapes, no GPU needed)."""
+    L = _lib.lib()
+    # LLaMA-3-8B: down 14336 -> 4096 in four slices, q|k|v 4096 -> 6144 in two slices: taken
+    n_d = L.elutq_hlq_gemv_slices(14336, 4096, 2, 128, 0, 0)
+    assert n_d == 4 and L.elutq_hlq_gemv_accepts_slices(4096, 6144, 2, 128, 2, 16, n_d) == 1
+    # a model with hidden 8192 and 64 + 2 x 8 heads of 128: q|k|v has 160 column blocks; in two K slices that is
+    # 320 tiles for 256 compute units -> the launch walks runs of column blocks and takes no slices, so
+    # down (16384 -> 8192, sliced) must sum for itself
+    n_d = L.elutq_hlq_gemv_slices(16384, 8192, 2, 128, 0, 0)
+    assert 2 <= n_d <= 4
+    assert L.elutq_hlq_gemv_accepts_slices(8192, 10240, 2, 128, 2, 16, n_d) == 0
 
 
 @pytest.mark.parametrize("k,n,bits,group", [(256, 64, 2, 128), (384, 70, 3, 128), (128, 1, 1, 64),
