@@ -28,6 +28,9 @@ SIGNATURES = {
     "elutq_hlq_gemv_f16_tuned": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _ci, _ci]),
     "elutq_hlq_gemv_fused_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
     "elutq_hlq_gemv_slices": (_ci, [_ci] * 6),
+    "elutq_hlq_static_scratch_bytes": (_sz, []),
+    "elutq_hlq_static_init": (_ci, []),
+    "elutq_hlq_gemv_f16_static": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp]),
     "elutq_hlq_gemv_accepts_slices": (_ci, [_ci] * 7),
     "elutq_decode_rope_attn_f16": (_ci, [_vp] * 5 + [_ci] * 4 + [ctypes.c_float, _vp]),
     "elutq_decode_rope_attn_split_f16": (_ci, [_vp] * 5 + [_ci] * 4 + [ctypes.c_float, _ci, _vp, _sz, _vp]),

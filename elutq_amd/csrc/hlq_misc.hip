@@ -64,6 +64,9 @@ const char *elutq_status_string(int status)
     case ELUTQ_ERR_SPARSE:
         return "malformed sparse block list: need (channel start, k start) pairs, channel start a multiple of 32 below N "
                "and ascending, k start a multiple of 4 with k + group <= K";
+    case ELUTQ_ERR_STATIC_LIMIT:
+        return "the shape needs more partial-sum scratch than the static buffer holds (ELUTQ_STATIC_PARTIAL_BYTES): "
+               "use elutq_hlq_gemv_f16 with a workspace";
     }
     return "unknown status";
 }

@@ -51,7 +51,8 @@ typedef enum elutq_status {
     ELUTQ_ERR_WORKSPACE = -5,  /* workspace smaller than elutq_hlq_workspace_bytes() */
     ELUTQ_ERR_HIP = -6,        /* a HIP runtime call failed (launch, attribute) */
     ELUTQ_ERR_TUNING = -7,     /* explicit ksplit / waves arguments out of range */
-    ELUTQ_ERR_SPARSE = -8      /* malformed block list of a sparse extra plane */
+    ELUTQ_ERR_SPARSE = -8,     /* malformed block list of a sparse extra plane */
+    ELUTQ_ERR_STATIC_LIMIT = -9 /* the shape needs more scratch than the static buffer of the _static entry point holds */
 } elutq_status;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -96,6 +97,28 @@ int elutq_hlq_gemv_f16(const void *d_planes, const void *d_scales, const void *d
                        const void *d_bias, const void *d_x, void *d_y,
                        int K, int N, int bits, int group,
                        void *d_workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * elutq_hlq_gemv_f16 for callers that cannot allocate and bring no workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference
+ * (whose arm_gemm takes a caller-owned temp_workplace, as elutq_hlq_gemv_f16 takes a workspace).
+ * Same inputs, outputs and results, bit for bit, as elutq_hlq_gemv_f16; the arrival counters and
+ * partial sums of a K-sliced launch live in a device array inside the library instead
+ * (elutq_hlq_static_scratch_bytes() = 64 KiB + ELUTQ_STATIC_PARTIAL_BYTES per GPU, held until the process
+ * ends).  The call allocates nothing and frees nothing.  Shapes whose launch would need more partial-sum
+ * space -- slices * ceil(N/64)*64 * 4 bytes with slices = elutq_hlq_gemv_slices(K, N, bits, group, 0, 0) --
+ * return ELUTQ_ERR_STATIC_LIMIT (every LLaMA-3-8B / LLaMA-2-13B projection fits many times over).
+ * All calls on one GPU share that GPU's array: calls that may overlap on one GPU (two streams, two
+ * threads) race on it and must be ordered by the caller.  elutq_hlq_static_init() looks the array's
+ * device address up for the current device; the first call on a device does it otherwise (call it
+ * once per device before capturing a graph).
+ */
+#define ELUTQ_STATIC_PARTIAL_BYTES (2u << 20)
+size_t elutq_hlq_static_scratch_bytes(void);
+int elutq_hlq_static_init(void);
+int elutq_hlq_gemv_f16_static(const void *d_planes, const void *d_scales, const void *d_zeros,
+                              const void *d_bias, const void *d_x, void *d_y,
+                              int K, int N, int bits, int group, void *stream);
 
 /*
  * Same computation with the launch shape chosen by the caller: `ksplit` slices of K
