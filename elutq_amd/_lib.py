@@ -36,6 +36,7 @@ SIGNATURES = {
     "elutq_decode_rope_attn_split_f16": (_ci, [_vp] * 5 + [_ci] * 4 + [ctypes.c_float, _ci, _vp, _sz, _vp]),
     "elutq_decode_attn_workspace_bytes": (_sz, [_ci] * 3),
     "elutq_decode_rope_attn_sliced_f16": (_ci, [_vp, _ci, _ci, _vp, _vp, _vp, _vp] + [_ci] * 4 + [ctypes.c_float, _ci, _vp, _sz, _vp]),
+    "elutq_decode_embed_f16": (_ci, [_vp] * 3 + [_ci, _ci, _vp]),
     "elutq_decode_rmsnorm_f16": (_ci, [_vp] * 3 + [_ci, ctypes.c_float, _vp]),
     "elutq_decode_argmax_f16": (_ci, [_vp, _ci, _vp, _vp, _vp]),
     "elutq_decode_argmax_ws_f16": (_ci, [_vp, _ci, _vp, _vp, _vp, _sz, _vp]),

@@ -458,6 +458,23 @@ __global__ __launch_bounds__(TAIL_THREADS) void rmsnorm_kernel(const uint16_t *x
     for (int i = tid; i < n; i += TAIL_THREADS) out[i] = f2h(h2f(x[i]) * rstd * h2f(w[i]));
 }
 
+// Embedding gather of the current token (arm_embedding, C++/ops/src/arm/arm_embedding.cpp:4-20: a row copy).
+// The token is a device scalar; one outside [0, vocab) yields a zero row instead of a read outside the table.
+__global__ __launch_bounds__(256) void embed_kernel(const uint16_t *embed, const long long *token, uint16_t *out, int hidden,
+                                                    int vocab)
+{
+    const long long t = *token;
+    const bool ok = t >= 0 && t < (long long)vocab;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;             // 8 values per thread
+    if (i * 8 + 8 <= hidden) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (ok) v = *(const uint4 *)(embed + (size_t)t * hidden + (size_t)i * 8);
+        *(uint4 *)(out + (size_t)i * 8) = v;
+    } else {
+        for (int j = i * 8; j < hidden; j++) out[j] = ok ? embed[(size_t)t * hidden + j] : (uint16_t)0;
+    }
+}
+
 // (value, index) order of the greedy pick: larger value first, lower index among equals.
 __device__ __forceinline__ void pick(float &v, int &i, float v2, int i2)
 {
@@ -649,6 +666,15 @@ extern "C" int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, vo
 {
     return elutq_decode_rope_attn_split_f16(d_qkv, d_k_cache, d_v_cache, d_pos, d_out, n_heads, n_kv_heads, head_dim,
                                             max_seq, rope_base, 1, nullptr, 0, stream);
+}
+
+extern "C" int elutq_decode_embed_f16(const void *d_embed, const void *d_token, void *d_out, int hidden, int vocab, void *stream)
+{
+    if (!d_embed || !d_token || !d_out) return ELUTQ_ERR_NULL;
+    if (hidden < 1 || vocab < 1 || hidden % 8 != 0) return ELUTQ_ERR_SHAPE;      // rows stay 16-byte aligned
+    hipLaunchKernelGGL(embed_kernel, dim3((hidden / 8 + 255) / 256), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)d_embed,
+                       (const long long *)d_token, (uint16_t *)d_out, hidden, vocab);
+    return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
 
 extern "C" int elutq_decode_rmsnorm_f16(const void *d_x, const void *d_weight, void *d_out, int n, float eps, void *stream)

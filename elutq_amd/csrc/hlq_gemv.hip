@@ -32,12 +32,13 @@
 #include "../../include/elutq_hip.h"
 #include "hlq_layout.h"
 #include "hlq_internal.h"
+#include "hlq_gemv_index.h"
 
 namespace {
 
 constexpr int MAX_LDS = HLQ_MAX_LDS;
-constexpr int TBL_BYTES = 64;                    // 16 int32 entries
-constexpr int UNIT_LUT_BYTES = 32 * TBL_BYTES;   // 32 chunks per unit
+constexpr int TBL_BYTES = HLQ_TBL_BYTES;             // 16 int32 entries
+constexpr int UNIT_LUT_BYTES = HLQ_UNIT_LUT_BYTES;   // 32 chunks per unit
 
 // Device pointers are declared in the global address space for the device pass: a pointer that a
 // kernel reads out of a struct in memory (the grouped launch) would otherwise be generic, and
@@ -329,13 +330,12 @@ __device__ __forceinline__ void lds_barrier()
 
 // 1 / rms of the whole activation vector for the fused RMSNorm prologue: the workgroup sums
 // the squares together (one chunk per thread and pass), two barriers.  `scratch` is LDS of
-// RSTD_SCRATCH floats.  Every workgroup does this for itself (2K bytes from cache).
-constexpr int RSTD_SCRATCH = 80;
+// HLQ_RSTD_SCRATCH floats (at hlq_lds_map().rstd).  Every workgroup does this for itself (2K bytes from cache).
 
 // Activations that arrive as a base vector plus the unsummed K slices of the launch that
 // produced them (its `defer` mode): element k is fp16(((s0[k] + s1[k]) + ...) + x[k]), the same
 // operations in the same order as that launch's own output stage would have used.
-constexpr int GEMV_MAX_SLICES_IN = 4;
+constexpr int GEMV_MAX_SLICES_IN = HLQ_GEMV_MAX_SLICES_IN;
 
 struct SliceChunk {
     float4 p[GEMV_MAX_SLICES_IN];
@@ -345,7 +345,7 @@ __device__ __forceinline__ void load_slice_chunk(const GemvArgs &a, int K, int c
 {
 #pragma unroll
     for (int s = 0; s < GEMV_MAX_SLICES_IN; s++)     // always GEMV_MAX_SLICES_IN loads: a fixed count
-        c.p[s] = *(const HLQ_GLOBAL float4 *)(a.slices_in + (size_t)min(s, a.n_slices_in - 1) * K + (size_t)chunk * 4);
+        c.p[s] = *(const HLQ_GLOBAL float4 *)(a.slices_in + (size_t)hlq_slice_row(s, a.n_slices_in) * K + (size_t)chunk * 4);
 }
 
 __device__ __forceinline__ uint2 combine_chunk(const GemvArgs &a, uint2 base, const SliceChunk &c)
@@ -473,15 +473,17 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
     const int nst = nU * BITS;                                             // sub-tasks of this workgroup
-    const int s_begin = min(wave * a.spw, nst), s_end = min(s_begin + a.spw, nst);
-    const int ub = s_begin / BITS;                                         // first unit (in the slice) of this wave
-    const int nuw = s_end > s_begin ? (s_end - 1) / BITS - ub + 1 : 0;     // units this wave touches
-    const int s_last = max(s_end - 1, 0);                                  // clamp target for loads past the run
+    const HlqWaveRun wr = hlq_wave_run(wave, a.spw, nst, BITS);
+    const int s_begin = wr.s_begin, s_end = wr.s_end;
+    const int ub = wr.ub;                                                  // first unit (in the slice) of this wave
+    const int nuw = wr.nuw;                                                // units this wave touches
+    const int s_last = wr.s_last;                                          // clamp target for loads past the run
 
+    const HlqLdsMap lm = hlq_lds_map(nw, a.wave_lds);
     unsigned char *lut = smem + (size_t)wave * a.wave_lds;                 // this wave's tables [nuw][32][16] int32
     float2 *xs_inv = (float2 *)(lut + (size_t)a.nuw_max * UNIT_LUT_BYTES); // [2 * nuw_max]
-    float *red0 = (float *)(smem + (size_t)nw * a.wave_lds);               // [2][nw][64]
-    float *rstd_scratch = red0 + 2 * nw * HLQ_CB;                          // [RSTD_SCRATCH]
+    float *red0 = (float *)(smem + lm.red);                                // [2][nw][64]
+    float *rstd_scratch = (float *)(smem + lm.rstd);                       // [HLQ_RSTD_SCRATCH]
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
     __builtin_amdgcn_s_setprio(3);
@@ -508,11 +510,11 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     // fp16 [K] behind the reduction scratch when `sliced` (not selected against a null pointer: the
     // accesses must stay LDS instructions, a generic access would also count as a vector-memory one
     // and wait behind the weight loads in flight)
-    uint2 *stage = (uint2 *)(rstd_scratch + RSTD_SCRATCH + 4);
+    uint2 *stage = (uint2 *)(smem + lm.stage);
     if (sliced) load_slice_chunk(a, K, min(tid, K / 4 - 1), sfirst);
     uint2 raw, raw2;
     // lanes past the run (and waves without one, whose k0 is the end of the slice) re-read a valid chunk
-    load_chunk<PLAIN>(a, prologue, K, nchunks ? k0 + (size_t)min(lane, nchunks - 1) * 4 : 0, raw, raw2);
+    load_chunk<PLAIN>(a, prologue, K, hlq_x_first_k(k0, nchunks, lane), raw, raw2);
     asm volatile("" ::: "memory");      // keep both activation loads ahead of the weight loads
 
     float acc = 0.f;
@@ -526,7 +528,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst, sfirst, sliced, stage,
                           sliced && a.x_out && blockIdx.x == 0 && blockIdx.y == 0);
     // the combined chunk replaces the base's (a wave without a run sits at the end of the slice: clamped)
-    if (sliced) raw = stage[min((int)(k0 >> 2) + (nchunks ? min(lane, nchunks - 1) : 0), K / 4 - 1)];
+    if (sliced) raw = stage[hlq_stage_first_index(k0, nchunks, lane, K)];
 
     // ... the tables are built as soon as the activations are in (a wave that first queued all
     // its weight loads would sit in the memory pipeline's back-pressure instead) ...
@@ -725,29 +727,11 @@ __global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *__
     }
 }
 
-// Per-wave LDS region and run length for a slice of `ups` units handled by `waves` waves.
-struct WavePlan {
-    int spw, nuw_max, wave_lds;
-};
-
-WavePlan wave_plan(int ups, int bits, int waves)
-{
-    WavePlan p;
-    const int nst = ups * bits;
-    p.spw = (nst + waves - 1) / waves;
-    if (p.spw > bits && p.spw % bits) p.spw += bits - p.spw % bits;     // whole units per wave when it has several
-    if (p.spw == 1) p.nuw_max = 1;
-    else if (p.spw % bits == 0) p.nuw_max = p.spw / bits;
-    else p.nuw_max = (p.spw + bits - 2) / bits + 1;
-    p.wave_lds = (p.nuw_max * (UNIT_LUT_BYTES + 2 * (int)sizeof(float2)) + 255) & ~255;
-    return p;
-}
-
-size_t gemv_lds_bytes(int ups, int bits, int waves)
-{
-    const WavePlan p = wave_plan(ups, bits, waves);
-    return (size_t)waves * p.wave_lds + 2 * (size_t)waves * HLQ_CB * sizeof(float) + RSTD_SCRATCH * sizeof(float) + 16;
-}
+// Per-wave LDS region and run length for a slice of `ups` units handled by `waves` waves, and the dynamic
+// LDS of the workgroup: hlq_gemv_index.h (shared with the CPU audit of the tile's index arithmetic).
+using WavePlan = HlqWavePlan;
+WavePlan wave_plan(int ups, int bits, int waves) { return hlq_wave_plan(ups, bits, waves); }
+size_t gemv_lds_bytes(int ups, int bits, int waves) { return hlq_gemv_lds_bytes(ups, bits, waves); }
 
 constexpr int NUM_CU_RUN = HLQ_NUM_CU;
 

@@ -1,0 +1,103 @@
+// Index arithmetic of the batch-1 GEMV tile (hlq_gemv.hip: gemv_tile, block_rstd, load_slice_chunk), in
+// a form that compiles for the device and for the host: the kernel computes every run boundary, LDS
+// offset and staging index with these functions, and a CPU program can replay them for every workgroup
+// and wave of a launch and check each access against the sizes the launcher allocates
+// (tests/gemv_index_audit.cpp).
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define HLQ_HD __host__ __device__ __forceinline__
+#else
+#define HLQ_HD inline
+#endif
+
+#define HLQ_TBL_BYTES 64                          /* one chunk's table: 16 int32 entries */
+#define HLQ_UNIT_LUT_BYTES (32 * HLQ_TBL_BYTES)   /* 32 chunks per unit of 128 k */
+#define HLQ_RSTD_SCRATCH 80                       /* floats of reduction scratch of the RMSNorm prologue */
+#define HLQ_STAGE_GAP 4                           /* floats between that scratch and the staged activations */
+#define HLQ_GEMV_MAX_SLICES_IN 4
+
+// Per-wave LDS region and run length for a slice of `ups` units handled by `waves` waves.
+struct HlqWavePlan {
+    int spw;        // sub-tasks (unit, plane) per wave: a contiguous run
+    int nuw_max;    // units a wave's run can touch
+    int wave_lds;   // bytes of a wave's LDS region: tables [nuw_max][32][16] int32, then float2 [2 * nuw_max]
+};
+
+HLQ_HD HlqWavePlan hlq_wave_plan(int ups, int bits, int waves)
+{
+    HlqWavePlan p;
+    const int nst = ups * bits;
+    p.spw = (nst + waves - 1) / waves;
+    if (p.spw > bits && p.spw % bits) p.spw += bits - p.spw % bits;     // whole units per wave when it has several
+    if (p.spw == 1) p.nuw_max = 1;
+    else if (p.spw % bits == 0) p.nuw_max = p.spw / bits;
+    else p.nuw_max = (p.spw + bits - 2) / bits + 1;
+    p.wave_lds = (p.nuw_max * (HLQ_UNIT_LUT_BYTES + 2 * 8) + 255) & ~255;
+    return p;
+}
+
+// Dynamic LDS of a workgroup, in bytes from its start:
+//   [waves][wave_lds] tables and half-unit records | [2][waves][64] float cross-wave sums |
+//   [HLQ_RSTD_SCRATCH] float | gap | fp16 [K] staged activations (launches that take handed-over slices only)
+struct HlqLdsMap {
+    uint32_t red, rstd, stage, end_plain;
+};
+
+HLQ_HD HlqLdsMap hlq_lds_map(int waves, int wave_lds)
+{
+    HlqLdsMap m;
+    m.red = (uint32_t)waves * (uint32_t)wave_lds;
+    m.rstd = m.red + 2u * (uint32_t)waves * 64u * 4u;
+    m.stage = m.rstd + (HLQ_RSTD_SCRATCH + HLQ_STAGE_GAP) * 4u;
+    m.end_plain = m.stage;                        // == hlq_gemv_lds_bytes(): what a launch without staging allocates
+    return m;
+}
+
+HLQ_HD size_t hlq_gemv_lds_bytes(int ups, int bits, int waves)
+{
+    const HlqWavePlan p = hlq_wave_plan(ups, bits, waves);
+    return hlq_lds_map(waves, p.wave_lds).end_plain;
+}
+
+// The run of one wave inside a workgroup that owns `nst` sub-tasks (units of the slice x planes).
+struct HlqWaveRun {
+    int s_begin, s_end;   // sub-tasks [s_begin, s_end) of the slice
+    int ub;               // first unit (in the slice) the run touches
+    int nuw;              // units it touches (0: a wave without a run)
+    int s_last;           // clamp target of loads past the run
+};
+
+HLQ_HD HlqWaveRun hlq_wave_run(int wave, int spw, int nst, int bits)
+{
+    HlqWaveRun r;
+    const int b = wave * spw;
+    r.s_begin = b < nst ? b : nst;
+    const int e = r.s_begin + spw;
+    r.s_end = e < nst ? e : nst;
+    r.ub = r.s_begin / bits;
+    r.nuw = r.s_end > r.s_begin ? (r.s_end - 1) / bits - r.ub + 1 : 0;
+    r.s_last = r.s_end - 1 > 0 ? r.s_end - 1 : 0;
+    return r;
+}
+
+// Chunk (4 activations) of the whole K that lane `lane` of a wave builds its first table from, as an index
+// into the staged activations uint2 [K/4]: k0 = first k of the run, nchunks = 32 * nuw.  `clamp` = the
+// upper clamp a wave without a run needs (its k0 is the end of the slice, for the last slice the end of K).
+HLQ_HD int hlq_stage_first_index(size_t k0, int nchunks, int lane, int K, bool clamp = true)
+{
+    const int within = nchunks ? (lane < nchunks - 1 ? lane : nchunks - 1) : 0;
+    const int i = (int)(k0 >> 2) + within;
+    return clamp && i > K / 4 - 1 ? K / 4 - 1 : i;
+}
+
+// Element offset (in k) of the activation chunk the same lane loads from global memory first.
+HLQ_HD size_t hlq_x_first_k(size_t k0, int nchunks, int lane)
+{
+    return nchunks ? k0 + (size_t)(lane < nchunks - 1 ? lane : nchunks - 1) * 4 : 0;
+}
+
+// Row of the handed-over slices a fixed-count load reads for position s (rows past the count re-read the last).
+HLQ_HD int hlq_slice_row(int s, int n_slices_in) { return s < n_slices_in - 1 ? s : n_slices_in - 1; }

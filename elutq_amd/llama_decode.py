@@ -11,7 +11,7 @@ pairs (j, j + d/2) with theta = pos * base^(-2j/d) and no frequency rescaling
 (arm_attention.cpp:199-274), SiLU*up in fp32 (arm_activation.cpp:36-49).
 
 impl="hip": five fused launches per layer, final norm and greedy pick as kernels of the
-library, embedding gather and the fp16 lm_head (hipBLASLt) through PyTorch; impl="torch": the
+library, the fp16 lm_head (hipBLASLt) through PyTorch; impl="torch": the
 same model with PyTorch-ROCm ops around the HLQ projections (the parity partner).  The step
 is captured in a HIP graph (token id and position live in device tensors), so one replay =
 one token.  q|k|v and gate|up are fused along N, which in the kernel layout is a
@@ -368,7 +368,9 @@ class LlamaDecoder(nn.Module):
         and pos + 1 back.  Returns the logits [1, vocab] (fp16)."""
         if self.impl == "hip":
             b = self._buf
-            torch.index_select(self.embed, 0, self.token, out=b.xa)
+            _lib.check(_lib.lib().elutq_decode_embed_f16(self.embed.data_ptr(), self.token.data_ptr(), b.xa.data_ptr(),
+                                                         self.s.hidden, self.s.vocab,
+                                                         torch.cuda.current_stream().cuda_stream), "elutq_decode_embed_f16")
             if self.defer_slices:
                 x, free, pending = b.xa, b.xb, 0
                 for i, layer in enumerate(self.layers):
@@ -459,7 +461,7 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
             "glue": ("5 launches per layer (rmsnorm+qkv | rope+cache+attention | o+residual | rmsnorm+gate|up | "
                      "silu*up+down+residual; the K slices of q|k|v and of down are summed by the launch that reads "
                      "them), " if impl == "hip" else "PyTorch-ROCm ops around the HLQ GEMVs, ")
-                    + ("own final norm and argmax kernels, torch embedding gather, "
+                    + ("own embedding gather, final norm and argmax kernels, "
                        + ("HLQ GEMV lm_head, " if hlq_lm_head else "hipBLASLt fp16 lm_head, ")
                        if impl == "hip" else "torch embedding / final norm / hipBLASLt fp16 lm_head / argmax, ")
                     + "one HIP graph per token"}

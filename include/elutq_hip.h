@@ -286,6 +286,11 @@ int elutq_decode_rope_attn_sliced_f16(const void *d_qkv_slices, int n_slices, in
  * fp16 logits (arm_argmax_last, C++/ops/src/arm/arm_argmax.cpp:3-30; NaNs never win), and, if
  * d_pos is not NULL, *d_pos (DEVICE int64) += 1 -- so a captured graph advances its own state.
  */
+/* Head of a decode step: out[0:hidden] = embed[*d_token][0:hidden], fp16 (arm_embedding,
+ * C++/ops/src/arm/arm_embedding.cpp:4-20).  d_token is a DEVICE int64, so a captured graph follows the
+ * token the previous step picked; a token outside [0, vocab) gives a zero row (the reference would read
+ * outside the table).  hidden % 8 == 0, d_embed 16-byte aligned. */
+int elutq_decode_embed_f16(const void *d_embed, const void *d_token, void *d_out, int hidden, int vocab, void *stream);
 int elutq_decode_rmsnorm_f16(const void *d_x, const void *d_weight, void *d_out, int n, float eps, void *stream);
 int elutq_decode_argmax_f16(const void *d_logits, int n, void *d_token, void *d_pos, void *stream);
 /* The same pick by 64 workgroups that meet in `d_workspace` (64 KiB + 512 bytes, zero-filled once like

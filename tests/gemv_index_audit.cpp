@@ -1,0 +1,143 @@
+// CPU audit of the index arithmetic of the batch-1 GEMV tile (elutq_amd/csrc/hlq_gemv.hip: gemv_tile,
+// block_rstd, load_slice_chunk).  The kernel computes its run boundaries, LDS offsets and staging indices
+// with the functions of elutq_amd/csrc/hlq_gemv_index.h; this program replays them for every slice and
+// every wave -- waves without a run included -- of a superset of the launch shapes the library can choose,
+// and checks the highest byte each access can touch against what the launcher allocates (dynamic LDS =
+// hlq_gemv_lds_bytes + the fp16 [K] staging area of a slice-taking launch) and against the buffers the
+// C ABI documents.  Built and run by tests/test_gemv_index_audit.py (g++, no GPU).
+//
+//   gemv_index_audit [--unclamped-stage]     prints "violations <n>" and per-category counts
+//
+// --unclamped-stage replays the staged-chunk read without its upper clamp (the kernel as it was before the
+// clamp was added): the audit must then report violations, which shows that it looks at that access.
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <string>
+
+#include "hlq_gemv_index.h"
+
+namespace {
+
+constexpr int MAX_LDS = 160 * 1024;
+constexpr int CB = 64, UNIT = 128;
+
+int depth_of(int bits) { return bits == 3 ? 6 : (bits == 4 ? 8 : 4); }
+
+std::map<std::string, long> g_viol;
+long g_checked = 0;
+
+void check(bool ok, const char *what, int bits, int g64, int waves, int U, int ups, int slice, int wave, int nsl, int multi)
+{
+    g_checked++;
+    if (ok) return;
+    if (g_viol[what]++ < 3)
+        std::printf("VIOLATION %-14s bits=%d G=%d waves=%d U=%d ups=%d slice=%d wave=%d slices_in=%d run_kernel=%d\n", what, bits,
+                    g64 ? 64 : 128, waves, U, ups, slice, wave, nsl, multi);
+}
+
+// One launch shape: U units of K, ncb column blocks, slices of `ups` units, `waves` waves per workgroup,
+// n_slices_in handed-over slices (0 = none), MULTI = the instances that walk runs of column blocks.
+void audit(int bits, bool g64, int waves, int U, int ups, int ncb, int n_slices_in, bool multi, bool clamp_stage)
+{
+    const int K = U * UNIT;
+    const HlqWavePlan wp = hlq_wave_plan(ups, bits, waves);
+    const size_t lds_alloc = hlq_gemv_lds_bytes(ups, bits, waves) + (n_slices_in ? (size_t)K * 2 : 0);
+    if (lds_alloc > (size_t)MAX_LDS) return;                       // the launcher halves the slice or refuses
+    const int nslot = wp.spw < depth_of(bits) ? wp.spw : depth_of(bits);
+    if (multi && (wp.spw > nslot || waves != 16)) return;          // the condition of the run kernels
+    const int ksplit = (U + ups - 1) / ups;
+    const HlqLdsMap lm = hlq_lds_map(waves, wp.wave_lds);
+    const int NT = ((g64 ? 2 * U : U) + 1) / 2;
+    const size_t planes_bytes = (size_t)ncb * U * bits * CB * 16;
+    const size_t scale_bytes = (size_t)ncb * NT * bits * CB * 4, zero_bytes = (size_t)ncb * NT * CB * 4;
+    const size_t npad = (size_t)ncb * CB;
+#define CHECK(ok, what) check((ok), what, bits, g64, waves, U, ups, slice, wave, n_slices_in, multi)
+    for (int slice = 0; slice < ksplit; slice++) {
+        const int u0 = slice * ups, nU = (u0 + ups < U ? u0 + ups : U) - u0, nst = nU * bits;
+        for (int wave = 0; wave < waves; wave++) {
+            const HlqWaveRun r = hlq_wave_run(wave, wp.spw, nst, bits);
+            const uint32_t lut = (uint32_t)wave * wp.wave_lds, xs = lut + (uint32_t)wp.nuw_max * HLQ_UNIT_LUT_BYTES;
+            const size_t k0 = (size_t)(u0 + r.ub) * UNIT;
+            const int nchunks = r.nuw * 32;
+            CHECK(r.nuw <= wp.nuw_max && r.ub + r.nuw <= nU && r.s_begin <= r.s_end && r.s_last < (nst > 0 ? nst : 1), "run");
+            // table build: chunk ci writes 64 bytes at lut + ci * 64 and, as a row leader, float2 xs[ci >> 4]
+            for (int ci = 0; ci < nchunks; ci++) {
+                CHECK(lut + (uint32_t)ci * 64 + 64 <= xs, "lds-table");
+                CHECK(xs + (uint32_t)(ci >> 4) * 8 + 8 <= lut + (uint32_t)wp.wave_lds, "lds-half");
+                CHECK(k0 + (size_t)ci * 4 + 4 <= (size_t)K, "x");
+                if (n_slices_in && ci >= 64) CHECK(lm.stage + ((uint32_t)(k0 >> 2) + ci) * 8 + 8 <= lds_alloc, "lds-stage");
+            }
+            for (int lane = 0; lane < 64; lane++) {
+                CHECK(hlq_x_first_k(k0, nchunks, lane) + 4 <= (size_t)K, "x");
+                if (n_slices_in) {
+                    const int i = hlq_stage_first_index(k0, nchunks, lane, K, clamp_stage);
+                    CHECK(i >= 0 && lm.stage + (uint32_t)i * 8 + 8 <= lds_alloc, "lds-stage");
+                }
+            }
+            // lookups of the wave's sub-tasks: 32 reads of 4 bytes inside the unit's tables, two half-unit records
+            for (int st = r.s_begin; st < r.s_end; st++) {
+                const int lu = st / bits - r.ub;
+                CHECK(lu >= 0 && lut + (uint32_t)lu * HLQ_UNIT_LUT_BYTES + 3 * 8 * 64 + 7 * 64 + 60 + 4 <= xs, "lds-lookup");
+                CHECK(xs + (uint32_t)(2 * lu + 1) * 8 + 8 <= lut + (uint32_t)wp.wave_lds, "lds-half");
+            }
+            // weight stream: slot d holds min(s_begin + d, s_last), refills hold min(st + NSLOT, s_last); every
+            // load is (column block base) + st * 1 KiB + lane * 16, scale / zero rows from the absolute unit
+            for (int d = 0; d < (r.s_end - r.s_begin > nslot ? r.s_end - r.s_begin : nslot) + nslot; d++) {
+                const int st = r.s_begin + d < r.s_last ? r.s_begin + d : r.s_last;
+                for (int cb = 0; cb < ncb; cb += (ncb > 1 ? ncb - 1 : 1)) {
+                    const size_t off = (((size_t)cb * U + u0) * bits + st) * (CB * 16) + 63 * 16 + 16;
+                    CHECK(st >= 0 && off <= planes_bytes, "planes");
+                    const int u = u0 + st / bits, b = st % bits, row = g64 ? u : (u >> 1);
+                    CHECK(row < NT && ((size_t)cb * NT * bits + (size_t)row * bits + b) * (CB * 4) + 63 * 4 + 4 <= scale_bytes, "scales");
+                    CHECK(((size_t)cb * NT + row) * (CB * 4) + 63 * 4 + 4 <= zero_bytes, "zeros");
+                }
+            }
+            // cross-wave sums (two alternating buffers), reduction scratch of the RMSNorm prologue
+            for (int sel = 0; sel < 2; sel++)
+                CHECK(lm.red + ((uint32_t)(sel * waves + wave) * 64 + 63) * 4 + 4 <= lm.rstd, "lds-red");
+            CHECK(lm.rstd + (uint32_t)((waves * 64 - 1) >> 4) * 4 + 4 <= lm.rstd + 64 * 4 && lm.rstd + 64 * 4 + 4 <= lm.stage, "lds-rstd");
+            // partial sums of the slice and handed-over slices
+            CHECK((size_t)slice * npad + (size_t)(ncb - 1) * CB + 63 < (size_t)ksplit * npad, "partial");
+        }
+        // block_rstd: thread tid stages chunks tid, tid + nthreads, ... of the whole K and reads 4 slice rows per chunk
+        if (n_slices_in) {
+            const int wave = -1;
+            for (int i = 0; i < K / 4; i++) CHECK(lm.stage + (uint32_t)i * 8 + 8 <= lds_alloc, "lds-stage");
+            for (int s = 0; s < HLQ_GEMV_MAX_SLICES_IN; s++) {
+                const int row = hlq_slice_row(s, n_slices_in);
+                CHECK(row >= 0 && row < n_slices_in && (size_t)row * K + (size_t)(K / 4 - 1) * 4 + 4 <= (size_t)n_slices_in * K, "slices-in");
+            }
+            const int first = (waves * 64 - 1 < K / 4 - 1 ? waves * 64 - 1 : K / 4 - 1);
+            CHECK(first >= 0 && first < K / 4, "slices-in");
+        }
+    }
+#undef CHECK
+}
+
+}  // namespace
+
+int main(int argc, char **argv)
+{
+    const bool clamp_stage = !(argc > 1 && std::strcmp(argv[1], "--unclamped-stage") == 0);
+    long shapes = 0;
+    const int Us[] = {1, 2, 3, 5, 8, 16, 28, 32, 40, 43, 108, 112};     // K = 128 .. 14336 (4096, 5120, 13824 among them)
+    const int wave_counts[] = {1, 2, 3, 4, 5, 7, 8, 12, 15, 16};
+    for (int bits = 1; bits <= 4; bits++)
+        for (int g64 = 0; g64 < 2; g64++)
+            for (int waves : wave_counts)
+                for (int U : Us)
+                    for (int ups = 1; ups <= U; ups++)
+                        for (int nsl = 0; nsl <= HLQ_GEMV_MAX_SLICES_IN; nsl++)
+                            for (int multi = 0; multi < 2; multi++) {
+                                audit(bits, g64 != 0, waves, U, ups, multi ? 448 : 3, nsl, multi != 0, clamp_stage);
+                                shapes++;
+                            }
+    long total = 0;
+    for (auto &kv : g_viol) {
+        std::printf("category %s %ld\n", kv.first.c_str(), kv.second);
+        total += kv.second;
+    }
+    std::printf("shapes %ld checks %ld\nviolations %ld\n", shapes, g_checked, total);
+    return total ? 1 : 0;
+}

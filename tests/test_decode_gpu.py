@@ -256,3 +256,27 @@ def test_final_rmsnorm_kernel(cuda, n):
     # same formula, different fp32 summation order: at most one fp16 ulp apart
     assert (out.float() - ref.float()).abs().max() <= 2.0 ** -10 * ref.float().abs().max()
     assert (out != ref).float().mean() < 0.02
+
+
+def test_embedding_gather_follows_the_device_token(cuda):
+    """elutq_decode_embed_f16: the row of the token held in device memory (arm_embedding.cpp:4-20); a token
+    outside the table gives a zero row instead of a read outside it."""
+    from elutq_amd import _lib
+    g = torch.Generator(device=cuda).manual_seed(3)
+    for vocab, hidden in ((1000, 512), (37, 4096), (5, 24)):
+        embed = torch.randn(vocab, hidden, generator=g, device=cuda).half()
+        out = torch.full((1, hidden), 7.0, dtype=torch.float16, device=cuda)
+        token = torch.zeros(1, dtype=torch.long, device=cuda)
+        for t in (0, vocab // 2, vocab - 1):
+            token.fill_(t)
+            _lib.check(_lib.lib().elutq_decode_embed_f16(embed.data_ptr(), token.data_ptr(), out.data_ptr(), hidden, vocab,
+                                                         torch.cuda.current_stream().cuda_stream), "embed")
+            assert torch.equal(out[0], embed[t])
+        for t in (-1, vocab, 1 << 40):
+            token.fill_(t)
+            out.fill_(7.0)
+            _lib.check(_lib.lib().elutq_decode_embed_f16(embed.data_ptr(), token.data_ptr(), out.data_ptr(), hidden, vocab,
+                                                         torch.cuda.current_stream().cuda_stream), "embed")
+            assert torch.count_nonzero(out) == 0
+    assert _lib.lib().elutq_decode_embed_f16(None, token.data_ptr(), out.data_ptr(), 512, 10, None) == -1
+    assert _lib.lib().elutq_decode_embed_f16(embed.data_ptr(), token.data_ptr(), out.data_ptr(), 12, 10, None) == -2
