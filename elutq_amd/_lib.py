@@ -28,6 +28,8 @@ SIGNATURES = {
     "elutq_hlq_gemv_f16_tuned": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _ci, _ci]),
     "elutq_hlq_gemv_fused_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
     "elutq_hlq_gemv_slices": (_ci, [_ci] * 6),
+    "elutq_hlq_set_gemv_engine": (_ci, [_ci]),
+    "elutq_hlq_get_gemv_engine": (_ci, []),
     "elutq_hlq_static_scratch_bytes": (_sz, []),
     "elutq_hlq_static_init": (_ci, []),
     "elutq_hlq_gemv_f16_static": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp]),
@@ -93,8 +95,22 @@ def lib() -> ctypes.CDLL:
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)          # AttributeError if the symbol is not exported
             fn.restype, fn.argtypes = res, args
+        # ELUTQ_GEMV_ENGINE=lut|mfma|auto pins the batch-1 GEMV kernel for the process (tests, benchmarks)
+        engine = os.environ.get("ELUTQ_GEMV_ENGINE", "").lower()
+        if engine:
+            if engine not in GEMV_ENGINES:
+                raise RuntimeError(f"ELUTQ_GEMV_ENGINE must be one of {sorted(GEMV_ENGINES)}, not {engine!r}")
+            handle.elutq_hlq_set_gemv_engine(GEMV_ENGINES[engine])
         _lib = handle
     return _lib
+
+
+GEMV_ENGINES = {"auto": 0, "lut": 1, "mfma": 2}
+
+
+def set_gemv_engine(name: str) -> None:
+    """Which kernel the batch-1 GEMV entry points launch: "lut", "mfma" or "auto" (the default)."""
+    check(lib().elutq_hlq_set_gemv_engine(GEMV_ENGINES[name]), "elutq_hlq_set_gemv_engine")
 
 
 def check(status: int, where: str) -> None:

@@ -34,404 +34,9 @@
 #include "hlq_internal.h"
 #include "hlq_gemv_index.h"
 
+#include "hlq_gemv_dev.h"
+
 namespace {
-
-constexpr int MAX_LDS = HLQ_MAX_LDS;
-constexpr int TBL_BYTES = HLQ_TBL_BYTES;             // 16 int32 entries
-constexpr int UNIT_LUT_BYTES = HLQ_UNIT_LUT_BYTES;   // 32 chunks per unit
-
-// Device pointers are declared in the global address space for the device pass: a pointer that a
-// kernel reads out of a struct in memory (the grouped launch) would otherwise be generic, and
-// generic loads count on the LDS counter too, which serialises them with the table lookups.
-#if defined(__HIP_DEVICE_COMPILE__)
-#define HLQ_GLOBAL __attribute__((address_space(1)))
-#else
-#define HLQ_GLOBAL
-#endif
-
-struct GemvArgs {
-    const HLQ_GLOBAL uint4 *planes;
-    const HLQ_GLOBAL uint32_t *scales;
-    const HLQ_GLOBAL uint32_t *zeros;
-    const HLQ_GLOBAL uint16_t *bias;    // fp16 or null
-    const HLQ_GLOBAL uint16_t *x;       // fp16 [K]
-    HLQ_GLOBAL uint16_t *y;             // fp16 [N]
-    HLQ_GLOBAL float *partial;          // [ksplit][ncb*64]   (ksplit > 1)
-    HLQ_GLOBAL unsigned *counters;      // [ncb], zero between calls
-    int N, U, NT, ncb;
-    int ksplit, ups;         // slices per column block, units per slice
-    int spw;                 // sub-tasks per wave (contiguous run)
-    int nuw_max, wave_lds;   // units a wave's run can touch, bytes of its LDS region
-    // optional fusion with the ops around the projection in a decoder layer
-    int prologue;            // 0: x as is; 1: rmsnorm(x) * norm_w; 2: silu(x[0:K]) * x[K:2K]
-    float eps;
-    const HLQ_GLOBAL uint16_t *norm_w;  // fp16 [K]      (prologue 1)
-    const HLQ_GLOBAL uint16_t *residual;  // fp16 [N] added to the output, or null
-    const HLQ_GLOBAL float *extra;        // fp32 [N] added to the output before it is rounded, or null
-    // K slices handed to the next launch instead of being summed here, and the consuming side
-    int defer;                            // 1: write the slices' partial sums to `partial` and nothing else
-    int n_slices_in;                      // > 0: x = fp16(sum of slices_in in order + x), prologue 1 only
-    const HLQ_GLOBAL float *slices_in;    // fp32 [n_slices_in][K]
-    HLQ_GLOBAL uint16_t *x_out;           // fp16 [K] or null: the combined x, written by workgroup (0, 0)
-};
-
-#ifdef HLQ_TIMING
-// Profiling builds only: per-stage wall-clock stamps (100 MHz) of every wave (up to 16) of every
-// workgroup, kept in registers and written once when the tile is done.
-__device__ unsigned long long *g_hlq_stamps = nullptr;
-#define HLQ_STAMP_DECL unsigned long long hlq_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}
-#define HLQ_STAMP(i) hlq_t[i] = wall_clock64()
-#define HLQ_STAMP_FLUSH                                                                           \
-    do {                                                                                          \
-        if (g_hlq_stamps && (threadIdx.x & 63) == 0)                                              \
-            for (int hlq_i = 0; hlq_i < 8; hlq_i++)                                               \
-                g_hlq_stamps[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 8 + hlq_i] = hlq_t[hlq_i]; \
-    } while (0)
-#else
-#define HLQ_STAMP_DECL do { } while (0)
-#define HLQ_STAMP(i) do { } while (0)
-#define HLQ_STAMP_FLUSH do { } while (0)
-#endif
-
-typedef __attribute__((address_space(3))) const int lds_cint;
-
-__device__ __forceinline__ int lds_ld(uint32_t addr, int imm)
-{
-    return *(lds_cint *)(uintptr_t)(addr + (uint32_t)imm);
-}
-
-__device__ __forceinline__ float h2f_lo(uint32_t v) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(v & 0xffffu)); }
-__device__ __forceinline__ float h2f_hi(uint32_t v) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(v >> 16)); }
-
-// dst = base | src.byte<SEL>: the table address of one lookup.  `src` is a plane dword (or its
-// rotation by 4) masked to bits 2..5 of every byte, i.e. 4 * nibble; `base` (wave-uniform, a
-// multiple of 256) is the LDS address of the unit's tables.
-#define HLQ_SDWA_OR(dst, base, src, SEL)                                                       \
-    asm("v_or_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD "         \
-        "src1_sel:BYTE_" #SEL                                                                  \
-        : "=v"(dst)                                                                            \
-        : "s"(base), "v"(src))
-
-// Eight lookups for one plane dword (32 k): chunks 8*D .. 8*D+7 of the unit.  Issue and sum are
-// separate so that the lookups of the next dword are on their way to LDS before the wave waits
-// for the results of this one (LDS returns a wave's reads in order).
-template <int D>
-__device__ __forceinline__ void lookup_issue(uint32_t w, uint32_t base, int (&v)[8])
-{
-    const uint32_t wm = w & 0x3C3C3C3Cu;
-    const uint32_t rm = __builtin_amdgcn_alignbit(w, w, 4) & 0x3C3C3C3Cu;
-    uint32_t a[8];
-    HLQ_SDWA_OR(a[0], base, wm, 0);
-    HLQ_SDWA_OR(a[1], base, rm, 0);
-    HLQ_SDWA_OR(a[2], base, wm, 1);
-    HLQ_SDWA_OR(a[3], base, rm, 1);
-    HLQ_SDWA_OR(a[4], base, wm, 2);
-    HLQ_SDWA_OR(a[5], base, rm, 2);
-    HLQ_SDWA_OR(a[6], base, wm, 3);
-    HLQ_SDWA_OR(a[7], base, rm, 3);
-    constexpr int off = D * 8 * TBL_BYTES;
-#pragma unroll
-    for (int j = 0; j < 8; j++) v[j] = lds_ld(a[j], off + j * TBL_BYTES);
-}
-
-__device__ __forceinline__ int lookup_sum(const int (&v)[8], int acc)
-{
-    acc = acc + v[0] + v[1];
-    acc = acc + v[2] + v[3];
-    acc = acc + v[4] + v[5];
-    acc = acc + v[6] + v[7];
-    return acc;
-}
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
-// A sub-task is one unit of one plane: 128 k of 64 columns = one dwordx4 per lane, plus the
-// meta dword(s) that scale it.
-struct Sub {
-    uint4 w;
-    uint32_t sc;   // fp16 scales of the group pair this unit belongs to (this plane)
-    uint32_t zz;   // fp16 zeros of the pair; loaded for plane 0 only, which folds the zero point
-};
-
-// Byte addresses of one column block's data, uniform over the wave: every load of a sub-task
-// is one of these (scalar registers) plus a 32-bit offset, so the per-load address arithmetic
-// stays short -- the scalar unit is shared by the four SIMDs of a CU and the index arithmetic
-// of sixteen waves would otherwise hold up the start of the weight stream.
-struct CbBase {
-    const HLQ_GLOBAL unsigned char *planes;   // sub-task 0 of the slice
-    const HLQ_GLOBAL unsigned char *scales;   // meta row 0 of the column block
-    const HLQ_GLOBAL unsigned char *zeros;    // meta row 0 of the column block
-};
-
-template <int BITS>
-__device__ __forceinline__ CbBase cb_base(const GemvArgs &a, int cb, int u0)
-{
-    CbBase p;
-    p.planes = (const HLQ_GLOBAL unsigned char *)a.planes + ((size_t)cb * a.U + u0) * (size_t)(BITS * HLQ_CB * 16);
-    p.scales = (const HLQ_GLOBAL unsigned char *)a.scales + (size_t)cb * a.NT * (size_t)(BITS * HLQ_CB * 4);
-    p.zeros = (const HLQ_GLOBAL unsigned char *)a.zeros + (size_t)cb * a.NT * (size_t)(HLQ_CB * 4);
-    return p;
-}
-
-// st = sub-task index inside the slice (unit u0 + st / BITS, plane st % BITS); planes of a
-// slice are contiguous in st.
-template <int BITS, bool G64, bool SC = true, bool ZZ = true>
-__device__ __forceinline__ void load_sub(Sub &t, const CbBase &p, int u0, int st, int lane)
-{
-    const uint32_t u = (uint32_t)(u0 + st / BITS), b = (uint32_t)(st % BITS);
-    const uint32_t row = G64 ? u : (u >> 1);
-    const u32x4 v = __builtin_nontemporal_load(
-        (const HLQ_GLOBAL u32x4 *)(p.planes + ((uint32_t)st * (uint32_t)(HLQ_CB * 16) + (uint32_t)lane * 16u)));
-    t.w = make_uint4(v.x, v.y, v.z, v.w);
-    if (SC) t.sc = *(const HLQ_GLOBAL uint32_t *)(p.scales + ((row * BITS + b) * (uint32_t)(HLQ_CB * 4) + (uint32_t)lane * 4u));
-    if (ZZ) t.zz = *(const HLQ_GLOBAL uint32_t *)(p.zeros + (row * (uint32_t)(HLQ_CB * 4) + (uint32_t)lane * 4u));
-}
-
-// Sub-tasks that share scale / zero dwords form a meta group: the planes of one unit at
-// G = 64, of a unit pair at G = 128.  When every wave's run starts on a group boundary and the
-// slots hold whole groups (`PAIRED`), position d of a pass is a compile-time (unit, plane) of
-// its group: only the first unit's positions load the scale dword of their plane, only position 0
-// the zero dword -- 7 loads instead of 12 for the four sub-tasks of a w2g128 pair -- and the
-// later positions reuse the values.  Otherwise every sub-task loads both (3 loads each, so
-// that the load count behind any point is still a compile-time constant).
-template <int BITS, bool G64>
-struct MetaGroup {
-    static constexpr int SIZE = G64 ? BITS : 2 * BITS;           // sub-tasks per group
-    static constexpr bool fits(int nslot) { return nslot % SIZE == 0; }
-    static constexpr bool sc_at(int d) { return d % SIZE < BITS; }
-    static constexpr bool zz_at(int d) { return d % SIZE == 0; }
-};
-
-template <int BITS, bool G64, bool PAIRED, int D>
-__device__ __forceinline__ void load_slot(Sub &t, const CbBase &p, int u0, int st, int lane)
-{
-    using MG = MetaGroup<BITS, G64>;
-    load_sub<BITS, G64, !PAIRED || MG::sc_at(D), !PAIRED || MG::zz_at(D)>(t, p, u0, st, lane);
-}
-
-// The two 64-k halves of a unit have their own table scale (2^-p) and activation sum; at
-// G = 64 they are also two quantization groups (lo / hi half of the meta dwords), at G = 128
-// one group (the half of the meta dwords selected by the unit's parity).
-template <bool G64>
-__device__ __forceinline__ float process_sub(const uint4 &w, uint32_t sc_raw, uint32_t zz_raw, int lu, int b, int odd,
-                                             uint32_t lut_base, const float2 *xs_inv, float acc)
-{
-    int v0[8], v1[8];
-    const uint32_t ub = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lut_base + (uint32_t)lu * UNIT_LUT_BYTES));
-    const float2 h0 = xs_inv[2 * lu], h1 = xs_inv[2 * lu + 1];      // .x = sum of x, .y = 2^-p
-    lookup_issue<0>(w.x, ub, v0);
-    lookup_issue<1>(w.y, ub, v1);
-    __builtin_amdgcn_sched_barrier(0);
-    int i0 = lookup_sum(v0, 0);
-    lookup_issue<2>(w.z, ub, v0);
-    __builtin_amdgcn_sched_barrier(0);
-    i0 = lookup_sum(v1, i0);
-    lookup_issue<3>(w.w, ub, v1);
-    __builtin_amdgcn_sched_barrier(0);
-    int i1 = lookup_sum(v0, 0);
-    i1 = lookup_sum(v1, i1);
-    const uint32_t sc = G64 ? sc_raw : (odd ? (sc_raw >> 16) * 0x10001u : (sc_raw & 0xffffu) * 0x10001u);
-    acc = fmaf((float)i0 * h0.y, h2f_lo(sc), acc);
-    acc = fmaf((float)i1 * h1.y, h2f_hi(sc), acc);
-    if (b == 0) {
-        const uint32_t zz = G64 ? zz_raw : (odd ? (zz_raw >> 16) * 0x10001u : (zz_raw & 0xffffu) * 0x10001u);
-        acc = fmaf(h2f_lo(zz), h0.x, acc);
-        acc = fmaf(h2f_hi(zz), h1.x, acc);
-    }
-    return acc;
-}
-
-// DPP lane exchanges inside a row of 16 lanes (no LDS traffic).
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
-}
-// all-reduce over the 16 lanes of a row: xor 1, xor 2 (quad_perm), then half-row and row mirrors
-#define HLQ_ROW_REDUCE(v, OP)             \
-    v = OP(v, dpp_f<0xB1>(v));            \
-    v = OP(v, dpp_f<0x4E>(v));            \
-    v = OP(v, dpp_f<0x141>(v));           \
-    v = OP(v, dpp_f<0x140>(v))
-__device__ __forceinline__ float op_add(float a, float b) { return a + b; }
-__device__ __forceinline__ float op_max(float a, float b) { return fmaxf(a, b); }
-
-// The four activations of a chunk after the optional prologue, as fp32 values that are
-// exactly representable in fp16 (the fused ops round to fp16 where the unfused pipeline
-// would have stored fp16: RMSNorm output, arm_rmsnorm.cpp:25-84; SiLU(gate)*up,
-// arm_activation.cpp:36-49).
-__device__ __forceinline__ void chunk_values(int prologue, uint2 raw, uint2 raw2, float rstd, float (&v)[4])
-{
-    v[0] = h2f_lo(raw.x); v[1] = h2f_hi(raw.x); v[2] = h2f_lo(raw.y); v[3] = h2f_hi(raw.y);
-    if (prologue == 0) return;
-    const float w[4] = {h2f_lo(raw2.x), h2f_hi(raw2.x), h2f_lo(raw2.y), h2f_hi(raw2.y)};
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        float t;
-        if (prologue == 1) t = v[i] * rstd * w[i];
-        else t = v[i] / (1.0f + __expf(-v[i])) * w[i];
-        v[i] = (float)(_Float16)t;
-    }
-}
-
-// Always two loads (without a prologue the second one re-reads the chunk): a fixed number
-// of loads lets the compiler wait for these with an exact vector-memory count while the
-// weight loads issued after them are still in flight.
-template <bool PLAIN>
-__device__ __forceinline__ void load_chunk(const GemvArgs &a, int prologue, int K, size_t k, uint2 &raw, uint2 &raw2)
-{
-    raw = *(const HLQ_GLOBAL uint2 *)(a.x + k);
-    if (PLAIN) {            // no prologue at compile time: one load
-        raw2 = raw;
-        return;
-    }
-    const HLQ_GLOBAL uint16_t *second = prologue == 1 ? a.norm_w + k : (prologue == 2 ? a.x + (size_t)K + k : a.x + k);
-    raw2 = *(const HLQ_GLOBAL uint2 *)second;
-}
-
-// Subset-sum table of one chunk of 4 activations as int32 fixed point, 64 bytes at `tbl`.
-// The 16 lanes of a DPP row cover one 64-k half unit, whose max|x| sets the power-of-two
-// table scale and whose sum feeds the zero-point fold (row leader stores both in *half).
-__device__ __forceinline__ void build_chunk(int prologue, uint2 raw, uint2 raw2, float rstd, unsigned char *tbl,
-                                            float2 *half, bool leader)
-{
-    float v[4];
-    chunk_values(prologue, raw, raw2, rstd, v);
-    const float x0 = v[0], x1 = v[1], x2 = v[2], x3 = v[3];
-    float amax = fmaxf(fmaxf(fabsf(x0), fabsf(x1)), fmaxf(fabsf(x2), fabsf(x3)));
-    float s = (x0 + x1) + (x2 + x3);
-    HLQ_ROW_REDUCE(s, op_add);
-    HLQ_ROW_REDUCE(amax, op_max);
-    // amax < 2^(eb-126): scale by 2^(149-eb) so |x * scale| < 2^23, a 4-subset < 2^25 and
-    // the 16 lookups of a half unit < 2^29.
-    const uint32_t eb = (__float_as_uint(amax) >> 23) & 0xffu;
-    const float scale = eb ? __uint_as_float((276u - eb) << 23) : 1.0f;
-    const float inv = eb ? __uint_as_float((eb - 22u) << 23) : 1.0f;
-    const int i0 = __float2int_rn(x0 * scale), i1 = __float2int_rn(x1 * scale);
-    const int i2 = __float2int_rn(x2 * scale), i3 = __float2int_rn(x3 * scale);
-    const int e3 = i0 + i1, e5 = i0 + i2, e6 = i1 + i2, e7 = e3 + i2;
-    int4 *dst = (int4 *)tbl;
-    dst[0] = make_int4(0, i0, i1, e3);
-    dst[1] = make_int4(i2, e5, e6, e7);
-    dst[2] = make_int4(i3, i3 + i0, i3 + i1, i3 + e3);
-    dst[3] = make_int4(i3 + i2, i3 + e5, i3 + e6, i3 + e7);
-    if (leader) *half = make_float2(s, inv);
-}
-
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
-// outstanding global load of the wave (its fence covers all address spaces), which here would
-// be the weight loads that are meant to stay in flight across the barrier.
-__device__ __forceinline__ void lds_barrier()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-// 1 / rms of the whole activation vector for the fused RMSNorm prologue: the workgroup sums
-// the squares together (one chunk per thread and pass), two barriers.  `scratch` is LDS of
-// HLQ_RSTD_SCRATCH floats (at hlq_lds_map().rstd).  Every workgroup does this for itself (2K bytes from cache).
-
-// Activations that arrive as a base vector plus the unsummed K slices of the launch that
-// produced them (its `defer` mode): element k is fp16(((s0[k] + s1[k]) + ...) + x[k]), the same
-// operations in the same order as that launch's own output stage would have used.
-constexpr int GEMV_MAX_SLICES_IN = HLQ_GEMV_MAX_SLICES_IN;
-
-struct SliceChunk {
-    float4 p[GEMV_MAX_SLICES_IN];
-};
-
-__device__ __forceinline__ void load_slice_chunk(const GemvArgs &a, int K, int chunk, SliceChunk &c)
-{
-#pragma unroll
-    for (int s = 0; s < GEMV_MAX_SLICES_IN; s++)     // always GEMV_MAX_SLICES_IN loads: a fixed count
-        c.p[s] = *(const HLQ_GLOBAL float4 *)(a.slices_in + (size_t)hlq_slice_row(s, a.n_slices_in) * K + (size_t)chunk * 4);
-}
-
-__device__ __forceinline__ uint2 combine_chunk(const GemvArgs &a, uint2 base, const SliceChunk &c)
-{
-    float v[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < GEMV_MAX_SLICES_IN; s++)
-        if (s < a.n_slices_in) { v[0] += c.p[s].x; v[1] += c.p[s].y; v[2] += c.p[s].z; v[3] += c.p[s].w; }
-    v[0] += h2f_lo(base.x); v[1] += h2f_hi(base.x); v[2] += h2f_lo(base.y); v[3] += h2f_hi(base.y);
-    auto pack = [](float lo, float hi) __attribute__((always_inline)) {
-        return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
-    };
-    return make_uint2(pack(v[0], v[1]), pack(v[2], v[3]));
-}
-
-// The chunk of x this thread squares first; issued ahead of the other loads of the tile so that
-// the reduction below overlaps with them.
-__device__ __forceinline__ uint2 rstd_first_load(const GemvArgs &a, int K, int tid)
-{
-    return *(const HLQ_GLOBAL uint2 *)(a.x + (size_t)min(tid, K / 4 - 1) * 4);
-}
-
-// With slices (`sliced`) every chunk of the combined x is formed here once, kept in
-// `stage` (LDS, fp16 [K]) for the table builds and, by the first workgroup, written to a.x_out.
-__device__ __forceinline__ float block_rstd(const GemvArgs &a, int K, float *scratch, int tid, int nthreads, uint2 first,
-                                            const SliceChunk &sfirst, bool sliced, uint2 *stage, bool write_out)
-{
-    auto sq4 = [](uint2 r) __attribute__((always_inline)) {
-        const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
-        return (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
-    };
-    float ssq = 0.f;
-    if (sliced) {
-        for (int i = tid; i < K / 4; i += nthreads) {
-            uint2 r;
-            if (i == tid) r = combine_chunk(a, first, sfirst);
-            else {
-                SliceChunk c;
-                load_slice_chunk(a, K, i, c);
-                r = combine_chunk(a, *(const HLQ_GLOBAL uint2 *)(a.x + (size_t)i * 4), c);
-            }
-            stage[i] = r;
-            if (write_out) *(HLQ_GLOBAL uint2 *)(a.x_out + (size_t)i * 4) = r;
-            ssq += sq4(r);
-        }
-    } else {
-        ssq = tid < K / 4 ? sq4(first) : 0.f;
-        for (int i = tid + nthreads; i < K / 4; i += nthreads) ssq += sq4(*(const HLQ_GLOBAL uint2 *)(a.x + (size_t)i * 4));
-    }
-    HLQ_ROW_REDUCE(ssq, op_add);
-    if ((tid & 15) == 0) scratch[tid >> 4] = ssq;
-    lds_barrier();
-    if (tid < 64) {
-        float v = tid < (nthreads >> 4) ? scratch[tid] : 0.f;
-        HLQ_ROW_REDUCE(v, op_add);
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
-        if (tid == 0) scratch[64] = v;
-    }
-    lds_barrier();
-    return rsqrtf(scratch[64] / (float)K + a.eps);
-}
-
-// A SIMD issues from its oldest wave first, so the waves of a workgroup finish their runs one
-// after the other and the last one works alone at the end.  Every wave therefore lowers its own
-// priority as it gets on with its run (3 at the start, 0 in the last quarter): the waves that are
-// behind are served first and all finish together.
-__device__ __forceinline__ void progress_prio(int done, int total)
-{
-    const int d4 = done * 4;                 // quarter of the run the wave is in, without a division
-    if (d4 < total) __builtin_amdgcn_s_setprio(3);
-    else if (d4 < 2 * total) __builtin_amdgcn_s_setprio(2);
-    else if (d4 < 3 * total) __builtin_amdgcn_s_setprio(1);
-    else __builtin_amdgcn_s_setprio(0);
-}
-
-// Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
-template <int B, int E, typename F>
-__device__ __forceinline__ void static_for(F &&f)
-{
-    if constexpr (B < E) {
-        f(std::integral_constant<int, B>{});
-        static_for<B + 1, E>(f);
-    }
-}
-
 // Sub-tasks a wave keeps in flight at most.  Three planes get six slots and four planes eight: a
 // unit pair (one meta group at G = 128) is that many sub-tasks, and K = 4096 gives a wave exactly
 // that run -- so a layer with more column blocks than CUs can run as column-block runs (which need
@@ -456,7 +61,6 @@ constexpr int depth_of(int bits) { return bits == 3 ? 6 : (bits == 4 ? 8 : 4); }
 //   GEMV_FUSED  prologue and residual as `a` says (the decode step's launches)
 //   GEMV_PLAIN  none of them (their fields of `a` are not read)
 //   GEMV_EXTRA  plain, plus the fp32 term `a.extra` added before the output is rounded
-enum { GEMV_FUSED = 0, GEMV_PLAIN = 1, GEMV_EXTRA = 2 };
 template <int BITS, bool G64, int NSLOT, bool MULTI, int VAR, bool PAIRED>
 __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, int ncb_run, unsigned char *smem, int &red_sel)
 {
@@ -943,6 +547,55 @@ void choose_shape(const HlqGeo &g, int &ksplit, int &waves)
     if (waves <= 0) waves = 16;
 }
 
+int g_gemv_engine = ELUTQ_GEMV_ENGINE_AUTO;
+
+// The launch shape of a batch-1 GEMV: which kernel, K slices, units per slice, waves per workgroup.  One
+// function for the launch itself and for the queries about it (elutq_hlq_gemv_slices, _accepts_slices).
+struct LaunchShape {
+    bool mfma;
+    int ksplit, ups, waves;
+};
+
+int plan_launch(const HlqGeo &g, int bits, int ksplit, int waves, LaunchShape &sh)
+{
+    if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return ELUTQ_ERR_TUNING;
+    const bool auto_waves = waves <= 0;
+    // measured on MI355X: the matrix-core kernel streams large layers as fast as the LUT kernel but a launch of one
+    // tile per workgroup takes 0.5-1 us longer (its A operands cost more to build than the tables), so the
+    // library's own choice is the LUT kernel throughout
+    sh.mfma = g_gemv_engine == ELUTQ_GEMV_ENGINE_MFMA;
+    choose_shape(g, ksplit, waves);
+    int ups = (g.U + ksplit - 1) / ksplit;
+    if (sh.mfma) {
+        // slices start on a unit pair (at G = 128 a pair shares its scale / zero dwords), and a wave holds the A
+        // operands of at most two pairs: 16 waves x 2 pairs x 256 k = 8192 k per slice
+        if (ksplit > 1 && (ups & 1)) ups++;
+        while ((ups + 1) / 2 > 2 * 16) ups = ((ups + 1) / 2 + 1) & ~1;
+        ksplit = (g.U + ups - 1) / ups;
+        const int npairs = (ups + 1) / 2;
+        if (auto_waves) waves = npairs < 16 ? npairs : 16;
+        if ((npairs + waves - 1) / waves > 2) {
+            if (g_gemv_engine == ELUTQ_GEMV_ENGINE_MFMA) return ELUTQ_ERR_TUNING;      // the caller's wave count is too small
+            sh.mfma = false;
+        }
+    }
+    if (!sh.mfma) {
+        // shrink the slice so its tables fit in LDS, then the slice count so that no slice is empty
+        ups = (g.U + ksplit - 1) / ksplit;
+        while (gemv_lds_bytes(ups, bits, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
+        ksplit = (g.U + ups - 1) / ups;
+        // a slice of at most 16 sub-tasks: eight waves with two each start sooner than sixteen with one
+        if (auto_waves && ups * bits <= 16) waves = 8;
+    }
+    sh.ksplit = ksplit; sh.ups = ups; sh.waves = waves;
+    return ELUTQ_OK;
+}
+
+size_t shape_lds_bytes(const LaunchShape &sh, int bits)
+{
+    return sh.mfma ? hlq_gemv_mfma_lds_bytes(sh.ups, sh.waves) : gemv_lds_bytes(sh.ups, bits, sh.waves);
+}
+
 }  // namespace
 
 extern "C" {
@@ -993,15 +646,11 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     if (rc != ELUTQ_OK) return rc;
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
     const HlqGeo g = hlq_geo(K, N, bits, group);
-    if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return ELUTQ_ERR_TUNING;
-    const bool auto_waves = waves <= 0;
-    choose_shape(g, ksplit, waves);
-    int ups = (g.U + ksplit - 1) / ksplit;
-    // shrink the slice so its tables fit in LDS, then the slice count so that no slice is empty
-    while (gemv_lds_bytes(ups, bits, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
-    ksplit = (g.U + ups - 1) / ups;
-    // a slice of at most 16 sub-tasks: eight waves with two each start sooner than sixteen with one
-    if (auto_waves && ups * bits <= 16) waves = 8;
+    LaunchShape sh;
+    rc = plan_launch(g, bits, ksplit, waves, sh);
+    if (rc != ELUTQ_OK) return rc;
+    ksplit = sh.ksplit; waves = sh.waves;
+    const int ups = sh.ups;
 
     GemvArgs a;
     a.planes = (const HLQ_GLOBAL uint4 *)d_planes;
@@ -1039,7 +688,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         if ((long long)g.ncb * ksplit > NUM_CU) return ELUTQ_ERR_TUNING;
         a.x_out = (HLQ_GLOBAL uint16_t *)fusion->d_x_out;
         stage_bytes = (size_t)K * sizeof(uint16_t);
-        if (gemv_lds_bytes(ups, bits, waves) + stage_bytes > (size_t)MAX_LDS) return ELUTQ_ERR_SHAPE;
+        if (shape_lds_bytes(sh, bits) + stage_bytes > (size_t)MAX_LDS) return ELUTQ_ERR_SHAPE;
     }
     if (fusion && fusion->d_slices_out) {
         // the K slices stay unsummed for the next launch: nothing else may be due in the output stage
@@ -1054,8 +703,19 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         a.counters = (HLQ_GLOBAL unsigned *)d_workspace;
         a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
+    if (sh.mfma) return hlq_gemv_mfma_launch(&a, sizeof(a), bits, group, waves, stage_bytes, stream);
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves) + stage_bytes, (hipStream_t)stream);
 }
+
+extern "C" int elutq_hlq_set_gemv_engine(int engine)
+{
+    if (engine != ELUTQ_GEMV_ENGINE_AUTO && engine != ELUTQ_GEMV_ENGINE_LUT && engine != ELUTQ_GEMV_ENGINE_MFMA)
+        return ELUTQ_ERR_TUNING;
+    g_gemv_engine = engine;
+    return ELUTQ_OK;
+}
+
+extern "C" int elutq_hlq_get_gemv_engine(void) { return g_gemv_engine; }
 
 // Whether a launch of this shape (ksplit / waves as the call would pass them) takes `n_slices` handed-over
 // K slices in its RMSNorm prologue: the same steps and limits as the launch itself.
@@ -1064,24 +724,19 @@ extern "C" int elutq_hlq_gemv_accepts_slices(int K, int N, int bits, int group, 
     if (check_shape(K, N, bits, group) != ELUTQ_OK) return 0;
     if (n_slices < 1 || n_slices > GEMV_MAX_SLICES_IN) return 0;
     const HlqGeo g = hlq_geo(K, N, bits, group);
-    if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return 0;
-    choose_shape(g, ksplit, waves);
-    int ups = (g.U + ksplit - 1) / ksplit;
-    while (gemv_lds_bytes(ups, bits, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
-    ksplit = (g.U + ups - 1) / ups;
-    if ((long long)g.ncb * ksplit > NUM_CU) return 0;
-    return gemv_lds_bytes(ups, bits, waves) + (size_t)K * sizeof(uint16_t) <= (size_t)MAX_LDS ? 1 : 0;
+    LaunchShape sh;
+    if (plan_launch(g, bits, ksplit, waves, sh) != ELUTQ_OK) return 0;
+    if ((long long)g.ncb * sh.ksplit > NUM_CU) return 0;
+    return shape_lds_bytes(sh, bits) + (size_t)K * sizeof(uint16_t) <= (size_t)MAX_LDS ? 1 : 0;
 }
 
 extern "C" int elutq_hlq_gemv_slices(int K, int N, int bits, int group, int ksplit, int waves)
 {
     if (check_shape(K, N, bits, group) != ELUTQ_OK) return 0;
     const HlqGeo g = hlq_geo(K, N, bits, group);
-    if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return 0;
-    choose_shape(g, ksplit, waves);                      // the same steps as the launch itself
-    int ups = (g.U + ksplit - 1) / ksplit;
-    while (gemv_lds_bytes(ups, bits, waves) > (size_t)MAX_LDS) ups = (ups + 1) / 2;
-    return (g.U + ups - 1) / ups;
+    LaunchShape sh;
+    if (plan_launch(g, bits, ksplit, waves, sh) != ELUTQ_OK) return 0;          // the same steps as the launch itself
+    return sh.ksplit;
 }
 
 extern "C" {

@@ -20,3 +20,11 @@ HLQ_INTERNAL int hlq_gemm_chunk_with_extra(const void *d_planes, const void *d_s
                                            const void *d_bias, const void *d_x, void *d_y, int M, int K, int N, int bits,
                                            int group, void *d_workspace, size_t workspace_bytes, void *stream, int kparts,
                                            int ksplit, const float *d_extra);
+
+// The matrix-core GEMV kernel (hlq_gemv_mfma.hip).  `gemv_args` is the launcher's argument block as
+// hlq_gemv.hip fills it for the LUT kernel (hlq_gemv_dev.h: GemvArgs); ELUTQ_ERR_TUNING if a wave would
+// have to hold more than two unit pairs.  hlq_gemv_mfma_lds_bytes: dynamic LDS of a launch without staged
+// activations.
+HLQ_INTERNAL int hlq_gemv_mfma_launch(const void *gemv_args, size_t args_bytes, int bits, int group, int waves,
+                                      size_t stage_bytes, void *stream);
+HLQ_INTERNAL size_t hlq_gemv_mfma_lds_bytes(int ups, int waves);

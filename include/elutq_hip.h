@@ -82,6 +82,22 @@ int elutq_hlq_unpack_host(const void *h_planes, const void *h_scales, const void
                           int K, int N, int bits, int group,
                           uint8_t *h_w_quant_out, uint16_t *h_w_scale_out, uint16_t *h_w_zero_out);
 
+/*
+ * Which kernel the batch-1 GEMV entry points launch (process-wide; for tests, benchmarks and debugging):
+ *   ELUTQ_GEMV_ENGINE_LUT   activation tables in LDS, 4-bit lookups (the T-MAC scheme of the reference's
+ *                           t_mac_g4_float_update_impl, C++/ops/src/arm/arm_t_mac_kernal.cpp:364-469)
+ *   ELUTQ_GEMV_ENGINE_MFMA  the plane bits go to the matrix cores as fp4 operands against fixed-point
+ *                           digits of the activations; no lookups
+ *   ELUTQ_GEMV_ENGINE_AUTO  the library's choice per shape (the default)
+ * Both compute the same sums (fp32 fold per group and plane); results agree to the final fp16 rounding and
+ * are bit-identical where the arithmetic is exact.  Returns ELUTQ_ERR_TUNING for another value.
+ */
+#define ELUTQ_GEMV_ENGINE_AUTO 0
+#define ELUTQ_GEMV_ENGINE_LUT 1
+#define ELUTQ_GEMV_ENGINE_MFMA 2
+int elutq_hlq_set_gemv_engine(int engine);
+int elutq_hlq_get_gemv_engine(void);
+
 /* Workspace size for a call with up to M activation rows. */
 size_t elutq_hlq_workspace_bytes(int K, int N, int bits, int group, int M);
 
