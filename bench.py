@@ -31,6 +31,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+KERNEL_TRACE_AVG_US = 6.51     # hlq_gemv_kernel<2, false, 4, true, 1> at 4096 x 14336 in the committed kernel trace
 BITS, GROUP = 2, 128
 N_LAYERS = 32
 
@@ -44,10 +45,16 @@ def parse():
     p.add_argument("--no-decode", action="store_true", help="skip the decode tokens/s leg")
     p.add_argument("--no-gemm", action="store_true", help="skip the small-batch GEMM leg")
     p.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
-    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "gemm", "group", "sparse"], default="full",
+    p.add_argument("--sweep-only", action="store_true",
+                   help="only the sweep and the per-shape rings of the per-GEMV entry point (no grouped / multi-stream / "
+                        "copy / other-format / large-shape legs): the run a kernel trace of the dominant kernel is taken from")
+    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "decode-eager", "gemm", "group", "sparse", "shape-sweep"],
+                   default="full",
                    help="kernel: only the dominant GEMV (4096x14336) over its weight ring, for counter runs; "
                         "copy: a plain 64 MiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE; "
                         "decode / gemm: only that leg (for kernel traces); "
+                        "decode-eager: three eager decode steps of a two-layer model of the same widths (for counter runs); "
+                        "shape-sweep: the small LLaMA-3-8B shapes at every K split x wave count of the tuned entry point; "
                         "sparse: GEMVs of layers with a block-sparse extra plane beside the same layers without it")
     p.add_argument("--launches", type=int, default=256, help="launches in --mode kernel / copy")
     return p.parse_args()
@@ -119,7 +126,32 @@ def cpu_baseline(budget_s):
                 break
         dt = (time.perf_counter() - t0) / reps
         out[threads] = {"GBps": nbytes / dt / 1e9, "ms_per_layer": dt * 1e3, "reps": reps}
+    # the op-for-op restatement (every fp16 rounding of the reference chain, F16C conversions around each
+    # operation; scalar inner loop) on the 4096 x 4096 projection, one thread and the reference's four
+    kq = (4096, 4096)
+    faithful = {}
+    for threads in (1, 4):
+        rw = lutref.RefWeight(weights[kq].w_quant, weights[kq].w_scale, weights[kq].w_zero, GROUP, threads)
+        rw.gemv(weights[kq].x[0])
+        t0, reps = time.perf_counter(), 0
+        while reps < 3 or time.perf_counter() - t0 < 1.0:
+            rw.gemv(weights[kq].x[0])
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        faithful[threads] = {"GBps": algorithmic_bytes(*kq, BITS, GROUP) / dt / 1e9, "ms_per_gemv": dt * 1e3, "reps": reps}
+    out["fp16_faithful_4096x4096"] = faithful
     return out, ncpu
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16
@@ -244,79 +276,11 @@ def counter_mode(a, torch, lib, dev):
                       "ring_sets": len(ring)}))
 
 
-def main():
-    a = parse()
-    if a.gpus != 1:
-        print(f"bench.py: this build measures ONE GPU (the path needs no collective); --gpus {a.gpus} is not supported",
-              file=sys.stderr)
-        sys.exit(2)
-    import torch
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(1)
-    from elutq_amd import _lib
-    from elutq_amd.synth import LLAMA3_8B_SHAPES, algorithmic_bytes, make_device_layer
-
-    lib = _lib.lib()
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    if a.mode == "decode":
-        from elutq_amd.llama_decode import bench_decode
-        print(json.dumps({"mode": "decode", "decode": bench_decode(dev),
-                          "decode_hlq_lm_head": bench_decode(dev, hlq_lm_head=True)}))
-        return
-    if a.mode == "gemm":
-        print(json.dumps({"mode": "gemm", "gemm_w2g128_llama2_13b": gemm_leg(torch, lib, dev, a.steps)}))
-        return
-    if a.mode == "group":
-        # the whole sweep as one grouped launch, `steps` times (for rocprofv3 --kernel-trace)
-        from elutq_amd.hlq_linear import GemvGroup
-        mods, nbytes = [], 0
-        for i in range(N_LAYERS):
-            for (k, n) in LLAMA3_8B_SHAPES.values():
-                mods.append(make_device_layer(k, n, BITS, GROUP, seed=len(mods), device=dev))
-                nbytes += algorithmic_bytes(k, n, BITS, GROUP)
-        xk = {k: torch.randn(1, k, device=dev).to(torch.float16) for k in {m.in_features for m in mods}}
-        grp = GemvGroup(mods, [xk[m.in_features] for m in mods],
-                        [torch.empty(1, m.out_features, dtype=torch.float16, device=dev) for m in mods])
-        sec = time_graph(torch, lambda s: grp.run(), a.steps, a.warmup)
-        print(json.dumps({"mode": "group", "gemvs_per_launch": len(mods), "bytes_per_launch": nbytes, "us_per_launch": sec * 1e6,
-                          "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}))
-        grp.close()
-        return
-    if a.mode == "sparse":
-        print(json.dumps({"mode": "sparse", "sparse_gemv_w2g128": sparse_leg(torch, lib, dev, a.steps, a.warmup)}))
-        return
-    if a.mode != "full":
-        counter_mode(a, torch, lib, dev)
-        return
-    ws_bytes = max(lib.elutq_hlq_workspace_bytes(k, n, BITS, GROUP, 1) for (k, n) in LLAMA3_8B_SHAPES.values())
-    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
-    xs = {k: torch.randn(1, k, device=dev).to(torch.float16) for k in {k for k, _ in LLAMA3_8B_SHAPES.values()}}
-    ys = {n: torch.empty(1, n, dtype=torch.float16, device=dev) for n in {n for _, n in LLAMA3_8B_SHAPES.values()}}
-
-    # ---- the sweep: 32 layers x 7 projections, all weight sets distinct -----------------
-    calls = []
-    step_bytes = 0
-    seed = 0
-    for layer in range(N_LAYERS):
-        for name, (k, n) in LLAMA3_8B_SHAPES.items():
-            mod = make_device_layer(k, n, BITS, GROUP, seed=seed, device=dev)
-            seed += 1
-            calls.append(Gemv(lib, mod, xs[k], ys[n], ws))
-            step_bytes += algorithmic_bytes(k, n, BITS, GROUP)
-    torch.cuda.synchronize()
-
-    def launch_step(stream):
-        for c in calls:
-            c(stream)
-
-    sec_step = time_graph(torch, launch_step, a.steps, a.warmup)
-    value = step_bytes / sec_step / 1e9
-
-    # ---- the same sweep through the grouped entry point: one launch for all 224 GEMVs, and one
-    # launch per layer (7 GEMVs); every GEMV writes its own output ---------------------------------
+def side_legs(a, torch, lib, dev, calls, xs, ws_bytes, step_bytes):
+    """The same 224 GEMVs through the grouped entry point (one launch, one launch per layer), the per-GEMV launches
+    dealt onto four streams of one graph, and a plain device copy as a yardstick."""
     from elutq_amd.hlq_linear import GemvGroup
+    from elutq_amd.synth import LLAMA3_8B_SHAPES
     g_mods = [c.mod for c in calls]
     g_xs = [xs[m.in_features] for m in g_mods]
     g_ys = [torch.empty(1, m.out_features, dtype=torch.float16, device=dev) for m in g_mods]
@@ -367,6 +331,139 @@ def main():
     del cp_a, cp_b
     torch.cuda.empty_cache()
 
+    return grouped
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print(f"bench.py: this build measures ONE GPU (the path needs no collective); --gpus {a.gpus} is not supported",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    from elutq_amd import _lib
+    from elutq_amd.synth import LLAMA3_8B_SHAPES, algorithmic_bytes, make_device_layer
+
+    lib = _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if a.mode == "decode":
+        from elutq_amd.llama_decode import bench_decode
+        print(json.dumps({"mode": "decode", "decode": bench_decode(dev),
+                          "decode_hlq_lm_head": bench_decode(dev, hlq_lm_head=True)}))
+        return
+    if a.mode == "decode-eager":
+        # a reduced decode for counter runs (rocprofv3 --pmc serialises every dispatch, and the full 32-layer graph
+        # replay does not finish under it): two layers of the LLaMA-3-8B widths, three eager steps, no graph
+        from elutq_amd.hlq_linear import HLQLinear
+        from elutq_amd.llama_decode import LlamaDecoder, LlamaShape
+        shape = LlamaShape(n_layers=2)
+        model = LlamaDecoder(shape, device=dev, seed=0, impl="hip")
+        model.fill_cache(512)
+        model.token.fill_(1)
+        steps = 3
+        for _ in range(steps):
+            model.step()
+        torch.cuda.synchronize()
+        hlq_bytes = sum(m.planes.numel() + m.scales.numel() + m.zeros.numel() for m in model.modules() if isinstance(m, HLQLinear))
+        kv_bytes = 2 * shape.n_layers * 512 * shape.n_kv_heads * shape.head_dim * 2
+        print(json.dumps({"mode": "decode-eager", "layers": shape.n_layers, "steps": steps,
+                          "algorithmic_bytes_per_step": {"hlq_layers": hlq_bytes, "fp16_lm_head": model.lm_head.numel() * 2,
+                                                         "kv_cache_read": kv_bytes, "embedding_row": shape.hidden * 2}}))
+        return
+    if a.mode == "shape-sweep":
+        # what a launch of the two small shapes costs however its work is arranged: every K split x wave count of the
+        # tuned entry point (and both kernels), each over a ring of distinct weight sets, one graph replay per ring
+        from elutq_amd.synth import make_device_layer as mk
+        table = {}
+        for (k, n) in ((4096, 1024), (4096, 4096)):
+            nbytes = algorithmic_bytes(k, n, BITS, GROUP)
+            ring = [mk(k, n, BITS, GROUP, seed=i, device=dev) for i in range(max(8, -(-400 * 2 ** 20 // nbytes)))]
+            x = torch.randn(1, k, device=dev).to(torch.float16)
+            y = torch.empty(1, n, dtype=torch.float16, device=dev)
+            ws = torch.zeros(max(lib.elutq_hlq_workspace_bytes(k, n, BITS, GROUP, 1), 1 << 22), dtype=torch.uint8, device=dev)
+            rows = []
+            for eng in ("lut", "mfma"):
+                _lib.set_gemv_engine(eng)
+                for ks in (0, 1, 2, 4, 8, 16):
+                    for wv in (0, 4, 8, 16):
+                        slices = lib.elutq_hlq_gemv_slices(k, n, BITS, GROUP, ks, wv)
+                        if slices == 0:
+                            continue
+
+                        def launch(stream, ks=ks, wv=wv):
+                            for m in ring:
+                                rc = lib.elutq_hlq_gemv_f16_tuned(m.planes.data_ptr(), m.scales.data_ptr(), m.zeros.data_ptr(), None,
+                                                                  x.data_ptr(), y.data_ptr(), k, n, BITS, GROUP, ws.data_ptr(),
+                                                                  ws.numel(), stream, ks, wv)
+                                if rc:
+                                    raise RuntimeError(f"elutq_hlq_gemv_f16_tuned: {rc}")
+
+                        us = time_graph(torch, launch, 10, 2) / len(ring) * 1e6
+                        rows.append({"engine": eng, "ksplit": ks, "waves": wv, "slices": slices,
+                                     "workgroups": slices * ((n + 63) // 64), "us": round(us, 3)})
+            _lib.set_gemv_engine("auto")
+            table[f"{k}x{n}"] = {"bytes": nbytes, "byte_floor_us_at_8TBps": nbytes / 8e6, "rows": rows}
+            del ring
+            torch.cuda.empty_cache()
+        print(json.dumps({"mode": "shape-sweep", "shapes": table}))
+        return
+    if a.mode == "gemm":
+        print(json.dumps({"mode": "gemm", "gemm_w2g128_llama2_13b": gemm_leg(torch, lib, dev, a.steps)}))
+        return
+    if a.mode == "group":
+        # the whole sweep as one grouped launch, `steps` times (for rocprofv3 --kernel-trace)
+        from elutq_amd.hlq_linear import GemvGroup
+        mods, nbytes = [], 0
+        for i in range(N_LAYERS):
+            for (k, n) in LLAMA3_8B_SHAPES.values():
+                mods.append(make_device_layer(k, n, BITS, GROUP, seed=len(mods), device=dev))
+                nbytes += algorithmic_bytes(k, n, BITS, GROUP)
+        xk = {k: torch.randn(1, k, device=dev).to(torch.float16) for k in {m.in_features for m in mods}}
+        grp = GemvGroup(mods, [xk[m.in_features] for m in mods],
+                        [torch.empty(1, m.out_features, dtype=torch.float16, device=dev) for m in mods])
+        sec = time_graph(torch, lambda s: grp.run(), a.steps, a.warmup)
+        print(json.dumps({"mode": "group", "gemvs_per_launch": len(mods), "bytes_per_launch": nbytes, "us_per_launch": sec * 1e6,
+                          "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}))
+        grp.close()
+        return
+    if a.mode == "sparse":
+        print(json.dumps({"mode": "sparse", "sparse_gemv_w2g128": sparse_leg(torch, lib, dev, a.steps, a.warmup)}))
+        return
+    if a.mode != "full":
+        counter_mode(a, torch, lib, dev)
+        return
+    ws_bytes = max(lib.elutq_hlq_workspace_bytes(k, n, BITS, GROUP, 1) for (k, n) in LLAMA3_8B_SHAPES.values())
+    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+    xs = {k: torch.randn(1, k, device=dev).to(torch.float16) for k in {k for k, _ in LLAMA3_8B_SHAPES.values()}}
+    ys = {n: torch.empty(1, n, dtype=torch.float16, device=dev) for n in {n for _, n in LLAMA3_8B_SHAPES.values()}}
+
+    # ---- the sweep: 32 layers x 7 projections, all weight sets distinct -----------------
+    calls = []
+    step_bytes = 0
+    seed = 0
+    for layer in range(N_LAYERS):
+        for name, (k, n) in LLAMA3_8B_SHAPES.items():
+            mod = make_device_layer(k, n, BITS, GROUP, seed=seed, device=dev)
+            seed += 1
+            calls.append(Gemv(lib, mod, xs[k], ys[n], ws))
+            step_bytes += algorithmic_bytes(k, n, BITS, GROUP)
+    torch.cuda.synchronize()
+
+    def launch_step(stream):
+        for c in calls:
+            c(stream)
+
+    sec_step = time_graph(torch, launch_step, a.steps, a.warmup)
+    value = step_bytes / sec_step / 1e9
+
+    grouped = {}
+    if not a.sweep_only:
+        grouped = side_legs(a, torch, lib, dev, calls, xs, ws_bytes, step_bytes)
+
     # ---- per shape, each over a ring of weight sets > 512 MB ------------------------------
     per_shape = {}
     by_shape = {}
@@ -404,7 +501,7 @@ def main():
 
     # ---- the same four shapes at w3g128 and w2g64 (plane count and group size in the fold) ---
     other_formats = {}
-    for bits, group in ((3, 128), (2, 64)):
+    for bits, group in (() if a.sweep_only else ((3, 128), (2, 64))):
         res = {}
         for (k, n) in sorted(set(LLAMA3_8B_SHAPES.values())):
             nbytes = algorithmic_bytes(k, n, bits, group)
@@ -425,22 +522,24 @@ def main():
             torch.cuda.empty_cache()
         other_formats[f"w{bits}g{group}"] = res
 
-    # ---- one GEMV large enough that the launch and its start-up no longer matter: an lm_head-sized
-    # layer (vocabulary 128256) at w2g128, over a ring of distinct weight sets
-    k, n = 4096, 128256
-    nbytes = algorithmic_bytes(k, n, BITS, GROUP)
-    ring = [Gemv(lib, make_device_layer(k, n, BITS, GROUP, seed=30_000 + i, device=dev), xs[k],
-                 torch.empty(1, n, dtype=torch.float16, device=dev), ws) for i in range(4)]
+    large_shape = {}
+    if not a.sweep_only:
+        # ---- one GEMV large enough that the launch and its start-up no longer matter: an lm_head-sized
+        # layer (vocabulary 128256) at w2g128, over a ring of distinct weight sets
+        k, n = 4096, 128256
+        nbytes = algorithmic_bytes(k, n, BITS, GROUP)
+        ring = [Gemv(lib, make_device_layer(k, n, BITS, GROUP, seed=30_000 + i, device=dev), xs[k],
+                     torch.empty(1, n, dtype=torch.float16, device=dev), ws) for i in range(4)]
 
-    def launch_big(stream, ring=ring):
-        for c in ring:
-            c(stream)
+        def launch_big(stream, ring=ring):
+            for c in ring:
+                c(stream)
 
-    sec = time_graph(torch, launch_big, max(3, min(a.steps, 10)), 2) / len(ring)
-    large_shape = {f"{k}x{n}": {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
-                                "bytes": nbytes, "ring_sets": len(ring)}}
-    del ring
-    torch.cuda.empty_cache()
+        sec = time_graph(torch, launch_big, max(3, min(a.steps, 10)), 2) / len(ring)
+        large_shape = {f"{k}x{n}": {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                                    "bytes": nbytes, "ring_sets": len(ring)}}
+        del ring
+        torch.cuda.empty_cache()
 
     dom = per_shape["4096x14336"]
     roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -449,8 +548,18 @@ def main():
                 # `bench.py --mode kernel`, each scaled by what the same counter reads for `--mode copy`
                 # (summary under profiles/); a property of the kernel's access pattern, not of this run.
                 "traffic": 17_644_000,
+                "traffic_source": "constant from profiles/hlq_gemv_w2g128_4096x14336_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE and "
+                                  "WRITE_SIZE of `bench.py --mode kernel`, scaled by the same counters of `--mode copy`), not measured in this run",
                 "kernel": "hlq_gemv_kernel<2,false> K=4096 N=14336", "us_per_launch": dom["us"],
-                "bytes_per_launch": dom["bytes"]}
+                "bytes_per_launch": dom["bytes"],
+                # the same kernel's average start-to-end duration in the rocprofv3 kernel trace of `bench.py --sweep-only`
+                # (profiles/hlq_gemv_w2g128_sweep_kernel_trace.md) and the fraction that follows from it: a replayed launch
+                # starts while its predecessor's completion is still being signalled, so the live per-launch period above
+                # is shorter than the traced duration
+                "kernel_trace_avg_us": KERNEL_TRACE_AVG_US,
+                "frac_kernel_trace": dom["bytes"] / (KERNEL_TRACE_AVG_US * 1e-6) / 1e9 / HBM_PEAK_GBPS}
+    if grouped.get("device_copy_1GiB_GBps"):
+        roofline["frac_of_device_copy_rate"] = dom["GBps"] / grouped["device_copy_1GiB_GBps"]
 
     out = {
         "metric": "LUT-GEMV HBM GB/s at LLaMA3-8B shapes bs1 (HLQ w2g128)",
@@ -495,11 +604,16 @@ def main():
 
     if not a.no_cpu:
         res, ncpu = cpu_baseline(a.cpu_seconds)
+        faithful = res.pop("fp16_faithful_4096x4096")
         tmax = max(res)
         out["cpu_baseline"] = {"value": res[tmax]["GBps"], "unit": "GB/s", "cores": tmax, "kind": "port",
                                "sample": f"one layer (7 GEMVs, {res[tmax]['reps']} repeats) of the same sweep, AVX2 port of the reference kernel with fp32 accumulators, {tmax} OpenMP threads of {ncpu} host CPUs",
                                "ms_per_layer": res[tmax]["ms_per_layer"],
-                               "at_4_threads_GBps": res[4]["GBps"] if 4 in res else None}
+                               "at_4_threads_GBps": res[4]["GBps"] if 4 in res else None,
+                               "cpu_model": cpu_model(), "host_cpus": ncpu,
+                               "fp16": "fp16 storage, F16C conversions, fp32 accumulate (the port); the reference's NEON kernel "
+                                       "accumulates in fp16, restated op for op below",
+                               "fp16_faithful_scalar_4096x4096": faithful}
     print(json.dumps(out))
 
 
