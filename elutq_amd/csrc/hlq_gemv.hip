@@ -137,7 +137,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     // ... the tables are built as soon as the activations are in (a wave that first queued all
     // its weight loads would sit in the memory pipeline's back-pressure instead) ...
     if (lane < nchunks)
-        build_chunk(prologue, raw, raw2, rstd, lut + (size_t)lane * TBL_BYTES, xs_inv + (lane >> 4), (lane & 15) == 0);
+        build_chunk(prologue, raw, raw2, rstd, lut + (size_t)lane * TBL_BYTES, xs_inv + (lane >> 4), (lane & 15) == 0, lane);
     asm volatile("" ::: "memory");
 
     // ... and the rest of the run's loads follow.
@@ -148,7 +148,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     for (int ci = lane + 64; ci < nchunks; ci += 64) {      // runs of more than two units (not the common case)
         load_chunk<PLAIN>(a, prologue, K, k0 + (size_t)ci * 4, raw, raw2);
         if (sliced) raw = stage[(k0 >> 2) + ci];
-        build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0);
+        build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0, lane);
     }
     HLQ_STAMP(1);
     // The tables were written by this wave and are read by this wave: LDS executes a wave's

@@ -271,7 +271,7 @@ __device__ __forceinline__ void load_chunk(const GemvArgs &a, int prologue, int 
 // The 16 lanes of a DPP row cover one 64-k half unit, whose max|x| sets the power-of-two
 // table scale and whose sum feeds the zero-point fold (row leader stores both in *half).
 __device__ __forceinline__ void build_chunk(int prologue, uint2 raw, uint2 raw2, float rstd, unsigned char *tbl,
-                                            float2 *half, bool leader)
+                                            float2 *half, bool leader, int rot_lane)
 {
     float v[4];
     chunk_values(prologue, raw, raw2, rstd, v);
@@ -287,12 +287,19 @@ __device__ __forceinline__ void build_chunk(int prologue, uint2 raw, uint2 raw2,
     const float inv = eb ? __uint_as_float((eb - 22u) << 23) : 1.0f;
     const int i0 = __float2int_rn(x0 * scale), i1 = __float2int_rn(x1 * scale);
     const int i2 = __float2int_rn(x2 * scale), i3 = __float2int_rn(x3 * scale);
-    const int e3 = i0 + i1, e5 = i0 + i2, e6 = i1 + i2, e7 = e3 + i2;
+    // Entry e = b0 + 2 b1 + 4 b2 + 8 b3 holds b0 i0 + b1 i1 + b2 i2 + b3 i3; quarter qq = (b2, b3) of the table is one
+    // 16-byte store.  A table is 64 bytes at a 64-byte lane stride, so lanes two apart would hit the same banks with
+    // the same quarter: every lane therefore starts with quarter (lane / 2) % 4 and goes round from there, and the
+    // stores of any eight neighbouring lanes fall into 32 different banks.
+    const int e3 = i0 + i1;
     int4 *dst = (int4 *)tbl;
-    dst[0] = make_int4(0, i0, i1, e3);
-    dst[1] = make_int4(i2, e5, e6, e7);
-    dst[2] = make_int4(i3, i3 + i0, i3 + i1, i3 + e3);
-    dst[3] = make_int4(i3 + i2, i3 + e5, i3 + e6, i3 + e7);
+    const int rot = (rot_lane >> 1) & 3;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int qq = (q + rot) & 3;
+        const int base = ((qq & 1) ? i2 : 0) + ((qq & 2) ? i3 : 0);
+        dst[qq] = make_int4(base, base + i0, base + i1, base + e3);
+    }
     if (leader) *half = make_float2(s, inv);
 }
 
