@@ -2,18 +2,22 @@
 // launch, replacing MultiThread_arm_gemm_w_lowbit_activation_fp_impl
 // (C++/ops/src/arm/arm_gemm.cpp:362-387), which re-runs the GEMV once per row.
 //
-// With M rows the contraction is dense enough for the matrix cores, bit-serially.  With
-// c[n,g] = z[n,g] + sum_b s[b,n,g]/2 (the centre of the group's value range),
+// With M rows the contraction is dense enough for the matrix cores, bit-serially:
 //
-//   y[m][n] = sum_g ( c[n,g] * (sum_{k in g} x[m][k])  +  sum_b sum_{k in g} x[m][k] * (+-s[b,n,g]/2) )
+//   y[m][n] = sum_g ( z[n,g] * (sum_{k in g} x[m][k])  +  sum_b s[b,n,g] * (sum_{k in g} x[m][k] * B_b[n][k]) )
 //
-// where the sign is + for a set plane bit.  The B operand of v_mfma_f32_32x32x16_f16 is
-// built in registers from the packed planes: one shift (a rotation where the bits wrap) moves two
-// plane bits (k and k + 16 of a 32-k dword) onto the sign bits of a packed fp16 pair, one v_bfi merges them
-// with |s|/2 -- so every B element is exactly +-s/2, every product exact in fp32, and the
-// fp32 accumulator of the MFMA sums planes and groups alike; nothing is rounded before the
-// final fp16 store.  The centre term uses per-row sums of x over 64-k halves, taken while
-// the activations are staged in LDS (in the element order the B operand uses) as A operand.
+// The inner sum over one group and one plane is a chain of v_mfma_f32_32x32x16_f16 whose B operand is the
+// plane itself as fp16 zeros and ones.  That operand is not computed: every byte of a plane dword (8 k of
+// one column) indexes a 256-row table in LDS whose row v holds the eight fp16 values of v's bits, so one
+// address instruction and one ds_read_b128 deliver the operand of one MFMA.  Every product is x or 0, the
+// chain accumulates in fp32 from zero, and its result is scaled once by the fp32 value of the group's
+// fp16 scale -- nothing else is rounded before the final fp16 store.  The zero term uses per-row sums of
+// x over 64-k halves, taken while the activations are staged in LDS as A operand.
+//
+// A workgroup is one column block (64 columns) x one K slice; its waves (eight, or four for more than 32
+// rows) take the units of the slice in turn (wave w: units w, w + 8, ...).  Every wave stages the activations of its own unit in
+// its own LDS region, so the waves never wait for each other until the final sum: while one wave of a SIMD
+// stages, the other one keeps the matrix core busy.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -27,9 +31,13 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
-constexpr int GW = HLQ_GEMM_WAVES;             // waves per workgroup
-constexpr int GEMM_THREADS = GW * 64;
+constexpr int GW = HLQ_GEMM_WAVES;             // waves per workgroup = K parts, launches of up to 32 rows
+constexpr int GW_WIDE = HLQ_GEMM_WAVES_WIDE;   // the same for launches of 33..64 rows
 constexpr int WS_COUNTER_BYTES = HLQ_WS_COUNTER_BYTES;
+#ifndef HLQ_GEMM_LA
+#define HLQ_GEMM_LA 2                          // MFMA steps between an operand read and its use
+#endif
+constexpr int ROW_BYTES = HLQ_UNIT * 2 + 16;   // one staged row of a unit, padded: conflict-free b128 reads
 
 struct GemmArgs {
     const uint4 *planes;
@@ -39,10 +47,11 @@ struct GemmArgs {
     const uint16_t *x;      // fp16 [M][K]
     uint16_t *y;            // fp16 [M][N]
     const float *extra;     // fp32 [M][N] added to the output before it is rounded, or null
-    float *partial;         // [ksplit][MR][ncb*64]
-    unsigned *counters;     // one per workgroup column (super block)
+    float *partial;         // [ksplit][mpad][ncb*64]
+    unsigned *counters;     // one per column block
     int M, N, K, U, NT, ncb;
-    int ksplit, ups;        // K slices per super block, units per slice (multiple of KW)
+    int ksplit, ups;        // K slices per column block, units per slice
+    int mpad;               // rows of `partial`: 32 or 64
 };
 
 #ifdef HLQ_TIMING
@@ -65,62 +74,49 @@ __device__ __forceinline__ float dpp_f(float v)
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
 
-// Staging of x[:, u0*128 .. (u0+KW)*128) into LDS.  Inside every 32-k block the fp16 values
-// are stored in operand order: position 8s + 2q + r holds k = 4s + q + 16r, so the 16 bytes
-// at 8s are the A operand of MFMA step s and pair q = (k, k + 16) lines up with what one
-// shift extracts from a plane dword.  One task = one such 16-byte slot of one row, built
-// from two 8-byte loads (k = 4s..4s+3 and k + 16); consecutive lanes write consecutive
-// slots, so the LDS stores are conflict-free.  xs[(ul*2 + half) * MR + m] receives the
-// fp32 sum of x[m] over 64-k half `half` of unit ul (eight consecutive lanes).  MR = rows staged
-// (16, 32 or 64).
-template <int MR, int KW>
+// Staging of x[0 .. MR, u*128 .. (u+1)*128) by one wave into its LDS region, rows in their natural k
+// order: the 16 bytes at k = 8t are the A operand of the MFMA step whose B operand comes from plane byte
+// t.  One task = one 16-byte slot of one row (16 slots per row); consecutive lanes write consecutive
+// slots, so the LDS stores are conflict-free.  xs[half * MR + m] receives the fp32 sum of x[m] over 64-k
+// half `half` of the unit (eight consecutive lanes).  MR = rows staged (16, 32 or 64).
+template <int MR>
 struct StageRegs {
-    static constexpr int SLOTS = KW * 16;                            // 16-byte slots per row
-    static constexpr int TASKS = MR * SLOTS;
-    static constexpr int TPT = TASKS / GEMM_THREADS;
-    static_assert(TASKS % GEMM_THREADS == 0, "whole waves of staging tasks");
-    uint2 lo[TPT], hi[TPT];
+    static constexpr int TPT = MR * 16 / 64;                         // tasks per lane
+    uint4 v[TPT];
 };
 
-template <int MR, int KW>
-__device__ __forceinline__ void stage_load(StageRegs<MR, KW> &r, const GemmArgs &a, int u0, int u_end, int tid)
+template <int MR>
+__device__ __forceinline__ void stage_load(StageRegs<MR> &r, const GemmArgs &a, int u, int lane)
 {
-    constexpr int SLOTS = StageRegs<MR, KW>::SLOTS;
+    // The lane number passes through an empty statement so that the row offsets below are recomputed for
+    // every unit (two instructions per task) instead of being kept in registers for the whole kernel.
+    asm volatile("" : "+v"(lane));
+    const uint32_t col_off = ((uint32_t)u * HLQ_UNIT + (lane & 15) * 8) * 2;
 #pragma unroll
-    for (int t = 0; t < StageRegs<MR, KW>::TPT; t++) {
-        const int idx = tid + t * GEMM_THREADS;
-        const int m = idx / SLOTS, o = idx % SLOTS, ul = o >> 4, blk = (o >> 2) & 3, sq = o & 3;
-        const int mm = m < a.M ? m : a.M - 1, uu = u0 + ul < u_end ? u0 + ul : u_end - 1;
-        const uint16_t *src = a.x + (size_t)mm * a.K + (size_t)uu * HLQ_UNIT + blk * 32 + sq * 4;
-        r.lo[t] = *(const uint2 *)src;
-        r.hi[t] = *(const uint2 *)(src + 16);
+    for (int t = 0; t < StageRegs<MR>::TPT; t++) {
+        const int m = (lane >> 4) + 4 * t;
+        const uint32_t mm = (uint32_t)(m < a.M ? m : a.M - 1);
+        r.v[t] = *(const uint4 *)((const unsigned char *)a.x + (mm * (uint32_t)a.K * 2 + col_off));
     }
 }
 
-template <int MR, int KW>
-__device__ __forceinline__ void stage_store(const StageRegs<MR, KW> &r, _Float16 *xl, float *xs, int tid)
+template <int MR>
+__device__ __forceinline__ void stage_store(const StageRegs<MR> &r, unsigned char *xw, float *xs, int lane)
 {
-    constexpr int SLOTS = StageRegs<MR, KW>::SLOTS;
-    constexpr int ROW_HALFS = KW * HLQ_UNIT + 8;
     const half2v ones = {(_Float16)1.f, (_Float16)1.f};
 #pragma unroll
-    for (int t = 0; t < StageRegs<MR, KW>::TPT; t++) {
-        const int idx = tid + t * GEMM_THREADS;
-        const int m = idx / SLOTS, o = idx % SLOTS;
-        float sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.lo[t].x), ones, 0.f, false);
-        sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.lo[t].y), ones, sum, false);
-        sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.hi[t].x), ones, sum, false);
-        sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.hi[t].y), ones, sum, false);
-        sum += dpp_f<0xB1>(sum);                 // lanes of a quad: the four slots of a 32-k block
+    for (int t = 0; t < StageRegs<MR>::TPT; t++) {
+        const int idx = lane + t * 64;
+        const int m = idx >> 4, o = idx & 15;
+        float sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].x), ones, 0.f, false);
+        sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].y), ones, sum, false);
+        sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].z), ones, sum, false);
+        sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].w), ones, sum, false);
+        sum += dpp_f<0xB1>(sum);                 // the eight slots of a 64-k half: quad, quad pair
         sum += dpp_f<0x4E>(sum);
-        sum += dpp_f<0x141>(sum);                // the other 32-k block of the same 64-k half
+        sum += dpp_f<0x141>(sum);
         if ((o & 7) == 0) xs[(o >> 3) * MR + m] = sum;
-        uint4 v;
-        v.x = __builtin_amdgcn_perm(r.hi[t].x, r.lo[t].x, 0x05040100u);
-        v.y = __builtin_amdgcn_perm(r.hi[t].x, r.lo[t].x, 0x07060302u);
-        v.z = __builtin_amdgcn_perm(r.hi[t].y, r.lo[t].y, 0x05040100u);
-        v.w = __builtin_amdgcn_perm(r.hi[t].y, r.lo[t].y, 0x07060302u);
-        *(uint4 *)(xl + (size_t)m * ROW_HALFS + o * 8) = v;
+        *(uint4 *)(xw + m * ROW_BYTES + o * 16) = r.v[t];
     }
 }
 
@@ -133,13 +129,12 @@ struct UnitData {
 };
 
 template <int BITS, bool G64>
-__device__ __forceinline__ void load_unit(UnitData<BITS> &d, const GemmArgs &a, int cb, int u, int u_end, int lane)
+__device__ __forceinline__ void load_unit(UnitData<BITS> &d, const GemmArgs &a, int cb, int u, int lane)
 {
-    const int uu = u < u_end ? u : u_end - 1;          // past the slice: reload a valid unit nobody uses
-    const size_t meta = (size_t)cb * a.NT + (G64 ? uu : (uu >> 1));
+    const size_t meta = (size_t)cb * a.NT + (G64 ? u : (u >> 1));
 #pragma unroll
     for (int b = 0; b < BITS; b++) {
-        d.w[b] = a.planes[(((size_t)cb * a.U + uu) * BITS + b) * HLQ_CB + lane];
+        d.w[b] = a.planes[(((size_t)cb * a.U + u) * BITS + b) * HLQ_CB + lane];
         d.sc[b] = a.scales[(meta * BITS + b) * HLQ_CB + lane];
     }
     d.zz = a.zeros[meta * HLQ_CB + lane];
@@ -159,29 +154,63 @@ __device__ __forceinline__ float h2f(uint32_t v, bool hi)
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(hi ? v >> 16 : v & 0xffffu));
 }
 
-// MR = activation rows of the launch, rounded up to 16, 32 or 64.  The MFMA tile has 32 rows; with
-// MR = 16 only rows 0..15 are staged (lanes of rows 16..31 read rows 0..15 again) and only the
-// accumulator registers of those rows (0..7 of 16) are reduced and stored.
-template <int BITS, bool G64, int MR, int KW>
-__global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a)
+// Byte offset of the operand-table row for byte S of w.  The table holds TREP = 16 copies of every row
+// side by side (row stride 256 bytes) and a lane reads copy lane % 16 (`lanepart` = 16 * that): the lanes
+// of one ds_read_b128 then fall on different banks whatever their bytes are.  One v_perm_b32 puts byte S
+// into bits 8..15 above the lane part.  A compiler builtin on purpose: the compiler knows which registers
+// a pending MFMA is still going to write and keeps other writes away from them for long enough, which it
+// does not do for instructions inside inline assembly.
+template <int TREP>
+__device__ __forceinline__ uint32_t row_addr(uint32_t w, int S, uint32_t lanepart)
 {
-    constexpr int MT = (MR + 31) / 32;              // 32-row MFMA tiles
-    constexpr int REGS = MR == 16 ? 8 : 16;         // accumulator registers per tile that hold real rows
+    if (TREP == 16) return __builtin_amdgcn_perm(w, lanepart, 0x0c0c0000u | ((4u + S) << 8));
+    return ((w >> (8 * S)) & 0xffu) * (16u * TREP) + lanepart;
+}
+
+// Emits no instruction.  `chain` is the 16-register result of a chain of MFMAs of which only some
+// registers are read, `first_use` a value computed from one of them.  Tying the two together keeps all 16
+// registers allocated to the chain until that value exists, i.e. until the last MFMA has written them;
+// otherwise the registers nobody reads are free from the moment that MFMA is issued and could be handed
+// to another value while the MFMA is still going to write them.
+__device__ __forceinline__ float hold_until_read(float first_use, const float16v &chain)
+{
+    asm volatile("" : "+v"(first_use) : "v"(chain));
+    return first_use;
+}
+
+// LDS of a workgroup: the operand table, then one region per wave (a staged unit of MR rows and its
+// half-unit row sums); the cross-wave reduction reuses the table's space after the last unit.
+template <int MR>
+struct GemmLds {
+    static constexpr int NW = MR <= 32 ? GW : GW_WIDE;               // waves
+    static constexpr int TREP = MR <= 32 ? 16 : 4;                   // copies of the operand table
+    static constexpr int MT = (MR + 31) / 32;                        // 32-row MFMA tiles
+    static constexpr int REGS = MR == 16 ? 8 : 16;
+    static constexpr int TAB_BYTES = 256 * 16 * TREP;
+    static constexpr int WAVE_BYTES = MR * ROW_BYTES + 2 * MR * 4;
+    static constexpr int RED_BYTES = NW * MT * 2 * REGS * 64 * 4;
+    static constexpr int BYTES = TAB_BYTES + NW * WAVE_BYTES;
+    static_assert(RED_BYTES <= BYTES, "the reduction reuses the table and the regions");
+    static_assert(WAVE_BYTES % 16 == 0, "aligned regions");
+};
+
+// MR = activation rows of the launch rounded up to 16, 32 or 64.  The MFMA tile has 32 rows; with
+// MR = 16 only rows 0..15 are staged (lanes of rows 16..31 read rows 0..15 again) and only the
+// accumulator registers of those rows (0..7 of 16) are scaled, reduced and stored.  With MR = 64 every B
+// operand serves two MFMAs (rows 0..31 and 32..63); the workgroup then has four waves, one per SIMD, and
+// each of them the whole register file: four accumulators, four chains and deeper operand rings.
+// grid = column blocks * K slices.
+template <int BITS, bool G64, int MR>
+__global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const GemmArgs a)
+{
+    using L = GemmLds<MR>;
+    constexpr int REGS = L::REGS, MT = L::MT, NW = L::NW, THREADS = NW * 64, TREP = L::TREP;
+    constexpr int VALS = MT * 2 * REGS * 64;        // fp32 results per wave
     extern __shared__ __align__(256) unsigned char smem[];
-    constexpr int CBW = GW / KW;                    // column blocks per workgroup
-    constexpr int ROW_HALFS = KW * HLQ_UNIT + 8;    // 16 B pad: conflict-free b128 reads
-    constexpr int TILES = MT * 2;
-    constexpr int VALS = TILES * REGS * 64;         // fp32 results per wave
-    constexpr int MROWS = MR;
-    constexpr int XBUF = MROWS * ROW_HALFS * 2 + KW * 2 * MROWS * 4;    // bytes of one staged chunk: x, then row sums
-    float *red = (float *)smem;                     // reused after the last step
+    float *red = (float *)smem;                     // reused after the last unit
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, h = lane >> 5;
-    const int ci = wave % CBW, kp = wave / CBW;
-    const int sb = blockIdx.x / a.ksplit, slice = blockIdx.x - sb * a.ksplit;
-    const int cb = sb * CBW + ci;
-    const bool cb_ok = cb < a.ncb;
-    const int cbc = cb_ok ? cb : a.ncb - 1;
+    const int cb = blockIdx.x / a.ksplit, slice = blockIdx.x - cb * a.ksplit;
     const int u_begin = slice * a.ups, u_end = min(u_begin + a.ups, a.U);
 
     float16v acc[MT][2];
@@ -193,177 +222,199 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
             for (int i = 0; i < 16; i++) acc[mt][j][i] = 0.f;
 
     GEMM_STAMP(0);
-    int stamp_i = 1;
-    (void)stamp_i;
-    // Two chunk buffers in LDS alternate: while the waves compute on one, the next chunk (its
-    // global loads were issued a step earlier) is written to the other, and the loads of the
-    // chunk after that are issued.  One barrier per step.
+    // The plane data of two of the wave's units is in registers at any time (two alternating sets, so no
+    // set is ever copied); the activations of the next unit wait in registers while the wave computes on
+    // the staged ones.
     UnitData<BITS> ua, ub;
-    StageRegs<MR, KW> xr;
-    load_unit<BITS, G64>(ua, a, cbc, u_begin + kp, u_end, lane);
-    stage_load<MR, KW>(xr, a, u_begin, u_end, tid);
-    stage_store<MR, KW>(xr, (_Float16 *)smem, (float *)(smem + MROWS * ROW_HALFS * 2), tid);
-    if (u_begin + KW < u_end) {
-        load_unit<BITS, G64>(ub, a, cbc, u_begin + KW + kp, u_end, lane);
-        stage_load<MR, KW>(xr, a, u_begin + KW, u_end, tid);
+    StageRegs<MR> xr;
+    const int u_first = u_begin + wave;
+    if (u_first < u_end) {
+        load_unit<BITS, G64>(ua, a, cb, u_first, lane);
+        stage_load<MR>(xr, a, u_first, lane);
+    }
+    if (u_first + NW < u_end) load_unit<BITS, G64>(ub, a, cb, u_first + NW, lane);
+    // operand table: row v holds the eight fp16 values (0 or 1) of the bits of v, TREP copies side by side
+#pragma unroll
+    for (int e = tid; e < 256 * TREP; e += THREADS) {
+        const int v = e / TREP;
+        uint4 row;
+        row.x = ((v & 1) ? 0x3C00u : 0u) | ((v & 2) ? 0x3C000000u : 0u);
+        row.y = ((v & 4) ? 0x3C00u : 0u) | ((v & 8) ? 0x3C000000u : 0u);
+        row.z = ((v & 16) ? 0x3C00u : 0u) | ((v & 32) ? 0x3C000000u : 0u);
+        row.w = ((v & 64) ? 0x3C00u : 0u) | ((v & 128) ? 0x3C000000u : 0u);
+        *(uint4 *)(smem + e * 16) = row;
     }
     __syncthreads();
+    GEMM_STAMP(1);
+    const uint32_t lanepart = (uint32_t)(lane % TREP) * 16u;
+    unsigned char *xw = smem + L::TAB_BYTES + wave * L::WAVE_BYTES;
+    float *xs = (float *)(xw + MR * ROW_BYTES);
+    const unsigned char *arow = xw + (MR == 16 ? (col & 15) : col) * ROW_BYTES + h * 64;
 
-    // One step: compute on `cur` (the unit of this step), then refill it with the unit two steps
-    // ahead; the caller alternates the two register sets, so no set is ever copied.
-    auto step = [&](UnitData<BITS> &cur, int u0, int par) __attribute__((always_inline)) {
-        GEMM_STAMP(stamp_i); stamp_i++;
-        const _Float16 *xl = (const _Float16 *)(smem + par * XBUF);
-        const float *xs = (const float *)(smem + par * XBUF + MROWS * ROW_HALFS * 2);
-        if (u0 + KW < u_end) {
-            unsigned char *nb = smem + (par ^ 1) * XBUF;
-            stage_store<MR, KW>(xr, (_Float16 *)nb, (float *)(nb + MROWS * ROW_HALFS * 2), tid);
-            if (u0 + 2 * KW < u_end) stage_load<MR, KW>(xr, a, u0 + 2 * KW, u_end, tid);
+    // One unit: stage its activations (LDS operations of one wave execute in order, so the wave reads
+    // what it has just written without a barrier), compute, then refill `cur` with the unit two turns ahead.
+    auto unit = [&](UnitData<BITS> &cur, int u) __attribute__((always_inline)) {
+        stage_store<MR>(xr, xw, xs, lane);
+        if (u + NW < u_end) stage_load<MR>(xr, a, u + NW, lane);
+        // Lane (col, h) of tile j works on column 32j + col of the block: bring that column's
+        // scale / zero dwords and its plane dwords (k half h of each 64-k pair, rotation undone:
+        // bit i of tw[b][j][pr] is k = 64 pr + 32 h + i) into the lane.
+        uint32_t scj[BITS][2], zzj[2], tw[BITS][2][2];
+#pragma unroll
+        for (int b = 0; b < BITS; b++) {
+            split_tiles(cur.sc[b], cur.sc[b], scj[b][0], scj[b][1]);
+            split_tiles(cur.w[b].x, cur.w[b].y, tw[b][0][0], tw[b][1][0]);
+            split_tiles(cur.w[b].z, cur.w[b].w, tw[b][0][1], tw[b][1][1]);
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int pr = 0; pr < 2; pr++) tw[b][j][pr] = __builtin_amdgcn_alignbit(tw[b][j][pr], tw[b][j][pr], HLQ_ROT);
         }
-        GEMM_STAMP(stamp_i); stamp_i++;
-        const int u = u0 + kp;
-        if (cb_ok && u < u_end) {
-            // Lane (col, h) of tile j works on column 32j + col of the block: bring that column's
-            // scale / zero dwords and its plane dwords (k half h of each 64-k pair) into the lane.
-            uint32_t scj[BITS][2], zzj[2], tw[BITS][2][2];
+        split_tiles(cur.zz, cur.zz, zzj[0], zzj[1]);
+        if (u + 2 * NW < u_end) load_unit<BITS, G64>(cur, a, cb, u + 2 * NW, lane);
+        // The unit is a list of MFMA steps: for every group of the unit, for every plane, the NQ 16-k
+        // steps of the group.  Step t uses the A operands of its 16 k (one per row tile) and one B
+        // operand per column tile; they are read from LDS LA steps before their use, into rotating
+        // register sets, so that the reads are not waited for.
+        constexpr int NG = G64 ? 2 : 1, NQ = G64 ? 4 : 8;
+        constexpr int NSTEP = NG * BITS * NQ, LA = 2, RING = LA + 1;
+        half8 aopr[RING][MT], bopr[RING][2];
+        auto issue = [&](int t) __attribute__((always_inline)) {
+            const int g = t / (BITS * NQ), b = (t / NQ) % BITS, q = t % NQ;
+            const int pr = G64 ? g : q / 4, sq = q % 4;
 #pragma unroll
-            for (int b = 0; b < BITS; b++) {
-                split_tiles(cur.sc[b], cur.sc[b], scj[b][0], scj[b][1]);
-                split_tiles(cur.w[b].x, cur.w[b].y, tw[b][0][0], tw[b][1][0]);
-                split_tiles(cur.w[b].z, cur.w[b].w, tw[b][0][1], tw[b][1][1]);
-            }
-            split_tiles(cur.zz, cur.zz, zzj[0], zzj[1]);
-            // A operands are read two MFMA steps ahead of their use (three rotating registers sets);
-            // scheduling barriers between the steps keep the compiler from sinking the reads
-            const _Float16 *arow = xl + (size_t)(MR == 16 ? (col & 15) : col) * ROW_HALFS + kp * HLQ_UNIT + h * 32;
-            half8 aop[3][MT];
+            for (int mt = 0; mt < MT; mt++) aopr[t % RING][mt] = *(const half8 *)(arow + mt * 32 * ROW_BYTES + pr * 128 + sq * 16);
 #pragma unroll
-            for (int st = 0; st < 2; st++)
+            for (int j = 0; j < 2; j++) bopr[t % RING][j] = *(const half8 *)(smem + row_addr<TREP>(tw[b][j][pr], sq, lanepart));
+        };
+        // zero term of group g: z[n, g] * sum_{k in g} x[m, k]; C rows of register i: 8*(i/4) + 4h + i%4
+        auto zero_term = [&](int g, bool hi) __attribute__((always_inline)) {
+            const float zf[2] = {h2f(zzj[0], hi), h2f(zzj[1], hi)};
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++)
-                    aop[st][mt] = *(const half8 *)(arow + (size_t)mt * 32 * ROW_HALFS + (st >> 2) * 64 + (st & 3) * 8);
+            for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int pr = 0; pr < 2; pr++) {          // 64-k pair of dwords: k = 64pr + 32h + ...
-                const bool hi = G64 ? pr == 1 : (u & 1) != 0;       // fp16 of the meta dwords this pair belongs to
-                uint32_t mag[BITS][2], bits[BITS][2];
-                float cen[2];
+                for (int i4 = 0; i4 < REGS / 4; i4++) {
+                    const int mr = mt * 32 + 8 * i4 + 4 * h;
+                    float4 sx = *(const float4 *)(xs + (G64 ? g : 1) * MR + mr);
+                    if (!G64) {
+                        const float4 s0 = *(const float4 *)(xs + mr);
+                        sx.x += s0.x; sx.y += s0.y; sx.z += s0.z; sx.w += s0.w;
+                    }
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        acc[mt][j][4 * i4 + 0] = fmaf(zf[j], sx.x, acc[mt][j][4 * i4 + 0]);
+                        acc[mt][j][4 * i4 + 1] = fmaf(zf[j], sx.y, acc[mt][j][4 * i4 + 1]);
+                        acc[mt][j][4 * i4 + 2] = fmaf(zf[j], sx.z, acc[mt][j][4 * i4 + 2]);
+                        acc[mt][j][4 * i4 + 3] = fmaf(zf[j], sx.w, acc[mt][j][4 * i4 + 3]);
+                    }
+                }
+        };
+#pragma unroll
+        for (int t = 0; t < LA && t < NSTEP; t++) issue(t);
+        if constexpr (MT == 1) {
+            // One row tile: every (group, plane, column tile) is a chain that starts from zero; its result is
+            // scaled by the group's scale and added to the accumulator (16 or 8 multiply-adds per chain).
+            float16v tmp[2];
+#pragma unroll
+            for (int t = 0; t < NSTEP; t++) {
+                const int g = t / (BITS * NQ), b = (t / NQ) % BITS, q = t % NQ;
+                if (t + LA < NSTEP) issue(t + LA);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
-                    cen[j] = h2f(zzj[j], hi);
+                    if (q == 0) {
+                        float16v zero;
 #pragma unroll
-                    for (int b = 0; b < BITS; b++) {
+                        for (int i = 0; i < 16; i++) zero[i] = 0.f;
+                        tmp[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aopr[t % RING][0], bopr[t % RING][j], zero, 0, 0, 0);
+                    } else {
+                        tmp[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aopr[t % RING][0], bopr[t % RING][j], tmp[j], 0, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (q == NQ - 1) {
+                    const bool hi = G64 ? g == 1 : (u & 1) != 0;      // fp16 of the meta dwords this group belongs to
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
                         const float sf = h2f(scj[b][j], hi);
-                        cen[j] = fmaf(0.5f, sf, cen[j]);
-                        const uint32_t m16 = (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)(0.5f * fabsf(sf)));
-                        mag[b][j] = m16 | (m16 << 16);
-                        // the sign of a B element is the plane bit, inverted unless the scale is negative
-                        bits[b][j] = sf < 0.f ? tw[b][j][pr] : ~tw[b][j][pr];
+#pragma unroll
+                        for (int i = 0; i < REGS; i++) acc[0][j][i] = fmaf(sf, tmp[j][i], acc[0][j][i]);
+                        if (REGS < 16) acc[0][j][REGS - 1] = hold_until_read(acc[0][j][REGS - 1], tmp[j]);
                     }
-                }
-#pragma unroll
-                for (int s = 0; s < 4; s++) {
-                    const int st = pr * 4 + s;        // step 0..7 of the unit
-                    if (st < 6) {
-                        const int nx = st + 2;
-#pragma unroll
-                        for (int mt = 0; mt < MT; mt++)
-                            aop[nx % 3][mt] = *(const half8 *)(arow + (size_t)mt * 32 * ROW_HALFS + (nx >> 2) * 64 + (nx & 3) * 8);
-                    }
-                    // planes outermost: consecutive MFMAs then go to different accumulators
-#pragma unroll
-                    for (int b = 0; b < BITS; b++)
-#pragma unroll
-                        for (int j = 0; j < 2; j++) {
-                            uint32_t o[4];
-#pragma unroll
-                            for (int q = 0; q < 4; q++) {
-                                // stored dwords are rotated left by HLQ_ROT: bit k = 4s + q goes to the sign of
-                                // the low fp16, bit k + 16 to the sign of the high one
-                                // (positions k + HLQ_ROT and k + 16 + HLQ_ROT move to 15 and 31).  Without a wrap a plain
-                                // shift does it -- a 32-bit-encoded instruction, which the SIMD retires in 2.4
-                                // cycles where v_alignbit (64-bit encoding) takes 4.25
-                                const int mv = 15 - (4 * s + q + HLQ_ROT);       // left shift that is needed (compile time)
-                                const uint32_t src = bits[b][j];
-                                const uint32_t rot = mv > 0 ? src << mv : (mv == 0 ? src : __builtin_amdgcn_alignbit(src, src, (uint32_t)-mv));
-                                o[q] = (rot & 0x80008000u) | (mag[b][j] & 0x7fff7fffu);
-                            }
-                            const half8 bop = __builtin_bit_cast(half8, make_uint4(o[0], o[1], o[2], o[3]));
-#pragma unroll
-                            for (int mt = 0; mt < MT; mt++)
-                                acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aop[st % 3][mt], bop, acc[mt][j], 0, 0, 0);
-                        }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                // centre term: c[n, g] * sum_{k in g} x[m, k]; C rows of register i: 8*(i/4) + 4h + i%4
-                if (G64 || pr == 1) {
-#pragma unroll
-                    for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-                        for (int i4 = 0; i4 < REGS / 4; i4++) {
-                            const int m0 = mt * 32 + 8 * i4 + 4 * h;
-                            float4 sx = *(const float4 *)(xs + (kp * 2 + pr) * MROWS + m0);
-                            if (!G64) {
-                                const float4 s0 = *(const float4 *)(xs + (kp * 2) * MROWS + m0);
-                                sx.x += s0.x; sx.y += s0.y; sx.z += s0.z; sx.w += s0.w;
-                            }
-#pragma unroll
-                            for (int j = 0; j < 2; j++) {
-                                acc[mt][j][4 * i4 + 0] = fmaf(cen[j], sx.x, acc[mt][j][4 * i4 + 0]);
-                                acc[mt][j][4 * i4 + 1] = fmaf(cen[j], sx.y, acc[mt][j][4 * i4 + 1]);
-                                acc[mt][j][4 * i4 + 2] = fmaf(cen[j], sx.z, acc[mt][j][4 * i4 + 2]);
-                                acc[mt][j][4 * i4 + 3] = fmaf(cen[j], sx.w, acc[mt][j][4 * i4 + 3]);
-                            }
-                        }
+                    if (b == BITS - 1) zero_term(g, hi);
                 }
             }
+        } else {
+            // Two row tiles: a B operand serves two MFMAs, which pays for scaling the operand itself (four
+            // packed fp16 multiplications, exact: the operand is 0 or 1) and accumulating straight into the
+            // result, with neither chain registers nor multiply-adds afterwards.
+#pragma unroll
+            for (int t = 0; t < NSTEP; t++) {
+                const int g = t / (BITS * NQ), b = (t / NQ) % BITS, q = t % NQ;
+                const bool hi = G64 ? g == 1 : (u & 1) != 0;
+                if (t + LA < NSTEP) issue(t + LA);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const uint32_t sc = scj[b][j];
+                    const uint32_t pk = hi ? __builtin_amdgcn_perm(sc, sc, 0x03020302u) : __builtin_amdgcn_perm(sc, sc, 0x01000100u);
+                    const half2v s2 = __builtin_bit_cast(half2v, pk);
+                    half8 bs;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const half2v v = {bopr[t % RING][j][2 * i], bopr[t % RING][j][2 * i + 1]};
+                        const half2v p = v * s2;
+                        bs[2 * i] = p[0];
+                        bs[2 * i + 1] = p[1];
+                    }
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++)
+                        acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aopr[t % RING][mt], bs, acc[mt][j], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (q == NQ - 1 && b == BITS - 1) zero_term(g, hi);
+            }
         }
-        GEMM_STAMP(stamp_i); stamp_i++;
-        if (u0 + 2 * KW < u_end) load_unit<BITS, G64>(cur, a, cbc, u0 + 2 * KW + kp, u_end, lane);
-        __syncthreads();
     };
-    for (int u0 = u_begin; u0 < u_end; u0 += 2 * KW) {
-        step(ua, u0, 0);
-        if (u0 + KW < u_end) step(ub, u0 + KW, 1);
+    for (int u = u_first; u < u_end; u += 2 * NW) {
+        unit(ua, u);
+        if (u + NW < u_end) unit(ub, u + NW);
     }
 
     GEMM_STAMP(13);
-    // Sum of the KW parts of every column block through LDS: red[wave][tile = mt*2+j][reg][lane].
+    // Sum of the K parts through LDS: red[wave][tile = mt*2+j][reg][lane].
     __syncthreads();
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int i = 0; i < REGS; i++) red[((wave * TILES + mt * 2 + j) * REGS + i) * 64 + lane] = acc[mt][j][i];
+            for (int i = 0; i < REGS; i++) red[((wave * MT * 2 + mt * 2 + j) * REGS + i) * 64 + lane] = acc[mt][j][i];
     __syncthreads();
 
-    constexpr int NV = CBW * VALS / GEMM_THREADS;    // results per thread
+    constexpr int NV = VALS / THREADS;               // results per thread
     const size_t npad = (size_t)a.ncb * HLQ_CB;
-    const int mpad = MROWS;
-    // value v = (column block, tile, reg, lane); C layout of the 32x32 MFMA: column = lane % 32,
+    // value v = (tile, reg, lane); C layout of the 32x32 MFMA: column = lane % 32,
     // row = 8 * (reg / 4) + 4 * (lane / 32) + reg % 4.
     auto decode = [&](int v, int &m, int &n) {
-        const int c = v / VALS, r = v % VALS;
-        const int ln = r & 63, reg = (r >> 6) % REGS, tile = r / (64 * REGS);
-        const int mt = tile >> 1, j = tile & 1;
-        m = mt * 32 + 8 * (reg >> 2) + 4 * (ln >> 5) + (reg & 3);
-        n = (sb * CBW + c) * HLQ_CB + j * 32 + (ln & 31);
+        const int ln = v & 63, reg = (v >> 6) % REGS, tile = v / (64 * REGS);
+        m = (tile >> 1) * 32 + 8 * (reg >> 2) + 4 * (ln >> 5) + (reg & 3);
+        n = cb * HLQ_CB + (tile & 1) * 32 + (ln & 31);
     };
     float outv[NV];
 #pragma unroll
     for (int it = 0; it < NV; it++) {
-        const int v = tid + it * GEMM_THREADS;
-        const int c = v / VALS, r = v % VALS;
+        const int v = tid + it * THREADS;
         float s = 0.f;
 #pragma unroll
-        for (int p = 0; p < KW; p++) s += red[(p * CBW + c) * VALS + r];
+        for (int p = 0; p < NW; p++) s += red[p * VALS + v];
         outv[it] = s;
     }
     if (a.ksplit == 1) {
 #pragma unroll
         for (int it = 0; it < NV; it++) {
             int m, n;
-            decode(tid + it * GEMM_THREADS, m, n);
+            decode(tid + it * THREADS, m, n);
             if (m < a.M && n < a.N) {
                 float s = outv[it];
                 if (a.bias) s += (float)__builtin_bit_cast(_Float16, a.bias[n]);
@@ -371,6 +422,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
                 a.y[(size_t)m * a.N + n] = __builtin_bit_cast(uint16_t, (_Float16)s);
             }
         }
+        GEMM_STAMP(15);
         return;
     }
     // Slices meet through device memory, as in the GEMV: agent-scope stores, wait for their
@@ -378,27 +430,27 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
 #pragma unroll
     for (int it = 0; it < NV; it++) {
         int m, n;
-        decode(tid + it * GEMM_THREADS, m, n);
-        if ((size_t)n < npad)
-            __hip_atomic_store(&a.partial[((size_t)slice * mpad + m) * npad + n], outv[it], __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
+        decode(tid + it * THREADS, m, n);
+        __hip_atomic_store(&a.partial[((size_t)slice * a.mpad + m) * npad + n], outv[it], __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     GEMM_STAMP(14);
     __syncthreads();
     __shared__ unsigned s_ticket;
-    if (tid == 0) s_ticket = __hip_atomic_fetch_add(&a.counters[sb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned *counter = a.counters + cb;
+    if (tid == 0) s_ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != (unsigned)a.ksplit - 1u) return;
     // a thread's loads for QB slices are in flight together; summed in slice order
-    constexpr int QB = NV <= 8 ? 4 : (NV <= 16 ? 2 : 1);
+    constexpr int QB = NV <= 8 ? 4 : 2;
     float sum[NV];
     size_t off[NV];
 #pragma unroll
     for (int it = 0; it < NV; it++) {
         int m, n;
-        decode(tid + it * GEMM_THREADS, m, n);
-        off[it] = (size_t)n < npad ? (size_t)m * npad + n : 0;
+        decode(tid + it * THREADS, m, n);
+        off[it] = (size_t)m * npad + n;
         sum[it] = 0.f;
     }
     for (int s0 = 0; s0 < a.ksplit; s0 += QB) {
@@ -408,7 +460,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
             const int sl = min(s0 + q, a.ksplit - 1);
 #pragma unroll
             for (int it = 0; it < NV; it++)
-                v[q][it] = __hip_atomic_load(&a.partial[(size_t)sl * mpad * npad + off[it]], __ATOMIC_RELAXED,
+                v[q][it] = __hip_atomic_load(&a.partial[(size_t)sl * a.mpad * npad + off[it]], __ATOMIC_RELAXED,
                                              __HIP_MEMORY_SCOPE_AGENT);
         }
 #pragma unroll
@@ -421,7 +473,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
 #pragma unroll
     for (int it = 0; it < NV; it++) {
         int m, n;
-        decode(tid + it * GEMM_THREADS, m, n);
+        decode(tid + it * THREADS, m, n);
         if (m < a.M && n < a.N) {
             float s = sum[it];
             if (a.bias) s += (float)__builtin_bit_cast(_Float16, a.bias[n]);
@@ -429,7 +481,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void hlq_gemm_kernel(const GemmArgs a
             a.y[(size_t)m * a.N + n] = __builtin_bit_cast(uint16_t, (_Float16)s);
         }
     }
-    if (tid == 0) __hip_atomic_store(&a.counters[sb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     GEMM_STAMP(15);
 }
 
@@ -447,51 +499,32 @@ inline bool allow_big_lds(const void *kern, size_t lds, int limit, bool (&done)[
     return true;
 }
 
-template <int MR, int KW>
-size_t gemm_lds_bytes()
-{
-    constexpr int MT = (MR + 31) / 32, REGS = MR == 16 ? 8 : 16;
-    const size_t x = 2 * ((size_t)MR * (KW * HLQ_UNIT + 8) * 2 + (size_t)KW * 2 * MR * sizeof(float));
-    const size_t r = (size_t)GW * MT * 2 * REGS * 64 * 4;
-    return (x > r ? x : r) + 256;
-}
-
-template <int BITS, bool G64, int MR, int KW>
+template <int BITS, bool G64, int MR>
 int launch_gemm(const GemmArgs &a, hipStream_t stream)
 {
-    auto kern = hlq_gemm_kernel<BITS, G64, MR, KW>;
-    const size_t lds = gemm_lds_bytes<MR, KW>();
+    auto kern = hlq_gemm_kernel<BITS, G64, MR>;
+    const size_t lds = GemmLds<MR>::BYTES;
+    static_assert(GemmLds<MR>::BYTES + 64 <= HLQ_MAX_LDS, "LDS of one workgroup");
     static bool big_lds_done[64] = {};        // per template instance
     if (!allow_big_lds((const void *)kern, lds, (int)lds, big_lds_done)) return ELUTQ_ERR_HIP;
-    const int cbw = GW / KW, nsb = (a.ncb + cbw - 1) / cbw;
-    hipLaunchKernelGGL(kern, dim3(nsb * a.ksplit), dim3(GEMM_THREADS), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3(a.ncb * a.ksplit), dim3(GemmLds<MR>::NW * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
 
-template <int BITS, bool G64, int MR>
-int launch_gemm_kw(const GemmArgs &a, int kw, hipStream_t stream)
-{
-    switch (kw) {
-    case 2: return launch_gemm<BITS, G64, MR, 2>(a, stream);
-    case 4: return launch_gemm<BITS, G64, MR, 4>(a, stream);
-    }
-    return ELUTQ_ERR_TUNING;
-}
-
 template <int BITS, bool G64>
-int launch_gemm_mt(const GemmArgs &a, int kw, hipStream_t stream)
+int launch_gemm_rows(const GemmArgs &a, hipStream_t stream)
 {
-    if (a.M <= 16) return launch_gemm_kw<BITS, G64, 16>(a, kw, stream);
-    return a.M <= 32 ? launch_gemm_kw<BITS, G64, 32>(a, kw, stream) : launch_gemm_kw<BITS, G64, 64>(a, kw, stream);
+    if (a.M <= 16) return launch_gemm<BITS, G64, 16>(a, stream);
+    return a.M <= 32 ? launch_gemm<BITS, G64, 32>(a, stream) : launch_gemm<BITS, G64, 64>(a, stream);
 }
 
-int dispatch_gemm(const GemmArgs &a, int bits, bool g64, int kw, hipStream_t stream)
+int dispatch_gemm(const GemmArgs &a, int bits, bool g64, hipStream_t stream)
 {
     switch (bits) {
-    case 1: return g64 ? launch_gemm_mt<1, true>(a, kw, stream) : launch_gemm_mt<1, false>(a, kw, stream);
-    case 2: return g64 ? launch_gemm_mt<2, true>(a, kw, stream) : launch_gemm_mt<2, false>(a, kw, stream);
-    case 3: return g64 ? launch_gemm_mt<3, true>(a, kw, stream) : launch_gemm_mt<3, false>(a, kw, stream);
-    case 4: return g64 ? launch_gemm_mt<4, true>(a, kw, stream) : launch_gemm_mt<4, false>(a, kw, stream);
+    case 1: return g64 ? launch_gemm_rows<1, true>(a, stream) : launch_gemm_rows<1, false>(a, stream);
+    case 2: return g64 ? launch_gemm_rows<2, true>(a, stream) : launch_gemm_rows<2, false>(a, stream);
+    case 3: return g64 ? launch_gemm_rows<3, true>(a, stream) : launch_gemm_rows<3, false>(a, stream);
+    case 4: return g64 ? launch_gemm_rows<4, true>(a, stream) : launch_gemm_rows<4, false>(a, stream);
     }
     return ELUTQ_ERR_BITS;
 }
@@ -540,11 +573,11 @@ int hlq_gemm_chunk_with_extra(const void *d_planes, const void *d_scales, const 
     if (group != 64 && group != 128) return ELUTQ_ERR_GROUP;
     if (K < HLQ_UNIT || N < 1 || K % HLQ_UNIT != 0 || K % group != 0) return ELUTQ_ERR_SHAPE;
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
-    if (kparts != 0 && kparts != 2 && kparts != 4) return ELUTQ_ERR_TUNING;
+    if (kparts != 0 && kparts != (M <= 32 ? HLQ_GEMM_WAVES : HLQ_GEMM_WAVES_WIDE)) return ELUTQ_ERR_TUNING;
     if (ksplit < 0 || ksplit > K / HLQ_UNIT) return ELUTQ_ERR_TUNING;
     const HlqGeo g = hlq_geo(K, N, bits, group);
-    int kw = kparts, ks = ksplit, ups;
-    hlq_gemm_shape(g, kw, ks, ups);
+    int ks = ksplit, ups;
+    hlq_gemm_shape(g, M, ks, ups);
 
     GemmArgs a;
     a.planes = (const uint4 *)d_planes;
@@ -557,17 +590,16 @@ int hlq_gemm_chunk_with_extra(const void *d_planes, const void *d_scales, const 
     a.M = M; a.N = N; a.K = K; a.U = g.U; a.NT = g.NT; a.ncb = g.ncb;
     a.ksplit = ks; a.ups = ups;
     a.partial = nullptr; a.counters = nullptr;
+    a.mpad = M <= 32 ? 32 : 64;
     if (ks > 1) {
-        const int mpad = M <= 32 ? 32 : 64;
-        const int cbw = GW / kw, nsb = (g.ncb + cbw - 1) / cbw;
         if (!d_workspace) return ELUTQ_ERR_NULL;
-        if ((size_t)nsb * sizeof(unsigned) > (size_t)WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
-        if (workspace_bytes < (size_t)WS_COUNTER_BYTES + (size_t)ks * mpad * g.ncb * HLQ_CB * sizeof(float))
+        if ((size_t)g.ncb * sizeof(unsigned) > (size_t)WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
+        if (workspace_bytes < (size_t)WS_COUNTER_BYTES + (size_t)ks * a.mpad * g.ncb * HLQ_CB * sizeof(float))
             return ELUTQ_ERR_WORKSPACE;
         a.counters = (unsigned *)d_workspace;
         a.partial = (float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
-    return dispatch_gemm(a, bits, group == 64, kw, (hipStream_t)stream);
+    return dispatch_gemm(a, bits, group == 64, (hipStream_t)stream);
 }
 
 extern "C" {

@@ -614,7 +614,7 @@ size_t elutq_hlq_workspace_bytes(int K, int N, int bits, int group, int M)
     // arrival counters (fixed region, so layers of any shape can share one workspace) +
     // partial sums: GEMV at its finest split (one unit per slice), GEMM at the split it uses
     const size_t gemv = (size_t)WS_COUNTER_BYTES + (size_t)g.U * g.ncb * HLQ_CB * sizeof(float);
-    const size_t gemm = M > 1 ? hlq_gemm_ws_bytes(g, M > 64 ? 64 : M) : 0;
+    const size_t gemm = M > 1 ? hlq_gemm_ws_bytes(g, M) : 0;
     return gemv > gemm ? gemv : gemm;
 }
 

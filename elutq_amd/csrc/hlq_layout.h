@@ -28,7 +28,8 @@
 #define HLQ_NUM_CU 256                 /* MI355X */
 #define HLQ_MAX_LDS (160 * 1024)       /* per workgroup on gfx950 */
 #define HLQ_WS_COUNTER_BYTES (64 * 1024) /* head of every workspace: one arrival counter per column block */
-#define HLQ_GEMM_WAVES 8               /* waves per GEMM workgroup */
+#define HLQ_GEMM_WAVES 8               /* waves per GEMM workgroup, up to 32 rows */
+#define HLQ_GEMM_WAVES_WIDE 8          /* the same for 33..64 rows */
 #define HLQ_GEMM_MAX_M 64              /* rows per GEMM launch; more rows run in chunks of this many (weights re-streamed) */
 
 struct HlqGeo {
@@ -56,27 +57,48 @@ static inline size_t hlq_planes_bytes(const HlqGeo &g) { return (size_t)g.ncb * 
 static inline size_t hlq_scales_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * g.bits * HLQ_CB * 4; }
 static inline size_t hlq_zeros_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * HLQ_CB * 4; }
 
-// Launch shape of the small-batch GEMM.  A workgroup has HLQ_GEMM_WAVES waves arranged as
-// (HLQ_GEMM_WAVES / kw) column blocks x kw K parts; a step consumes kw units (one per K part).
-// K is further cut into ksplit slices of ups units (whole steps) handled by different
-// workgroups, about one workgroup per CU in total.
-static inline void hlq_gemm_shape(const HlqGeo &g, int &kw, int &ksplit, int &ups)
+// Launch shape of the small-batch GEMM.  A workgroup is one column block x one K slice; its waves
+// (HLQ_GEMM_WAVES, or HLQ_GEMM_WAVES_WIDE above 32 rows) take the units of the slice in turn.  K is cut
+// into ksplit slices of ups units handled by different workgroups that meet through device memory.  That
+// meeting costs about as much as two units per wave, so K is cut only where the units saved outweigh it,
+// and never into more workgroups than the chip has CUs.
+static inline void hlq_gemm_shape(const HlqGeo &g, int M, int &ksplit, int &ups)
 {
-    if (kw != 2 && kw != 4) kw = 4;
-    const int cbw = HLQ_GEMM_WAVES / kw;
-    const int nsb = (g.ncb + cbw - 1) / cbw;                 // workgroups along N
-    const int steps = (g.U + kw - 1) / kw;                   // steps over all of K
-    int ks = ksplit > 0 ? ksplit : (HLQ_NUM_CU + nsb / 2) / nsb;
-    if (ks > steps) ks = steps;
+    const int waves = M <= 32 ? HLQ_GEMM_WAVES : HLQ_GEMM_WAVES_WIDE;
+    const int turns = (g.U + waves - 1) / waves;        // units per wave over all of K
+    int ks = ksplit;
+    if (ks <= 0) {
+        const int turn_cost = M <= 32 ? 24 : 16, meet_cost = 40;       // tenths of a microsecond
+        int most = HLQ_NUM_CU / g.ncb;
+        if (most > turns) most = turns;
+        ks = 1;
+        int best = turns * turn_cost;
+        for (int k = 2; k <= most; k++) {
+            const int cost = (turns + k - 1) / k * turn_cost + meet_cost;
+            if (cost < best) { best = cost; ks = k; }
+        }
+    }
+    if (ks > g.U) ks = g.U;
     if (ks < 1) ks = 1;
-    ups = (steps + ks - 1) / ks * kw;
+    ups = (g.U + ks - 1) / ks;
     ksplit = (g.U + ups - 1) / ups;
 }
 
-static inline size_t hlq_gemm_ws_bytes(const HlqGeo &g, int M)
+static inline size_t hlq_gemm_ws_rows(const HlqGeo &g, int M)
 {
-    int kw = 0, ks = 0, ups;
-    hlq_gemm_shape(g, kw, ks, ups);
+    int ks = 0, ups;
+    hlq_gemm_shape(g, M, ks, ups);
     const int mpad = M <= 32 ? 32 : 64;
     return (size_t)HLQ_WS_COUNTER_BYTES + (ks > 1 ? (size_t)ks * mpad * g.ncb * HLQ_CB * sizeof(float) : 0);
+}
+
+// Workspace of a GEMM call with M rows: launches take up to HLQ_GEMM_MAX_M rows, the last one the rest.
+static inline size_t hlq_gemm_ws_bytes(const HlqGeo &g, int M)
+{
+    size_t w = hlq_gemm_ws_rows(g, M > HLQ_GEMM_MAX_M ? HLQ_GEMM_MAX_M : M);
+    if (M > HLQ_GEMM_MAX_M) {
+        const size_t r = hlq_gemm_ws_rows(g, 32);
+        if (r > w) w = r;
+    }
+    return w;
 }

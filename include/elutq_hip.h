@@ -238,11 +238,11 @@ int elutq_hlq_gemm_f16(const void *d_planes, const void *d_scales, const void *d
 
 /*
  * Same computation with the launch shape chosen by the caller: `kparts` K parts inside a
- * workgroup (2 or 4; the workgroup then covers 8 / kparts column blocks of 64) and
- * `ksplit` K slices across workgroups (1..K/128); 0 = library default.  The workspace
- * must hold 64 KiB + ksplit * (M <= 32 ? 32 : 64) * ceil(N/64)*64 * 4 bytes when the shape
- * ends up with more than one slice.  For tuning and for tests that must reach every
- * reduction path; results do not depend on these beyond fp32 summation order.
+ * workgroup (8 = its eight waves, or 0 for the default, which is the same; anything else
+ * returns ELUTQ_ERR_TUNING) and `ksplit` K slices across workgroups (1..K/128); 0 = library
+ * default.  The workspace must hold 64 KiB + ksplit * (M <= 32 ? 32 : 64) * ceil(N/64)*64 * 4
+ * bytes when the shape ends up with more than one slice.  For tuning and for tests that must
+ * reach every reduction path; results do not depend on these beyond fp32 summation order.
  */
 int elutq_hlq_gemm_f16_tuned(const void *d_planes, const void *d_scales, const void *d_zeros,
                              const void *d_bias, const void *d_x, void *d_y,

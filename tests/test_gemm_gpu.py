@@ -72,14 +72,14 @@ def test_llama2_13b_prefill_shapes(cuda, m, k, n):
     assert O.rel_err(y, ref) <= TOL
 
 
-@pytest.mark.parametrize("kparts", [2, 4])
+@pytest.mark.parametrize("kparts", [0, 8])
 @pytest.mark.parametrize("ksplit", [1, 2, 3, 0])
 @pytest.mark.parametrize("m,k,n,bits,group", [(16, 1024, 100, 2, 128), (64, 1280, 320, 2, 128), (40, 1152, 576, 3, 64),
                                                (7, 896, 64, 4, 128), (33, 640, 200, 1, 64)])
 def test_gemm_every_launch_shape(cuda, kparts, ksplit, m, k, n, bits, group):
-    """Every arrangement of a workgroup (K parts x column blocks) and of the K slices across
-    workgroups, including column blocks past N, slices of unequal length and steps only some
-    K parts take part in, against the float64 oracle; a second call on the same workspace
+    """Every cut of K into slices across workgroups, including a last column block past N, slices of
+    unequal length, slices shorter than the eight waves of a workgroup and launches of two row tiles,
+    against the float64 oracle; a second call on the same workspace
     must give the same bits (arrival counters are left at zero)."""
     from elutq_amd import _lib
     L = make_layer(k, n, bits=bits, group=group, m=m, seed=k + n + kparts, bias=True)
@@ -112,8 +112,9 @@ def test_gemm_tuned_rejects_bad_shapes(cuda):
     call = lambda kp, ks, wsb: _lib.lib().elutq_hlq_gemm_f16_tuned(
         mod.planes.data_ptr(), mod.scales.data_ptr(), mod.zeros.data_ptr(), None, x.data_ptr(), y.data_ptr(), 4, 512, 64,
         2, 128, ws.data_ptr(), wsb, torch.cuda.current_stream().cuda_stream, kp, ks)
-    assert call(3, 0, ws.numel()) == -7          # K parts must be 2 or 4
-    assert call(4, 5, ws.numel()) == -7          # more slices than units
-    assert call(2, 2, ws.numel()) == -5          # two slices need room for partial sums
-    assert call(4, 1, 0) == 0                    # one slice needs no workspace
+    assert call(3, 0, ws.numel()) == -7          # K parts: 8 (or 0 for the default, which is 8)
+    assert call(4, 0, ws.numel()) == -7
+    assert call(8, 5, ws.numel()) == -7          # more slices than units
+    assert call(8, 2, ws.numel()) == -5          # two slices need room for partial sums
+    assert call(8, 1, 0) == 0                    # one slice needs no workspace
     torch.cuda.synchronize()
