@@ -37,6 +37,9 @@ constexpr int WS_COUNTER_BYTES = HLQ_WS_COUNTER_BYTES;
 #ifndef HLQ_GEMM_LA
 #define HLQ_GEMM_LA 2                          // MFMA steps between an operand read and its use
 #endif
+#ifndef HLQ_GEMM_LA
+#define HLQ_GEMM_LA 2                          // MFMA steps between an operand read and its use
+#endif
 constexpr int ROW_BYTES = HLQ_UNIT * 2 + 16;   // one staged row of a unit, padded: conflict-free b128 reads
 
 struct GemmArgs {
@@ -277,7 +280,7 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
         // operand per column tile; they are read from LDS LA steps before their use, into rotating
         // register sets, so that the reads are not waited for.
         constexpr int NG = G64 ? 2 : 1, NQ = G64 ? 4 : 8;
-        constexpr int NSTEP = NG * BITS * NQ, LA = 2, RING = LA + 1;
+        constexpr int NSTEP = NG * BITS * NQ, LA = HLQ_GEMM_LA, RING = LA + 1;
         half8 aopr[RING][MT], bopr[RING][2];
         auto issue = [&](int t) __attribute__((always_inline)) {
             const int g = t / (BITS * NQ), b = (t / NQ) % BITS, q = t % NQ;
