@@ -5,6 +5,7 @@
 """
 from __future__ import annotations
 
+import ctypes
 import glob
 import os
 import shutil
@@ -63,6 +64,13 @@ def build(verbose: bool = False, force: bool = True, jobs: int = 6) -> str:
         list(pool.map(lambda so: _run([hipcc(), *HIPCC_FLAGS, "-I", include, "-c", "-o", so[1], so[0]], verbose), todo))
     tmp = LIB_PATH + ".tmp"
     _run([hipcc(), "--offload-arch=gfx950", "-fPIC", "-shared", "-o", tmp, *objs], verbose)
+    # A kernel whose host stub the compiler dropped links as an undefined symbol: load the library now
+    # (all symbols resolved at once) rather than find out at the first call.
+    try:
+        ctypes.CDLL(tmp, mode=os.RTLD_NOW)
+    except OSError as e:
+        os.unlink(tmp)
+        raise RuntimeError(f"the linked library does not load: {e}") from e
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
 

@@ -30,6 +30,7 @@ namespace {
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
+typedef const half8 __attribute__((address_space(3))) *lds_half8_ptr;
 
 constexpr int GW = HLQ_GEMM_WAVES;             // waves per workgroup = K parts, launches of up to 32 rows
 constexpr int GW_WIDE = HLQ_GEMM_WAVES_WIDE;   // the same for launches of 33..64 rows
@@ -40,7 +41,6 @@ constexpr int WS_COUNTER_BYTES = HLQ_WS_COUNTER_BYTES;
 #ifndef HLQ_GEMM_LA
 #define HLQ_GEMM_LA 2                          // MFMA steps between an operand read and its use
 #endif
-constexpr int ROW_BYTES = HLQ_UNIT * 2 + 16;   // one staged row of a unit, padded: conflict-free b128 reads
 
 struct GemmArgs {
     const uint4 *planes;
@@ -77,49 +77,69 @@ __device__ __forceinline__ float dpp_f(float v)
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
 
-// Staging of x[0 .. MR, u*128 .. (u+1)*128) by one wave into its LDS region, rows in their natural k
-// order: the 16 bytes at k = 8t are the A operand of the MFMA step whose B operand comes from plane byte
-// t.  One task = one 16-byte slot of one row (16 slots per row); consecutive lanes write consecutive
-// slots, so the LDS stores are conflict-free.  xs[half * MR + m] receives the fp32 sum of x[m] over 64-k
-// half `half` of the unit (eight consecutive lanes).  MR = rows staged (16, 32 or 64).
+// Staging of x[0 .. MR, k0 .. k0 + KS) by one wave into its LDS region, rows in their natural k order:
+// the 16 bytes at k = 8t are the A operand of the MFMA step whose B operand comes from plane byte t.
+// KS = 128 (a whole unit) for up to 32 rows, 64 (half a unit at a time: `half` = 0, 1) for 64 rows, so that
+// a round always fits 32 registers per lane and 9 KiB of LDS per wave.  One task = one 16-byte slot of one
+// row; consecutive lanes write consecutive slots, so the LDS stores are conflict-free.  xs[half * MR + m]
+// receives the fp32 sum of x[m] over 64-k half `half` of the unit (eight consecutive lanes).
 template <int MR>
 struct StageRegs {
-    static constexpr int TPT = MR * 16 / 64;                         // tasks per lane
+    static constexpr int KS = MR <= 32 ? HLQ_UNIT : HLQ_UNIT / 2;    // k per round
+    static constexpr int SLOTS = KS / 8;                             // 16-byte slots per row
+    static constexpr int TPT = MR * SLOTS / 64;                      // tasks per lane
+    static constexpr int ROW_BYTES = KS * 2 + 16;                    // padded row: conflict-free b128 reads
     uint4 v[TPT];
 };
 
 template <int MR>
-__device__ __forceinline__ void stage_load(StageRegs<MR> &r, const GemmArgs &a, int u, int lane)
+__device__ __forceinline__ void stage_load(StageRegs<MR> &r, const GemmArgs &a, int u, int half, int lane)
 {
-    // The lane number passes through an empty statement so that the row offsets below are recomputed for
-    // every unit (two instructions per task) instead of being kept in registers for the whole kernel.
+    using S = StageRegs<MR>;
+    // The lane number passes through an empty statement so that the offsets below are recomputed for
+    // every round (two instructions per task) instead of being kept in registers for the whole kernel.
     asm volatile("" : "+v"(lane));
-    const uint32_t col_off = ((uint32_t)u * HLQ_UNIT + (lane & 15) * 8) * 2;
+    const uint32_t row_bytes = (uint32_t)a.K * 2;
+    const uint32_t col_off = ((uint32_t)u * HLQ_UNIT + half * S::KS + (lane & (S::SLOTS - 1)) * 8) * 2;
+    const uint32_t last = (uint32_t)(a.M - 1) * row_bytes + col_off;         // rows past M read row M - 1 again
+    uint32_t off = (uint32_t)(lane / S::SLOTS) * row_bytes + col_off;
 #pragma unroll
-    for (int t = 0; t < StageRegs<MR>::TPT; t++) {
-        const int m = (lane >> 4) + 4 * t;
-        const uint32_t mm = (uint32_t)(m < a.M ? m : a.M - 1);
-        r.v[t] = *(const uint4 *)((const unsigned char *)a.x + (mm * (uint32_t)a.K * 2 + col_off));
+    for (int t = 0; t < S::TPT; t++) {
+        r.v[t] = *(const uint4 *)((const unsigned char *)a.x + (off < last ? off : last));
+        off += (64 / S::SLOTS) * row_bytes;
+        asm volatile("" : "+v"(off));            // one add per task: keeps the compiler from re-deriving every offset with a multiply
     }
 }
 
 template <int MR>
-__device__ __forceinline__ void stage_store(const StageRegs<MR> &r, unsigned char *xw, float *xs, int lane)
+__device__ __forceinline__ void stage_store(const StageRegs<MR> &r, unsigned char *xw, float *xs, int half, int lane)
 {
+    using S = StageRegs<MR>;
     const half2v ones = {(_Float16)1.f, (_Float16)1.f};
+    float sum[S::TPT];
+    // the reduction steps of all tasks side by side: no instruction waits for the one just before it
 #pragma unroll
-    for (int t = 0; t < StageRegs<MR>::TPT; t++) {
-        const int idx = lane + t * 64;
-        const int m = idx >> 4, o = idx & 15;
-        float sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].x), ones, 0.f, false);
-        sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].y), ones, sum, false);
-        sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].z), ones, sum, false);
-        sum = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].w), ones, sum, false);
-        sum += dpp_f<0xB1>(sum);                 // the eight slots of a 64-k half: quad, quad pair
-        sum += dpp_f<0x4E>(sum);
-        sum += dpp_f<0x141>(sum);
-        if ((o & 7) == 0) xs[(o >> 3) * MR + m] = sum;
-        *(uint4 *)(xw + m * ROW_BYTES + o * 16) = r.v[t];
+    for (int t = 0; t < S::TPT; t++) {
+        sum[t] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].x), ones, 0.f, false);
+        sum[t] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].y), ones, sum[t], false);
+    }
+#pragma unroll
+    for (int t = 0; t < S::TPT; t++) {
+        sum[t] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].z), ones, sum[t], false);
+        sum[t] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2v, r.v[t].w), ones, sum[t], false);
+    }
+#pragma unroll
+    for (int t = 0; t < S::TPT; t++) sum[t] += dpp_f<0xB1>(sum[t]);      // the eight slots of a 64-k half: quad,
+#pragma unroll
+    for (int t = 0; t < S::TPT; t++) sum[t] += dpp_f<0x4E>(sum[t]);      // quad pair,
+#pragma unroll
+    for (int t = 0; t < S::TPT; t++) sum[t] += dpp_f<0x141>(sum[t]);     // both quad pairs
+    const int m0 = lane / S::SLOTS, o = lane % S::SLOTS;
+#pragma unroll
+    for (int t = 0; t < S::TPT; t++) {
+        const int m = m0 + (64 / S::SLOTS) * t;
+        if ((o & 7) == 0) xs[((o >> 3) + half) * MR + m] = sum[t];
+        *(uint4 *)(xw + m * S::ROW_BYTES + o * 16) = r.v[t];
     }
 }
 
@@ -175,43 +195,52 @@ __device__ __forceinline__ uint32_t row_addr(uint32_t w, int S, uint32_t lanepar
 // registers allocated to the chain until that value exists, i.e. until the last MFMA has written them;
 // otherwise the registers nobody reads are free from the moment that MFMA is issued and could be handed
 // to another value while the MFMA is still going to write them.
+// Operand-table row at LDS address `addr`.  The kernel has no static LDS, so its dynamic LDS -- the table
+// first -- starts at address 0 and the offset formed by row_addr is the address itself; going through the
+// generic `smem + offset` form would cost one more vector instruction per operand (an add of the base).
+__device__ __forceinline__ half8 table_row(uint32_t addr)
+{
+    return *(lds_half8_ptr)(uintptr_t)addr;
+}
+
 __device__ __forceinline__ float hold_until_read(float first_use, const float16v &chain)
 {
     asm volatile("" : "+v"(first_use) : "v"(chain));
     return first_use;
 }
 
-// LDS of a workgroup: the operand table, then one region per wave (a staged unit of MR rows and its
-// half-unit row sums); the cross-wave reduction reuses the table's space after the last unit.
+// LDS of a workgroup: the operand table, then one region per wave (a staged unit, or half unit, of MR rows
+// and the row sums of both halves); the cross-wave reduction reuses the space after the last unit.
 template <int MR>
 struct GemmLds {
     static constexpr int NW = MR <= 32 ? GW : GW_WIDE;               // waves
-    static constexpr int TREP = MR <= 32 ? 16 : 4;                   // copies of the operand table
+    static constexpr int TREP = 16;                                  // copies of the operand table
+    static constexpr int ROW_BYTES = StageRegs<MR>::ROW_BYTES;
     static constexpr int MT = (MR + 31) / 32;                        // 32-row MFMA tiles
     static constexpr int REGS = MR == 16 ? 8 : 16;
     static constexpr int TAB_BYTES = 256 * 16 * TREP;
     static constexpr int WAVE_BYTES = MR * ROW_BYTES + 2 * MR * 4;
     static constexpr int RED_BYTES = NW * MT * 2 * REGS * 64 * 4;
-    static constexpr int BYTES = TAB_BYTES + NW * WAVE_BYTES;
-    static_assert(RED_BYTES <= BYTES, "the reduction reuses the table and the regions");
+    static constexpr int TICKET_OFF = TAB_BYTES + NW * WAVE_BYTES;   // arrival ticket of a K-sliced launch
+    static constexpr int BYTES = TICKET_OFF + 16;                    // no static LDS: the table starts at address 0
+    static_assert(RED_BYTES <= TICKET_OFF, "the reduction reuses the table and the regions");
     static_assert(WAVE_BYTES % 16 == 0, "aligned regions");
 };
 
 // MR = activation rows of the launch rounded up to 16, 32 or 64.  The MFMA tile has 32 rows; with
 // MR = 16 only rows 0..15 are staged (lanes of rows 16..31 read rows 0..15 again) and only the
 // accumulator registers of those rows (0..7 of 16) are scaled, reduced and stored.  With MR = 64 every B
-// operand serves two MFMAs (rows 0..31 and 32..63); the workgroup then has four waves, one per SIMD, and
-// each of them the whole register file: four accumulators, four chains and deeper operand rings.
+// operand serves two MFMAs (rows 0..31 and 32..63) and the activations are staged half a unit at a time.
 // grid = column blocks * K slices.
 template <int BITS, bool G64, int MR>
 __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const GemmArgs a)
 {
     using L = GemmLds<MR>;
-    constexpr int REGS = L::REGS, MT = L::MT, NW = L::NW, THREADS = NW * 64, TREP = L::TREP;
+    constexpr int REGS = L::REGS, MT = L::MT, NW = L::NW, THREADS = NW * 64, TREP = L::TREP, ROW_BYTES = L::ROW_BYTES;
     constexpr int VALS = MT * 2 * REGS * 64;        // fp32 results per wave
     extern __shared__ __align__(256) unsigned char smem[];
     float *red = (float *)smem;                     // reused after the last unit
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, h = lane >> 5;
     const int cb = blockIdx.x / a.ksplit, slice = blockIdx.x - cb * a.ksplit;
     const int u_begin = slice * a.ups, u_end = min(u_begin + a.ups, a.U);
@@ -233,7 +262,7 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
     const int u_first = u_begin + wave;
     if (u_first < u_end) {
         load_unit<BITS, G64>(ua, a, cb, u_first, lane);
-        stage_load<MR>(xr, a, u_first, lane);
+        stage_load<MR>(xr, a, u_first, 0, lane);
     }
     if (u_first + NW < u_end) load_unit<BITS, G64>(ub, a, cb, u_first + NW, lane);
     // operand table: row v holds the eight fp16 values (0 or 1) of the bits of v, TREP copies side by side
@@ -255,10 +284,12 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
     const unsigned char *arow = xw + (MR == 16 ? (col & 15) : col) * ROW_BYTES + h * 64;
 
     // One unit: stage its activations (LDS operations of one wave execute in order, so the wave reads
-    // what it has just written without a barrier), compute, then refill `cur` with the unit two turns ahead.
+    // what it has just written without a barrier), refill `cur` with the unit two turns ahead, compute.
     auto unit = [&](UnitData<BITS> &cur, int u) __attribute__((always_inline)) {
-        stage_store<MR>(xr, xw, xs, lane);
-        if (u + NW < u_end) stage_load<MR>(xr, a, u + NW, lane);
+        if constexpr (MT == 1) {
+            stage_store<MR>(xr, xw, xs, 0, lane);
+            if (u + NW < u_end) stage_load<MR>(xr, a, u + NW, 0, lane);
+        }
         // Lane (col, h) of tile j works on column 32j + col of the block: bring that column's
         // scale / zero dwords and its plane dwords (k half h of each 64-k pair, rotation undone:
         // bit i of tw[b][j][pr] is k = 64 pr + 32 h + i) into the lane.
@@ -275,21 +306,6 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
         }
         split_tiles(cur.zz, cur.zz, zzj[0], zzj[1]);
         if (u + 2 * NW < u_end) load_unit<BITS, G64>(cur, a, cb, u + 2 * NW, lane);
-        // The unit is a list of MFMA steps: for every group of the unit, for every plane, the NQ 16-k
-        // steps of the group.  Step t uses the A operands of its 16 k (one per row tile) and one B
-        // operand per column tile; they are read from LDS LA steps before their use, into rotating
-        // register sets, so that the reads are not waited for.
-        constexpr int NG = G64 ? 2 : 1, NQ = G64 ? 4 : 8;
-        constexpr int NSTEP = NG * BITS * NQ, LA = HLQ_GEMM_LA, RING = LA + 1;
-        half8 aopr[RING][MT], bopr[RING][2];
-        auto issue = [&](int t) __attribute__((always_inline)) {
-            const int g = t / (BITS * NQ), b = (t / NQ) % BITS, q = t % NQ;
-            const int pr = G64 ? g : q / 4, sq = q % 4;
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++) aopr[t % RING][mt] = *(const half8 *)(arow + mt * 32 * ROW_BYTES + pr * 128 + sq * 16);
-#pragma unroll
-            for (int j = 0; j < 2; j++) bopr[t % RING][j] = *(const half8 *)(smem + row_addr<TREP>(tw[b][j][pr], sq, lanepart));
-        };
         // zero term of group g: z[n, g] * sum_{k in g} x[m, k]; C rows of register i: 8*(i/4) + 4h + i%4
         auto zero_term = [&](int g, bool hi) __attribute__((always_inline)) {
             const float zf[2] = {h2f(zzj[0], hi), h2f(zzj[1], hi)};
@@ -312,12 +328,26 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
                     }
                 }
         };
-#pragma unroll
-        for (int t = 0; t < LA && t < NSTEP; t++) issue(t);
+        constexpr int LA = HLQ_GEMM_LA, RING = LA + 1;
         if constexpr (MT == 1) {
-            // One row tile: every (group, plane, column tile) is a chain that starts from zero; its result is
-            // scaled by the group's scale and added to the accumulator (16 or 8 multiply-adds per chain).
+            // The unit is a list of MFMA steps: for every group of the unit, for every plane, the NQ 16-k
+            // steps of the group.  Step t uses the A operand of its 16 k and one B operand per column
+            // tile; they are read from LDS LA steps before their use, into rotating register sets, so that
+            // the reads are not waited for.  Every (group, plane, column tile) is a chain that starts from
+            // zero; its result is scaled by the group's scale and added to the accumulator (16 or 8
+            // multiply-adds per chain).
+            constexpr int NG = G64 ? 2 : 1, NQ = G64 ? 4 : 8, NSTEP = NG * BITS * NQ;
+            half8 aopr[RING], bopr[RING][2];
             float16v tmp[2];
+            auto issue = [&](int t) __attribute__((always_inline)) {
+                const int g = t / (BITS * NQ), b = (t / NQ) % BITS, q = t % NQ;
+                const int pr = G64 ? g : q / 4, sq = q % 4;
+                aopr[t % RING] = *(const half8 *)(arow + pr * 128 + sq * 16);
+#pragma unroll
+                for (int j = 0; j < 2; j++) bopr[t % RING][j] = table_row(row_addr<TREP>(tw[b][j][pr], sq, lanepart));
+            };
+#pragma unroll
+            for (int t = 0; t < LA && t < NSTEP; t++) issue(t);
 #pragma unroll
             for (int t = 0; t < NSTEP; t++) {
                 const int g = t / (BITS * NQ), b = (t / NQ) % BITS, q = t % NQ;
@@ -329,9 +359,9 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
                         float16v zero;
 #pragma unroll
                         for (int i = 0; i < 16; i++) zero[i] = 0.f;
-                        tmp[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aopr[t % RING][0], bopr[t % RING][j], zero, 0, 0, 0);
+                        tmp[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aopr[t % RING], bopr[t % RING][j], zero, 0, 0, 0);
                     } else {
-                        tmp[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aopr[t % RING][0], bopr[t % RING][j], tmp[j], 0, 0, 0);
+                        tmp[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aopr[t % RING], bopr[t % RING][j], tmp[j], 0, 0, 0);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -350,32 +380,59 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
         } else {
             // Two row tiles: a B operand serves two MFMAs, which pays for scaling the operand itself (four
             // packed fp16 multiplications, exact: the operand is 0 or 1) and accumulating straight into the
-            // result, with neither chain registers nor multiply-adds afterwards.
+            // result, with neither chain registers nor multiply-adds afterwards.  The unit is worked on half
+            // by half (one 64-k pair of every plane dword at a time); a step is (16 k, plane): the two A
+            // operands of 16 k are read once for all planes.
+            constexpr int NSTEP = 4 * BITS;
 #pragma unroll
-            for (int t = 0; t < NSTEP; t++) {
-                const int g = t / (BITS * NQ), b = (t / NQ) % BITS, q = t % NQ;
-                const bool hi = G64 ? g == 1 : (u & 1) != 0;
-                if (t + LA < NSTEP) issue(t + LA);
-                __builtin_amdgcn_sched_barrier(0);
+            for (int half = 0; half < 2; half++) {
+                stage_store<MR>(xr, xw, xs, half, lane);
+                if (half == 0) stage_load<MR>(xr, a, u, 1, lane);
+                else if (u + NW < u_end) stage_load<MR>(xr, a, u + NW, 0, lane);
+                const bool hi = G64 ? half == 1 : (u & 1) != 0;
+                half2v s2[BITS][2];
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const uint32_t sc = scj[b][j];
-                    const uint32_t pk = hi ? __builtin_amdgcn_perm(sc, sc, 0x03020302u) : __builtin_amdgcn_perm(sc, sc, 0x01000100u);
-                    const half2v s2 = __builtin_bit_cast(half2v, pk);
-                    half8 bs;
+                for (int b = 0; b < BITS; b++)
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const half2v v = {bopr[t % RING][j][2 * i], bopr[t % RING][j][2 * i + 1]};
-                        const half2v p = v * s2;
-                        bs[2 * i] = p[0];
-                        bs[2 * i + 1] = p[1];
+                    for (int j = 0; j < 2; j++) {
+                        const uint32_t sc = scj[b][j];
+                        s2[b][j] = __builtin_bit_cast(half2v, hi ? __builtin_amdgcn_perm(sc, sc, 0x03020302u)
+                                                                 : __builtin_amdgcn_perm(sc, sc, 0x01000100u));
+                    }
+                half8 aopr[3][MT], bopr[RING][2];
+                auto issue = [&](int t) __attribute__((always_inline)) {
+                    const int q = t / BITS, b = t % BITS;
+                    if (b == 0) {
+#pragma unroll
+                        for (int mt = 0; mt < MT; mt++) aopr[q % 3][mt] = *(const half8 *)(arow + mt * 32 * ROW_BYTES + q * 16);
                     }
 #pragma unroll
-                    for (int mt = 0; mt < MT; mt++)
-                        acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aopr[t % RING][mt], bs, acc[mt][j], 0, 0, 0);
+                    for (int j = 0; j < 2; j++) bopr[t % RING][j] = table_row(row_addr<TREP>(tw[b][j][half], q, lanepart));
+                };
+#pragma unroll
+                for (int t = 0; t < LA && t < NSTEP; t++) issue(t);
+#pragma unroll
+                for (int t = 0; t < NSTEP; t++) {
+                    const int q = t / BITS, b = t % BITS;
+                    if (t + LA < NSTEP) issue(t + LA);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        half8 bs;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const half2v v = {bopr[t % RING][j][2 * i], bopr[t % RING][j][2 * i + 1]};
+                            const half2v p = v * s2[b][j];
+                            bs[2 * i] = p[0];
+                            bs[2 * i + 1] = p[1];
+                        }
+#pragma unroll
+                        for (int mt = 0; mt < MT; mt++)
+                            acc[mt][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(aopr[q % 3][mt], bs, acc[mt][j], 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                __builtin_amdgcn_sched_barrier(0);
-                if (q == NQ - 1 && b == BITS - 1) zero_term(g, hi);
+                if (G64 || half == 1) zero_term(half, hi);
             }
         }
     };
@@ -440,11 +497,11 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     GEMM_STAMP(14);
     __syncthreads();
-    __shared__ unsigned s_ticket;
+    unsigned *s_ticket = (unsigned *)(smem + L::TICKET_OFF);
     unsigned *counter = a.counters + cb;
-    if (tid == 0) s_ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) *s_ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (s_ticket != (unsigned)a.ksplit - 1u) return;
+    if (*s_ticket != (unsigned)a.ksplit - 1u) return;
     // a thread's loads for QB slices are in flight together; summed in slice order
     constexpr int QB = NV <= 8 ? 4 : 2;
     float sum[NV];
@@ -507,9 +564,18 @@ int launch_gemm(const GemmArgs &a, hipStream_t stream)
 {
     auto kern = hlq_gemm_kernel<BITS, G64, MR>;
     const size_t lds = GemmLds<MR>::BYTES;
-    static_assert(GemmLds<MR>::BYTES + 64 <= HLQ_MAX_LDS, "LDS of one workgroup");
+    static_assert(GemmLds<MR>::BYTES <= HLQ_MAX_LDS, "LDS of one workgroup");
     static bool big_lds_done[64] = {};        // per template instance
     if (!allow_big_lds((const void *)kern, lds, (int)lds, big_lds_done)) return ELUTQ_ERR_HIP;
+    // table_row() takes LDS offsets for addresses: true only while the kernel has no static LDS in front of
+    // its dynamic LDS
+    static int static_lds = -1;
+    if (static_lds < 0) {
+        hipFuncAttributes attr;
+        if (hipFuncGetAttributes(&attr, (const void *)kern) != hipSuccess) return ELUTQ_ERR_HIP;
+        static_lds = (int)attr.sharedSizeBytes;
+    }
+    if (static_lds != 0) return ELUTQ_ERR_HIP;
     hipLaunchKernelGGL(kern, dim3(a.ncb * a.ksplit), dim3(GemmLds<MR>::NW * 64), lds, stream, a);
     return hipGetLastError() == hipSuccess ? ELUTQ_OK : ELUTQ_ERR_HIP;
 }
