@@ -31,7 +31,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-KERNEL_TRACE_AVG_US = 6.51     # hlq_gemv_kernel<2, false, 4, true, 1> at 4096 x 14336 in the committed kernel trace
+KERNEL_TRACE_AVG_US = 6.55     # hlq_gemv_kernel<2, false, 4, true, 1> at 4096 x 14336 in the committed kernel trace
 BITS, GROUP = 2, 128
 N_LAYERS = 32
 
