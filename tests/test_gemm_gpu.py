@@ -72,6 +72,22 @@ def test_llama2_13b_prefill_shapes(cuda, m, k, n):
     assert O.rel_err(y, ref) <= TOL
 
 
+@pytest.mark.parametrize("m", [16, 32, 64])
+@pytest.mark.parametrize("bits,group", [(1, 128), (3, 128), (4, 64), (2, 64)])
+def test_prefill_shape_other_formats(cuda, m, bits, group):
+    """The instances of the other formats at a LLaMA-2-13B shape (5120 x 5120: 40 units per column, 80 column
+    blocks, K cut into slices that meet through the workspace): every row count class x planes 1, 3, 4 and
+    groups of 64, against the float64 oracle; bit-identical repeats."""
+    k, n = 5120, 5120
+    L = make_layer(k, n, bits=bits, group=group, m=m, seed=100 + bits + m)
+    _, y = gemm(L, cuda)
+    _, y2 = gemm(L, cuda)
+    w = O.dequantize(L.w_quant, L.w_scale, L.w_zero, group, np.float32)
+    ref = L.x.astype(np.float64) @ w.astype(np.float64).T
+    assert O.rel_err(y, ref) <= TOL
+    assert np.array_equal(y, y2)
+
+
 @pytest.mark.parametrize("kparts", [0, 8])
 @pytest.mark.parametrize("ksplit", [1, 2, 3, 0])
 @pytest.mark.parametrize("m,k,n,bits,group", [(16, 1024, 100, 2, 128), (64, 1280, 320, 2, 128), (40, 1152, 576, 3, 64),
