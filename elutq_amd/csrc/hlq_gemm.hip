@@ -14,8 +14,8 @@
 // fp16 scale -- nothing else is rounded before the final fp16 store.  The zero term uses per-row sums of
 // x over 64-k halves, taken while the activations are staged in LDS as A operand.
 //
-// A workgroup is one column block (64 columns) x one K slice; its waves (eight, or four for more than 32
-// rows) take the units of the slice in turn (wave w: units w, w + 8, ...).  Every wave stages the activations of its own unit in
+// A workgroup is one column block (64 columns) x one K slice; its eight waves take the units of the slice
+// in turn (wave w: units w, w + 8, ...).  Every wave stages the activations of its own unit in
 // its own LDS region, so the waves never wait for each other until the final sum: while one wave of a SIMD
 // stages, the other one keeps the matrix core busy.
 #include <hip/hip_runtime.h>
@@ -32,8 +32,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 typedef const half8 __attribute__((address_space(3))) *lds_half8_ptr;
 
-constexpr int GW = HLQ_GEMM_WAVES;             // waves per workgroup = K parts, launches of up to 32 rows
-constexpr int GW_WIDE = HLQ_GEMM_WAVES_WIDE;   // the same for launches of 33..64 rows
+constexpr int GW = HLQ_GEMM_WAVES;             // waves per workgroup = K parts
 constexpr int WS_COUNTER_BYTES = HLQ_WS_COUNTER_BYTES;
 #ifndef HLQ_GEMM_LA
 #define HLQ_GEMM_LA 2                          // MFMA steps between an operand read and its use
@@ -213,7 +212,7 @@ __device__ __forceinline__ float hold_until_read(float first_use, const float16v
 // and the row sums of both halves); the cross-wave reduction reuses the space after the last unit.
 template <int MR>
 struct GemmLds {
-    static constexpr int NW = MR <= 32 ? GW : GW_WIDE;               // waves
+    static constexpr int NW = GW;                                    // waves
     static constexpr int TREP = 16;                                  // copies of the operand table
     static constexpr int ROW_BYTES = StageRegs<MR>::ROW_BYTES;
     static constexpr int MT = (MR + 31) / 32;                        // 32-row MFMA tiles
@@ -642,7 +641,7 @@ int hlq_gemm_chunk_with_extra(const void *d_planes, const void *d_scales, const 
     if (group != 64 && group != 128) return ELUTQ_ERR_GROUP;
     if (K < HLQ_UNIT || N < 1 || K % HLQ_UNIT != 0 || K % group != 0) return ELUTQ_ERR_SHAPE;
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
-    if (kparts != 0 && kparts != (M <= 32 ? HLQ_GEMM_WAVES : HLQ_GEMM_WAVES_WIDE)) return ELUTQ_ERR_TUNING;
+    if (kparts != 0 && kparts != HLQ_GEMM_WAVES) return ELUTQ_ERR_TUNING;
     if (ksplit < 0 || ksplit > K / HLQ_UNIT) return ELUTQ_ERR_TUNING;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     int ks = ksplit, ups;

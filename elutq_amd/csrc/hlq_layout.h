@@ -28,8 +28,7 @@
 #define HLQ_NUM_CU 256                 /* MI355X */
 #define HLQ_MAX_LDS (160 * 1024)       /* per workgroup on gfx950 */
 #define HLQ_WS_COUNTER_BYTES (64 * 1024) /* head of every workspace: one arrival counter per column block */
-#define HLQ_GEMM_WAVES 8               /* waves per GEMM workgroup, up to 32 rows */
-#define HLQ_GEMM_WAVES_WIDE 8          /* the same for 33..64 rows */
+#define HLQ_GEMM_WAVES 8               /* waves per GEMM workgroup */
 #define HLQ_GEMM_MAX_M 64              /* rows per GEMM launch; more rows run in chunks of this many (weights re-streamed) */
 
 struct HlqGeo {
@@ -57,14 +56,14 @@ static inline size_t hlq_planes_bytes(const HlqGeo &g) { return (size_t)g.ncb * 
 static inline size_t hlq_scales_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * g.bits * HLQ_CB * 4; }
 static inline size_t hlq_zeros_bytes(const HlqGeo &g) { return (size_t)g.ncb * g.NT * HLQ_CB * 4; }
 
-// Launch shape of the small-batch GEMM.  A workgroup is one column block x one K slice; its waves
-// (HLQ_GEMM_WAVES, or HLQ_GEMM_WAVES_WIDE above 32 rows) take the units of the slice in turn.  K is cut
+// Launch shape of the small-batch GEMM.  A workgroup is one column block x one K slice; its
+// HLQ_GEMM_WAVES waves take the units of the slice in turn.  K is cut
 // into ksplit slices of ups units handled by different workgroups that meet through device memory.  That
 // meeting costs about as much as two units per wave, so K is cut only where the units saved outweigh it,
 // and never into more workgroups than the chip has CUs.
 static inline void hlq_gemm_shape(const HlqGeo &g, int M, int &ksplit, int &ups)
 {
-    const int waves = M <= 32 ? HLQ_GEMM_WAVES : HLQ_GEMM_WAVES_WIDE;
+    const int waves = HLQ_GEMM_WAVES;
     const int turns = (g.U + waves - 1) / waves;        // units per wave over all of K
     int ks = ksplit;
     if (ks <= 0) {
