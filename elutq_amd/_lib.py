@@ -106,6 +106,8 @@ def lib() -> ctypes.CDLL:
 
 
 GEMV_ENGINES = {"auto": 0, "lut": 1, "mfma": 2}
+# values of the `ksplit` tuning argument that name a kernel instead of a slice count (include/elutq_hip.h)
+GEMV_NARROW16, GEMV_NARROW32, GEMV_WIDE = -16, -32, -64
 
 
 def set_gemv_engine(name: str) -> None:

@@ -553,11 +553,37 @@ int g_gemv_engine = ELUTQ_GEMV_ENGINE_AUTO;
 // function for the launch itself and for the queries about it (elutq_hlq_gemv_slices, _accepts_slices).
 struct LaunchShape {
     bool mfma;
+    int narrow;              // 0, or the columns per wave of the narrow-tile kernel (16 / 32)
     int ksplit, ups, waves;
 };
 
-int plan_launch(const HlqGeo &g, int bits, int ksplit, int waves, LaunchShape &sh)
+// `allow_narrow`: the call has nothing the narrow-tile kernel lacks (extra term, handed-over slices).
+int plan_launch(const HlqGeo &g, int bits, int ksplit, int waves, bool allow_narrow, LaunchShape &sh)
 {
+    sh.mfma = false;
+    sh.narrow = 0;
+    if (ksplit == ELUTQ_GEMV_WIDE) {
+        ksplit = 0;
+        allow_narrow = false;
+    }
+    if (ksplit == ELUTQ_GEMV_NARROW16 || ksplit == ELUTQ_GEMV_NARROW32) {
+        // the caller's choice of the narrow-tile kernel
+        const int cw = ksplit == ELUTQ_GEMV_NARROW16 ? 16 : 32;
+        const int rounds = hlq_gemv_narrow_rounds(g.U, cw);
+        if (!allow_narrow || waves != 0 || rounds == 0) return ELUTQ_ERR_TUNING;
+        sh.narrow = cw;
+    } else if (allow_narrow && ksplit == 0 && waves == 0 && g_gemv_engine != ELUTQ_GEMV_ENGINE_MFMA) {
+        // Fewer column blocks than compute units: tiles of 16 (32) columns give four (two) times the
+        // workgroups without cutting K, where the tables of all of K fit one workgroup's LDS (measured on
+        // MI355X: 4096x4096 5.1 -> 3.x us, where K slices only trade lookups for their meeting).
+        if (g.ncb * 4 <= NUM_CU && hlq_gemv_narrow_rounds(g.U, 16)) sh.narrow = 16;
+        else if (g.ncb * 2 <= NUM_CU && hlq_gemv_narrow_rounds(g.U, 32)) sh.narrow = 32;
+    }
+    if (sh.narrow) {
+        const int per_wave = 64 / sh.narrow * hlq_gemv_narrow_rounds(g.U, sh.narrow);
+        sh.ksplit = 1; sh.ups = g.U; sh.waves = (g.U + per_wave - 1) / per_wave;
+        return ELUTQ_OK;
+    }
     if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return ELUTQ_ERR_TUNING;
     const bool auto_waves = waves <= 0;
     // measured on MI355X: the matrix-core kernel streams large layers as fast as the LUT kernel but a launch of one
@@ -647,7 +673,8 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     LaunchShape sh;
-    rc = plan_launch(g, bits, ksplit, waves, sh);
+    const bool allow_narrow = !d_extra && !(fusion && (fusion->n_slices_in != 0 || fusion->d_slices_out));
+    rc = plan_launch(g, bits, ksplit, waves, allow_narrow, sh);
     if (rc != ELUTQ_OK) return rc;
     ksplit = sh.ksplit; waves = sh.waves;
     const int ups = sh.ups;
@@ -703,6 +730,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         a.counters = (HLQ_GLOBAL unsigned *)d_workspace;
         a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
+    if (sh.narrow) return hlq_gemv_narrow_launch(&a, sizeof(a), bits, group, sh.narrow, stream);
     if (sh.mfma) return hlq_gemv_mfma_launch(&a, sizeof(a), bits, group, waves, stage_bytes, stream);
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves) + stage_bytes, (hipStream_t)stream);
 }
@@ -725,7 +753,7 @@ extern "C" int elutq_hlq_gemv_accepts_slices(int K, int N, int bits, int group, 
     if (n_slices < 1 || n_slices > GEMV_MAX_SLICES_IN) return 0;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     LaunchShape sh;
-    if (plan_launch(g, bits, ksplit, waves, sh) != ELUTQ_OK) return 0;
+    if (plan_launch(g, bits, ksplit, waves, false, sh) != ELUTQ_OK) return 0;
     if ((long long)g.ncb * sh.ksplit > NUM_CU) return 0;
     return shape_lds_bytes(sh, bits) + (size_t)K * sizeof(uint16_t) <= (size_t)MAX_LDS ? 1 : 0;
 }
@@ -735,7 +763,8 @@ extern "C" int elutq_hlq_gemv_slices(int K, int N, int bits, int group, int kspl
     if (check_shape(K, N, bits, group) != ELUTQ_OK) return 0;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     LaunchShape sh;
-    if (plan_launch(g, bits, ksplit, waves, sh) != ELUTQ_OK) return 0;          // the same steps as the launch itself
+    // the wide-tile kernel's figure (a producer of handed-over slices runs on it), unless the caller names the narrow one
+    if (plan_launch(g, bits, ksplit, waves, ksplit == ELUTQ_GEMV_NARROW16 || ksplit == ELUTQ_GEMV_NARROW32, sh) != ELUTQ_OK) return 0;
     return sh.ksplit;
 }
 

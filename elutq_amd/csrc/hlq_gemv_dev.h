@@ -82,31 +82,48 @@ __device__ __forceinline__ float h2f_lo(uint32_t v) { return (float)__builtin_bi
 __device__ __forceinline__ float h2f_hi(uint32_t v) { return (float)__builtin_bit_cast(_Float16, (uint16_t)(v >> 16)); }
 
 // dst = base | src.byte<SEL>: the table address of one lookup.  `src` is a plane dword (or its
-// rotation by 4) masked to bits 2..5 of every byte, i.e. 4 * nibble; `base` (wave-uniform, a
-// multiple of 256) is the LDS address of the unit's tables.
+// rotation by 4) masked to bits 2..5 of every byte, i.e. 4 * nibble; `base` (a multiple of 64) is the
+// LDS address of the unit's tables: wave-uniform where all lanes of a wave work on the same unit
+// (HLQ_SDWA_OR), a vector register where they do not (HLQ_SDWA_OR_V).
 #define HLQ_SDWA_OR(dst, base, src, SEL)                                                       \
     asm("v_or_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD "         \
         "src1_sel:BYTE_" #SEL                                                                  \
         : "=v"(dst)                                                                            \
         : "s"(base), "v"(src))
+#define HLQ_SDWA_OR_V(dst, base, src, SEL)                                                     \
+    asm("v_or_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD "         \
+        "src1_sel:BYTE_" #SEL                                                                  \
+        : "=v"(dst)                                                                            \
+        : "v"(base), "v"(src))
 
 // Eight lookups for one plane dword (32 k): chunks 8*D .. 8*D+7 of the unit.  Issue and sum are
 // separate so that the lookups of the next dword are on their way to LDS before the wave waits
-// for the results of this one (LDS returns a wave's reads in order).
-template <int D>
+// for the results of this one (LDS returns a wave's reads in order).  VBASE: `base` differs between lanes.
+template <int D, bool VBASE = false>
 __device__ __forceinline__ void lookup_issue(uint32_t w, uint32_t base, int (&v)[8])
 {
     const uint32_t wm = w & 0x3C3C3C3Cu;
     const uint32_t rm = __builtin_amdgcn_alignbit(w, w, 4) & 0x3C3C3C3Cu;
     uint32_t a[8];
-    HLQ_SDWA_OR(a[0], base, wm, 0);
-    HLQ_SDWA_OR(a[1], base, rm, 0);
-    HLQ_SDWA_OR(a[2], base, wm, 1);
-    HLQ_SDWA_OR(a[3], base, rm, 1);
-    HLQ_SDWA_OR(a[4], base, wm, 2);
-    HLQ_SDWA_OR(a[5], base, rm, 2);
-    HLQ_SDWA_OR(a[6], base, wm, 3);
-    HLQ_SDWA_OR(a[7], base, rm, 3);
+    if constexpr (VBASE) {
+        HLQ_SDWA_OR_V(a[0], base, wm, 0);
+        HLQ_SDWA_OR_V(a[1], base, rm, 0);
+        HLQ_SDWA_OR_V(a[2], base, wm, 1);
+        HLQ_SDWA_OR_V(a[3], base, rm, 1);
+        HLQ_SDWA_OR_V(a[4], base, wm, 2);
+        HLQ_SDWA_OR_V(a[5], base, rm, 2);
+        HLQ_SDWA_OR_V(a[6], base, wm, 3);
+        HLQ_SDWA_OR_V(a[7], base, rm, 3);
+    } else {
+        HLQ_SDWA_OR(a[0], base, wm, 0);
+        HLQ_SDWA_OR(a[1], base, rm, 0);
+        HLQ_SDWA_OR(a[2], base, wm, 1);
+        HLQ_SDWA_OR(a[3], base, rm, 1);
+        HLQ_SDWA_OR(a[4], base, wm, 2);
+        HLQ_SDWA_OR(a[5], base, rm, 2);
+        HLQ_SDWA_OR(a[6], base, wm, 3);
+        HLQ_SDWA_OR(a[7], base, rm, 3);
+    }
     constexpr int off = D * 8 * TBL_BYTES;
 #pragma unroll
     for (int j = 0; j < 8; j++) v[j] = lds_ld(a[j], off + j * TBL_BYTES);

@@ -343,6 +343,14 @@ class LlamaDecoder(nn.Module):
             self._defer_down = [i + 1 < len(self.layers) and 2 <= layer.down_proj.slices <= MAX_DEFERRED_SLICES
                                 and self.layers[i + 1].qkv.accepts_slices(layer.down_proj.slices)
                                 for i, layer in enumerate(self.layers)]
+            # a launch that takes or leaves K slices runs on the wide-tile kernel; a q|k|v that may do either is
+            # pinned to it, so that the step computes the same bits whether or not the slices are handed over
+            for i, layer in enumerate(self.layers):
+                q = layer.qkv
+                if q.ksplit == 0 and ((i > 0 and self._defer_down[i - 1]) or (d == 128 and q.bias is None and q.slices >= 2)):
+                    q.ksplit = _lib.GEMV_WIDE
+                if self._defer_down[i] and layer.down_proj.ksplit == 0:
+                    layer.down_proj.ksplit = _lib.GEMV_WIDE
 
     @classmethod
     def from_export(cls, root: str, s: LlamaShape, device="cuda", fuse: bool = True, impl: str = "hip",

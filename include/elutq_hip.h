@@ -141,7 +141,16 @@ int elutq_hlq_gemv_f16_static(const void *d_planes, const void *d_scales, const 
  * per column block (1..K/128) and `waves` wavefronts per workgroup
  * (1..16); 0 = library default.  For tuning and for tests that must reach every
  * reduction path; results do not depend on these beyond fp32 summation order.
+ * ksplit = ELUTQ_GEMV_NARROW16 / ELUTQ_GEMV_NARROW32 (with waves = 0) names the narrow-tile kernel:
+ * a workgroup owns 16 / 32 columns over all of K, so a layer with few column blocks fills the chip
+ * without K slices; K <= 8192, else ELUTQ_ERR_TUNING.  With ksplit = waves = 0 the library takes it
+ * where the layer has at most 64 / 128 column blocks of 64; ksplit = ELUTQ_GEMV_WIDE keeps it on the
+ * wide-tile kernel (64 columns per wavefront) with the library's own K slicing -- the kernel a call with
+ * handed-over slices (elutq_gemv_fusion) or an extra term always runs on.
  */
+#define ELUTQ_GEMV_NARROW16 (-16)
+#define ELUTQ_GEMV_NARROW32 (-32)
+#define ELUTQ_GEMV_WIDE (-64)
 int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const void *d_zeros,
                              const void *d_bias, const void *d_x, void *d_y,
                              int K, int N, int bits, int group,
@@ -186,7 +195,9 @@ typedef struct elutq_gemv_fusion {
 } elutq_gemv_fusion;
 
 /* K slices the GEMV launch of this shape is divided into (ksplit / waves as in
- * elutq_hlq_gemv_f16_tuned, 0 = default); 0 for an unsupported shape or tuning. */
+ * elutq_hlq_gemv_f16_tuned, 0 = default); 0 for an unsupported shape or tuning.  With ksplit = 0 the
+ * figure is that of the wide-tile kernel, on which a producer of handed-over slices runs (and an upper
+ * bound otherwise: the narrow-tile kernel has no slices). */
 int elutq_hlq_gemv_slices(int K, int N, int bits, int group, int ksplit, int waves);
 
 /* 1 if a launch of this shape (ksplit / waves as the call would pass them) accepts `n_slices`

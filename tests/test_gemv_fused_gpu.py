@@ -20,7 +20,8 @@ def build(k, n, bits, group, seed, dev):
 
 
 @pytest.mark.parametrize("k,n,bits,group", [(1024, 256, 2, 128), (512, 100, 3, 64), (4096, 1024, 2, 128)])
-@pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 4), (2, 16)])
+@pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 4), (2, 16), (_lib.GEMV_NARROW16, 0), (_lib.GEMV_NARROW32, 0),
+                                          (_lib.GEMV_WIDE, 0)])
 def test_rmsnorm_prologue_and_residual(cuda, k, n, bits, group, ksplit, waves):
     L, mod = build(k, n, bits, group, 5, cuda)
     mod.ksplit, mod.waves = ksplit, waves
@@ -43,8 +44,10 @@ def test_rmsnorm_prologue_and_residual(cuda, k, n, bits, group, ksplit, waves):
 
 
 @pytest.mark.parametrize("k,n,bits,group", [(1024, 256, 2, 128), (1536, 192, 4, 64)])
-def test_silu_mul_prologue(cuda, k, n, bits, group):
+@pytest.mark.parametrize("ksplit", [0, _lib.GEMV_NARROW16, _lib.GEMV_NARROW32, _lib.GEMV_WIDE])
+def test_silu_mul_prologue(cuda, k, n, bits, group, ksplit):
     L, mod = build(k, n, bits, group, 7, cuda)
+    mod.ksplit = ksplit
     g = torch.Generator(device=cuda).manual_seed(2)
     gu = torch.randn(1, 2 * k, generator=g, device=cuda).half()
     res = torch.randn(1, n, generator=g, device=cuda).half()

@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 import torch
 
+from elutq_amd import _lib
 from elutq_amd.hlq_linear import HLQLinear
 from elutq_amd.synth import LLAMA3_8B_SHAPES, make_layer
 from oracle import hlq_oracle as O
@@ -35,7 +36,8 @@ def run(m, x, dev):
     (256, 64, 2, 128), (512, 128, 2, 128), (1024, 256, 3, 128), (1024, 192, 2, 64),
     (384, 70, 2, 128), (128, 1, 1, 128), (640, 100, 4, 64), (2048, 512, 4, 128), (384, 64, 3, 64),
 ])
-@pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 1), (1, 4), (2, 2), (3, 8)])
+@pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 1), (1, 4), (2, 2), (3, 8), (_lib.GEMV_NARROW16, 0),
+                                          (_lib.GEMV_NARROW32, 0), (_lib.GEMV_WIDE, 0)])
 def test_gemv_matches_oracle(cuda, k, n, bits, group, ksplit, waves):
     L = make_layer(k, n, bits=bits, group=group, seed=k + n + bits, bias=(n % 3 == 0))
     ks = min(ksplit, k // 128)
@@ -56,7 +58,10 @@ def test_gemv_close_to_reference_fp16_chain(cuda, lutref, bits, group):
     assert np.max(np.abs(y - yref)) <= 2e-2 * rms
 
 
-@pytest.mark.parametrize("bits,group,ksplit", [(2, 128, 1), (2, 128, 2), (3, 64, 0), (4, 128, 3)])
+@pytest.mark.parametrize("bits,group,ksplit", [(2, 128, 1), (2, 128, 2), (3, 64, 0), (4, 128, 3),
+                                               (2, 128, _lib.GEMV_NARROW16), (3, 64, _lib.GEMV_NARROW32),
+                                               (4, 128, _lib.GEMV_NARROW16), (1, 64, _lib.GEMV_NARROW32),
+                                               (2, 128, _lib.GEMV_WIDE)])
 def test_gemv_bit_exact_on_integer_inputs(cuda, lutref, bits, group, ksplit):
     """x in {-2..2}, power-of-two scales, quarter-integer zeros: every partial sum is exactly
     representable, so GPU == float64 == the reference's fp16 chain, bit for bit."""
@@ -147,13 +152,16 @@ def test_dequantize_matches_oracle(cuda):
         assert np.array_equal(w, v.astype(np.float16))
 
 
-@pytest.mark.parametrize("name", ["q_proj", "k_proj", "gate_proj", "down_proj"])
+@pytest.mark.parametrize("name,ksplit", [("q_proj", 0), ("q_proj", _lib.GEMV_WIDE), ("k_proj", 0), ("k_proj", _lib.GEMV_WIDE),
+                                         ("gate_proj", 0), ("down_proj", 0)])
 @pytest.mark.parametrize("bits,group", [(2, 128), (3, 128), (2, 64)])
-def test_llama3_8b_shapes_full_size(cuda, name, bits, group):
-    """The LLaMA-3-8B projection shapes at full size: oracle comparison plus size-independent properties."""
+def test_llama3_8b_shapes_full_size(cuda, name, bits, group, ksplit):
+    """The LLaMA-3-8B projection shapes at full size: oracle comparison plus size-independent properties, on the
+    kernel the library picks (narrow tiles for q and k, wide tiles for gate and down) and, for q and k, on the
+    wide-tile kernel as well."""
     k, n = LLAMA3_8B_SHAPES[name]
     L = make_layer(k, n, bits=bits, group=group, seed=7)
-    m = to_mod(L, cuda)
+    m = to_mod(L, cuda, ksplit)
     y = run(m, L.x, cuda)[0]
     w = O.dequantize(L.w_quant, L.w_scale, L.w_zero, group, np.float32)
     ref = w.astype(np.float64) @ L.x[0].astype(np.float64)
@@ -209,7 +217,7 @@ def test_two_streams_with_their_own_workspaces(cuda):
 
 
 @pytest.mark.parametrize("bad", [float("nan"), float("inf"), float("-inf")])
-@pytest.mark.parametrize("ksplit,waves", [(0, 0), (2, 8)])
+@pytest.mark.parametrize("ksplit,waves", [(0, 0), (2, 8), (_lib.GEMV_WIDE, 0)])
 def test_non_finite_activations_reach_the_output(cuda, bad, ksplit, waves):
     """The reference's fp16 table entries and sums carry a NaN or an infinity in x into every output it
     touches (arm_t_mac_kernal.cpp:111-126, arm_gemm.cpp:250-279).  The integer tables here cannot hold

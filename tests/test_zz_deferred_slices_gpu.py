@@ -25,6 +25,7 @@ def test_consumer_sees_what_the_producer_would_have_written(cuda, ffn, hidden, n
     """down (SiLU*up prologue, K slices) -> next q|k|v (RMSNorm prologue), at the shapes of the small test
     model and of LLaMA-3-8B, and at the other plane counts / group size."""
     down, qkv = build(ffn, hidden, 1, cuda, bits, group), build(hidden, n_next, 2, cuda, bits, group)
+    qkv.ksplit = _lib.GEMV_WIDE          # the kernel a launch with handed-over slices runs on, for the reference too
     S = down.slices
     assert 2 <= S <= 4
     g = torch.Generator(device=cuda).manual_seed(3)
