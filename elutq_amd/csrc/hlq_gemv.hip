@@ -580,8 +580,8 @@ int plan_launch(const HlqGeo &g, int bits, int ksplit, int waves, bool allow_nar
         else if (g.ncb * 2 <= NUM_CU && hlq_gemv_narrow_rounds(g.U, 32)) sh.narrow = 32;
     }
     if (sh.narrow) {
-        const int per_wave = 64 / sh.narrow * hlq_gemv_narrow_rounds(g.U, sh.narrow);
-        sh.ksplit = 1; sh.ups = g.U; sh.waves = (g.U + per_wave - 1) / per_wave;
+        const int per_wave = 64 / sh.narrow;         // units a wave covers per round
+        sh.ksplit = 1; sh.ups = g.U; sh.waves = g.U < 16 * per_wave ? (g.U + per_wave - 1) / per_wave : 16;
         return ELUTQ_OK;
     }
     if (ksplit < 0 || waves < 0 || waves > 16 || ksplit > g.U) return ELUTQ_ERR_TUNING;

@@ -51,14 +51,19 @@ __device__ __forceinline__ float process_sub_lane(const uint4 &w, uint32_t sc_ra
     lookup_issue<0, true>(w.x, ub, v0);
     lookup_issue<1, true>(w.y, ub, v1);
     __builtin_amdgcn_sched_barrier(0);
+    // (the empty statements pin each sum in front of the scheduling barrier that follows it: a pure integer add
+    // has no place of its own in the instruction order, and the lookups of a whole round piled up in registers)
     int i0 = lookup_sum(v0, 0);
+    asm volatile("" : "+v"(i0));
     lookup_issue<2, true>(w.z, ub, v0);
     __builtin_amdgcn_sched_barrier(0);
     i0 = lookup_sum(v1, i0);
+    asm volatile("" : "+v"(i0));
     lookup_issue<3, true>(w.w, ub, v1);
     __builtin_amdgcn_sched_barrier(0);
     int i1 = lookup_sum(v0, 0);
     i1 = lookup_sum(v1, i1);
+    asm volatile("" : "+v"(i1));
     const uint32_t sh = odd ? 16u : 0u;
     const uint32_t sc = G64 ? sc_raw : ((sc_raw >> sh) & 0xffffu) * 0x10001u;
     acc = fmaf((float)i0 * h0.y, h2f_lo(sc), acc);
