@@ -619,6 +619,7 @@ int plan_launch(const HlqGeo &g, int bits, int ksplit, int waves, bool allow_nar
 
 size_t shape_lds_bytes(const LaunchShape &sh, int bits)
 {
+    if (sh.narrow) return hlq_gemv_narrow_lds_bytes(sh.ups, sh.narrow);
     return sh.mfma ? hlq_gemv_mfma_lds_bytes(sh.ups, sh.waves) : gemv_lds_bytes(sh.ups, bits, sh.waves);
 }
 
@@ -673,7 +674,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     LaunchShape sh;
-    const bool allow_narrow = !d_extra && !(fusion && (fusion->n_slices_in != 0 || fusion->d_slices_out));
+    const bool allow_narrow = !d_extra && !(fusion && fusion->d_slices_out);
     rc = plan_launch(g, bits, ksplit, waves, allow_narrow, sh);
     if (rc != ELUTQ_OK) return rc;
     ksplit = sh.ksplit; waves = sh.waves;
@@ -712,7 +713,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         if (fusion->d_x_out == d_x) return ELUTQ_ERR_TUNING;       // other workgroups still read the base
         // only launches of one tile per workgroup take slices: the instances that walk a run of column
         // blocks (more tiles than compute units) have not been validated as consumers
-        if ((long long)g.ncb * ksplit > NUM_CU) return ELUTQ_ERR_TUNING;
+        if (!sh.narrow && (long long)g.ncb * ksplit > NUM_CU) return ELUTQ_ERR_TUNING;
         a.x_out = (HLQ_GLOBAL uint16_t *)fusion->d_x_out;
         stage_bytes = (size_t)K * sizeof(uint16_t);
         if (shape_lds_bytes(sh, bits) + stage_bytes > (size_t)MAX_LDS) return ELUTQ_ERR_SHAPE;
@@ -730,7 +731,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         a.counters = (HLQ_GLOBAL unsigned *)d_workspace;
         a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
     }
-    if (sh.narrow) return hlq_gemv_narrow_launch(&a, sizeof(a), bits, group, sh.narrow, stream);
+    if (sh.narrow) return hlq_gemv_narrow_launch(&a, sizeof(a), bits, group, sh.narrow, stage_bytes, stream);
     if (sh.mfma) return hlq_gemv_mfma_launch(&a, sizeof(a), bits, group, waves, stage_bytes, stream);
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves) + stage_bytes, (hipStream_t)stream);
 }
@@ -753,8 +754,8 @@ extern "C" int elutq_hlq_gemv_accepts_slices(int K, int N, int bits, int group, 
     if (n_slices < 1 || n_slices > GEMV_MAX_SLICES_IN) return 0;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     LaunchShape sh;
-    if (plan_launch(g, bits, ksplit, waves, false, sh) != ELUTQ_OK) return 0;
-    if ((long long)g.ncb * sh.ksplit > NUM_CU) return 0;
+    if (plan_launch(g, bits, ksplit, waves, true, sh) != ELUTQ_OK) return 0;
+    if (!sh.narrow && (long long)g.ncb * sh.ksplit > NUM_CU) return 0;
     return shape_lds_bytes(sh, bits) + (size_t)K * sizeof(uint16_t) <= (size_t)MAX_LDS ? 1 : 0;
 }
 

@@ -33,11 +33,12 @@ struct NarrowGeo {
     static constexpr int WAVE_LDS = (NU * UNIT_STRIDE + 2 * NU * 8 + 255) & ~255;
 };
 
-// dynamic LDS: [waves][WAVE_LDS] | float [waves][64] cross-wave sums | float [HLQ_RSTD_SCRATCH]
+// dynamic LDS: [waves][WAVE_LDS] | float [waves][64] cross-wave sums | float [HLQ_RSTD_SCRATCH] | gap |
+// fp16 [K] staged activations (launches that take handed-over slices only)
 template <int CW, int R>
 constexpr size_t narrow_lds_bytes(int waves)
 {
-    return (size_t)waves * NarrowGeo<CW, R>::WAVE_LDS + (size_t)waves * 64 * 4 + HLQ_RSTD_SCRATCH * 4;
+    return (size_t)waves * NarrowGeo<CW, R>::WAVE_LDS + (size_t)waves * 64 * 4 + (HLQ_RSTD_SCRATCH + HLQ_STAGE_GAP) * 4;
 }
 
 // The lookups of one sub-task (128 k of one plane) where every lane has its own unit: `ub` is the LDS
@@ -110,6 +111,12 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     // activations: chunk p * 64 + lane of the wave's NU units (clamped to K: units past the end are masked below)
     uint2 rfirst = make_uint2(0, 0);
     if (prologue == 1) rfirst = rstd_first_load(a, K, tid);
+    // x as a base vector plus the unsummed K slices of the launch that produced it (host: prologue 1 only):
+    // block_rstd forms every chunk once, into `stage`
+    const bool sliced = !PLAIN && a.n_slices_in > 0;
+    SliceChunk sfirst = {};
+    uint2 *stage = (uint2 *)(rstd_scratch + HLQ_RSTD_SCRATCH + HLQ_STAGE_GAP);
+    if (sliced) load_slice_chunk(a, K, min(tid, K / 4 - 1), sfirst);
     uint2 raw[PASSES], raw2[PASSES];
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
@@ -140,9 +147,11 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     asm volatile("" ::: "memory");
 
     float rstd = 1.f;
-    if (prologue == 1) {
-        const SliceChunk none = {};
-        rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst, none, false, nullptr, false);
+    if (prologue == 1)
+        rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst, sfirst, sliced, stage, sliced && a.x_out && blockIdx.x == 0);
+    if (sliced) {
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) raw[p] = stage[min(ub * 32 + p * 64 + lane, K / 4 - 1)];
     }
 
     // the wave's own tables: chunk ci of the wave belongs to unit ci / 32, half unit ci / 16
@@ -185,12 +194,13 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
 }
 
 template <int BITS, bool G64, int CW, int R, bool PLAIN>
-int launch_narrow_v(const GemvArgs &a, hipStream_t stream)
+int launch_narrow_v(const GemvArgs &a, size_t stage_bytes, hipStream_t stream)
 {
     using Geo = NarrowGeo<CW, R>;
     const int waves = (a.U + Geo::NU - 1) / Geo::NU;
-    const size_t lds = narrow_lds_bytes<CW, R>(waves);
-    if (waves < 1 || waves > 16 || lds > (size_t)MAX_LDS) return ELUTQ_ERR_TUNING;
+    const size_t lds = narrow_lds_bytes<CW, R>(waves) + stage_bytes;
+    if (waves < 1 || waves > 16) return ELUTQ_ERR_TUNING;
+    if (lds > (size_t)MAX_LDS) return ELUTQ_ERR_SHAPE;
     auto kern = hlq_gemv_narrow_kernel<BITS, G64, CW, R, PLAIN>;
     static bool big_lds_done[64] = {};        // per template instance
     if (lds > 64 * 1024) {
@@ -207,19 +217,19 @@ int launch_narrow_v(const GemvArgs &a, hipStream_t stream)
 }
 
 template <int BITS, bool G64, int CW, int R>
-int launch_narrow_r(const GemvArgs &a, hipStream_t stream)
+int launch_narrow_r(const GemvArgs &a, size_t stage_bytes, hipStream_t stream)
 {
-    if (a.prologue == 0 && !a.residual) return launch_narrow_v<BITS, G64, CW, R, true>(a, stream);
-    return launch_narrow_v<BITS, G64, CW, R, false>(a, stream);
+    if (a.prologue == 0 && !a.residual) return launch_narrow_v<BITS, G64, CW, R, true>(a, stage_bytes, stream);
+    return launch_narrow_v<BITS, G64, CW, R, false>(a, stage_bytes, stream);
 }
 
 template <int BITS, bool G64>
-int launch_narrow(const GemvArgs &a, int cw, hipStream_t stream)
+int launch_narrow(const GemvArgs &a, int cw, size_t stage_bytes, hipStream_t stream)
 {
     const int rounds = hlq_gemv_narrow_rounds(a.U, cw);
-    if (cw == 16 && rounds == 1) return launch_narrow_r<BITS, G64, 16, 1>(a, stream);
-    if (cw == 32 && rounds == 1) return launch_narrow_r<BITS, G64, 32, 1>(a, stream);
-    if (cw == 32 && rounds == 2) return launch_narrow_r<BITS, G64, 32, 2>(a, stream);
+    if (cw == 16 && rounds == 1) return launch_narrow_r<BITS, G64, 16, 1>(a, stage_bytes, stream);
+    if (cw == 32 && rounds == 1) return launch_narrow_r<BITS, G64, 32, 1>(a, stage_bytes, stream);
+    if (cw == 32 && rounds == 2) return launch_narrow_r<BITS, G64, 32, 2>(a, stage_bytes, stream);
     return ELUTQ_ERR_TUNING;
 }
 
@@ -232,18 +242,28 @@ int hlq_gemv_narrow_rounds(int U, int cw)
     return 0;
 }
 
-int hlq_gemv_narrow_launch(const void *gemv_args, size_t args_bytes, int bits, int group, int cw, void *stream)
+size_t hlq_gemv_narrow_lds_bytes(int U, int cw)
+{
+    const int rounds = hlq_gemv_narrow_rounds(U, cw);
+    if (cw == 16 && rounds == 1) return narrow_lds_bytes<16, 1>((U + 3) / 4);
+    if (cw == 32 && rounds == 1) return narrow_lds_bytes<32, 1>((U + 1) / 2);
+    if (cw == 32 && rounds == 2) return narrow_lds_bytes<32, 2>((U + 3) / 4);
+    return 0;
+}
+
+int hlq_gemv_narrow_launch(const void *gemv_args, size_t args_bytes, int bits, int group, int cw, size_t stage_bytes,
+                           void *stream)
 {
     if (args_bytes != sizeof(GemvArgs)) return ELUTQ_ERR_HIP;
     const GemvArgs &a = *(const GemvArgs *)gemv_args;
-    if (a.extra || a.defer || a.n_slices_in) return ELUTQ_ERR_TUNING;      // the wide-tile kernel's
+    if (a.extra || a.defer) return ELUTQ_ERR_TUNING;      // the wide-tile kernel's
     const bool g64 = group == 64;
     hipStream_t st = (hipStream_t)stream;
     switch (bits) {
-    case 1: return g64 ? launch_narrow<1, true>(a, cw, st) : launch_narrow<1, false>(a, cw, st);
-    case 2: return g64 ? launch_narrow<2, true>(a, cw, st) : launch_narrow<2, false>(a, cw, st);
-    case 3: return g64 ? launch_narrow<3, true>(a, cw, st) : launch_narrow<3, false>(a, cw, st);
-    case 4: return g64 ? launch_narrow<4, true>(a, cw, st) : launch_narrow<4, false>(a, cw, st);
+    case 1: return g64 ? launch_narrow<1, true>(a, cw, stage_bytes, st) : launch_narrow<1, false>(a, cw, stage_bytes, st);
+    case 2: return g64 ? launch_narrow<2, true>(a, cw, stage_bytes, st) : launch_narrow<2, false>(a, cw, stage_bytes, st);
+    case 3: return g64 ? launch_narrow<3, true>(a, cw, stage_bytes, st) : launch_narrow<3, false>(a, cw, stage_bytes, st);
+    case 4: return g64 ? launch_narrow<4, true>(a, cw, stage_bytes, st) : launch_narrow<4, false>(a, cw, stage_bytes, st);
     }
     return ELUTQ_ERR_BITS;
 }

@@ -31,8 +31,12 @@ HLQ_INTERNAL size_t hlq_gemv_mfma_lds_bytes(int ups, int waves);
 
 // The narrow-tile LUT GEMV kernel (hlq_gemv_narrow.hip): a workgroup owns `cw` = 16 or 32 columns over all of K,
 // no K slices.  hlq_gemv_narrow_rounds: units per unit lane of a wave for a layer of U = K / 128 units, 0 where the
-// kernel has no instance for it (its tables of all of K must fit the LDS of one workgroup).  The launch takes
-// the launcher's argument block like hlq_gemv_mfma_launch; prologues, bias and residual as the wide-tile
-// kernel, no extra term and no handed-over slices (ELUTQ_ERR_TUNING).
+// kernel has no instance for it (its tables of all of K must fit the LDS of one workgroup);
+// hlq_gemv_narrow_lds_bytes: dynamic LDS of a launch without staged activations (0: no instance).  The launch
+// takes the launcher's argument block like hlq_gemv_mfma_launch; prologues, bias, residual and handed-over
+// slices (n_slices_in, with `stage_bytes` = 2 K) as the wide-tile kernel, no extra term and no slices left
+// to the next launch (ELUTQ_ERR_TUNING).
 HLQ_INTERNAL int hlq_gemv_narrow_rounds(int U, int cw);
-HLQ_INTERNAL int hlq_gemv_narrow_launch(const void *gemv_args, size_t args_bytes, int bits, int group, int cw, void *stream);
+HLQ_INTERNAL size_t hlq_gemv_narrow_lds_bytes(int U, int cw);
+HLQ_INTERNAL int hlq_gemv_narrow_launch(const void *gemv_args, size_t args_bytes, int bits, int group, int cw,
+                                        size_t stage_bytes, void *stream);

@@ -19,6 +19,7 @@ concatenation of the packed buffers.
 """
 from __future__ import annotations
 
+import os
 import time
 from dataclasses import dataclass
 
@@ -289,9 +290,11 @@ class LlamaDecoder(nn.Module):
     """Random-init LLaMA-shaped decoder for the decode benchmark and its parity test."""
 
     def __init__(self, s: LlamaShape, device="cuda", seed: int = 0, fuse: bool = True, impl: str = "hip",
-                 parts: dict | None = None):
+                 parts: dict | None = None, qkv_to_attention: bool = True):
         """impl "hip": five fused launches per layer through the C ABI (needs fuse=True);
-        impl "torch": the same step with PyTorch ops around plain HLQLinear calls."""
+        impl "torch": the same step with PyTorch ops around plain HLQLinear calls.
+        qkv_to_attention: run q|k|v in two K slices that the attention launch sums (head_dim 128) rather than
+        on the narrow-tile kernel (measured on MI355X at the LLaMA-3-8B shape: 835 against 817 tokens/s)."""
         super().__init__()
         assert impl in ("hip", "torch") and (fuse or impl == "torch")
         self.s = s
@@ -320,7 +323,7 @@ class LlamaDecoder(nn.Module):
         # leave the K slices of down to the launch that reads them (deferred_layer_step); the
         # logits are bit for bit those of fused_layer_step.  Set before capture().
         self.defer_slices = True
-        self.defer_qkv = True              # likewise q|k|v -> attention (takes effect where q|k|v is K-sliced)
+        self.defer_qkv = False             # likewise q|k|v -> attention (set by the constructor, see qkv_to_attention)
         if impl == "hip":
             if any(m.sparse_count for m in self.modules() if isinstance(m, HLQLinear)):
                 raise NotImplementedError("the fused decode step takes no sparse extra plane held as blocks: load the "
@@ -332,23 +335,25 @@ class LlamaDecoder(nn.Module):
             # q|k|v in two K slices where that still leaves at most one workgroup per compute unit: the
             # attention launch sums the slices of its own head for free, so the projection gets twice
             # the workgroups without the meeting that otherwise makes the split a loss
-            # (LLaMA-3-8B: 96 -> 192 workgroups, 6.7 -> 5.7 us)
-            for layer in self.layers:
-                q = layer.qkv
-                if d == 128 and q.bias is None and q.slices == 1 and 2 * ((q.out_features + 63) // 64) <= 256:
-                    q.ksplit, q.waves = 2, 16
+            # (LLaMA-3-8B: 96 -> 192 workgroups, 6.7 -> 5.7 us).  The alternative: narrow tiles (two
+            # workgroups per column block, all of K each), nothing for the attention to sum.
+            self.defer_qkv = bool(qkv_to_attention) and d == 128
+            if self.defer_qkv:
+                for layer in self.layers:
+                    q = layer.qkv
+                    if q.bias is None and q.slices == 1 and 2 * ((q.out_features + 63) // 64) <= 256:
+                        q.ksplit, q.waves = 2, 16
+                    elif q.ksplit == 0:
+                        q.ksplit = _lib.GEMV_WIDE        # a launch that leaves K slices runs on the wide-tile kernel
             # down leaves its K slices unsummed only where the next layer's q|k|v launch takes them (a q|k|v
             # with more tiles than compute units, or tables that leave no room for the staged activations,
             # does not): decided here, once, so that a step never meets a refusing launch
             self._defer_down = [i + 1 < len(self.layers) and 2 <= layer.down_proj.slices <= MAX_DEFERRED_SLICES
                                 and self.layers[i + 1].qkv.accepts_slices(layer.down_proj.slices)
                                 for i, layer in enumerate(self.layers)]
-            # a launch that takes or leaves K slices runs on the wide-tile kernel; a q|k|v that may do either is
-            # pinned to it, so that the step computes the same bits whether or not the slices are handed over
+            # a launch that leaves its K slices to the next one runs on the wide-tile kernel: a down that may do so
+            # is pinned to it, so that the step computes the same bits whether or not the slices are handed over
             for i, layer in enumerate(self.layers):
-                q = layer.qkv
-                if q.ksplit == 0 and ((i > 0 and self._defer_down[i - 1]) or (d == 128 and q.bias is None and q.slices >= 2)):
-                    q.ksplit = _lib.GEMV_WIDE
                 if self._defer_down[i] and layer.down_proj.ksplit == 0:
                     layer.down_proj.ksplit = _lib.GEMV_WIDE
 

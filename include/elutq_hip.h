@@ -146,7 +146,7 @@ int elutq_hlq_gemv_f16_static(const void *d_planes, const void *d_scales, const 
  * without K slices; K <= 8192, else ELUTQ_ERR_TUNING.  With ksplit = waves = 0 the library takes it
  * where the layer has at most 64 / 128 column blocks of 64; ksplit = ELUTQ_GEMV_WIDE keeps it on the
  * wide-tile kernel (64 columns per wavefront) with the library's own K slicing -- the kernel a call with
- * handed-over slices (elutq_gemv_fusion) or an extra term always runs on.
+ * slices to hand over (elutq_gemv_fusion.d_slices_out) or an extra term always runs on.
  */
 #define ELUTQ_GEMV_NARROW16 (-16)
 #define ELUTQ_GEMV_NARROW32 (-32)
@@ -180,7 +180,8 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
  *             the producer would have written with d_residual = d_x, bit for bit; the RMSNorm
  *             follows.  d_x_out (fp16 [K], or NULL; not d_x) receives that x for later readers.
  *             The consuming launch must have at most one tile per compute unit
- *             (ceil(N/64) * slices <= 256); wider projections return ELUTQ_ERR_TUNING.
+ *             (ceil(N/64) * slices <= 256 on the wide-tile kernel; the narrow-tile kernel always has);
+ *             wider projections return ELUTQ_ERR_TUNING.
  * No counterpart in the reference, whose operators run one after the other on whole vectors.
  */
 typedef struct elutq_gemv_fusion {

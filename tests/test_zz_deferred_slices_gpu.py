@@ -21,11 +21,13 @@ def build(k, n, seed, dev, bits=2, group=128):
 @pytest.mark.parametrize("ffn,hidden,n_next,bits,group", [(1024, 512, 768, 2, 128), (14336, 4096, 6144, 2, 128),
                                                           (1024, 512, 768, 3, 64), (1024, 512, 768, 4, 128),
                                                           (2048, 1024, 1536, 2, 64)])
-def test_consumer_sees_what_the_producer_would_have_written(cuda, ffn, hidden, n_next, bits, group):
+@pytest.mark.parametrize("consumer", [_lib.GEMV_WIDE, 0, _lib.GEMV_NARROW32])
+def test_consumer_sees_what_the_producer_would_have_written(cuda, ffn, hidden, n_next, bits, group, consumer):
     """down (SiLU*up prologue, K slices) -> next q|k|v (RMSNorm prologue), at the shapes of the small test
-    model and of LLaMA-3-8B, and at the other plane counts / group size."""
+    model and of LLaMA-3-8B, and at the other plane counts / group size; the consumer on the wide-tile kernel,
+    on the library's choice (narrow tiles at these widths) and on 32-column tiles."""
     down, qkv = build(ffn, hidden, 1, cuda, bits, group), build(hidden, n_next, 2, cuda, bits, group)
-    qkv.ksplit = _lib.GEMV_WIDE          # the kernel a launch with handed-over slices runs on, for the reference too
+    qkv.ksplit = consumer                # the reference call below runs on the same kernel
     S = down.slices
     assert 2 <= S <= 4
     g = torch.Generator(device=cuda).manual_seed(3)
