@@ -186,46 +186,24 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
             }
             return;
         }
-        // Slices meet through device memory.  Partial sums are written and read with
-        // agent-scope atomics (they bypass the per-XCD L2s' non-coherent lines), the writer
-        // waits for its stores to be acknowledged before it takes a ticket, and the reader's
-        // loads depend on the ticket it drew -- so no cache write-back / invalidate is needed.
         const size_t npad = (size_t)a.ncb * HLQ_CB;
         if (!PLAIN && a.defer) {
             // the consumer is a later launch on the same stream: an ordinary store, no meeting
             if (wave == fin) a.partial[(size_t)slice * npad + n] = total;
             return;
         }
+        // the slices meet through device memory (slices_meet): all but the last store and leave
         if (wave == fin) {
-            __hip_atomic_store(&a.partial[(size_t)slice * npad + n], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            float sum;
             HLQ_STAMP(5);
-            unsigned ticket = 0;
-            if (lane == 0)
-                ticket = __hip_atomic_fetch_add(&a.counters[cbf], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            ticket = __builtin_amdgcn_readfirstlane(ticket);
-            HLQ_STAMP(6);
-            if (ticket == (unsigned)a.ksplit - 1u) {
-                // eight independent loads in flight at a time, summed in slice order
-                float sum = 0.f;
-                for (int s0 = 0; s0 < a.ksplit; s0 += 8) {
-                    float v[8];
-#pragma unroll
-                    for (int j = 0; j < 8; j++) {
-                        const int sl = min(s0 + j, a.ksplit - 1);
-                        v[j] = __hip_atomic_load(&a.partial[(size_t)sl * npad + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
-#pragma unroll
-                    for (int j = 0; j < 8; j++)
-                        if (s0 + j < a.ksplit) sum += v[j];
-                }
+            if (slices_meet(a, cbf, slice, npad, n, lane, total, sum)) {
+                HLQ_STAMP(6);
                 if (n < a.N) {
                     if (a.bias) sum += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
                     if (residual) sum += (float)__builtin_bit_cast(_Float16, MULTI ? residual[n] : pre_res);
                     if (extra) sum += extra[n];
                     a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
                 }
-                if (lane == 0) __hip_atomic_store(&a.counters[cbf], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 HLQ_STAMP(7);
             }
         }
@@ -691,7 +669,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     a.ksplit = ksplit; a.ups = ups;
     const WavePlan wp = wave_plan(ups, bits, waves);
     a.spw = wp.spw; a.nuw_max = wp.nuw_max; a.wave_lds = wp.wave_lds;
-    a.partial = nullptr; a.counters = nullptr;
+    a.partial = nullptr; a.counters = nullptr; a.meet_slots = 0;
     a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
     a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr;
     if (fusion) {
@@ -728,8 +706,15 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         if ((size_t)g.ncb * sizeof(unsigned) > (size_t)WS_COUNTER_BYTES) return ELUTQ_ERR_SHAPE;
         if (workspace_bytes < (size_t)WS_COUNTER_BYTES + (size_t)ksplit * g.ncb * HLQ_CB * sizeof(float))
             return ELUTQ_ERR_WORKSPACE;
-        a.counters = (HLQ_GLOBAL unsigned *)d_workspace;
-        a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
+        // slots that fit the head of the workspace, which every kernel leaves zero-filled, are filled and emptied
+        // instead of counted (slices_meet_slots); else arrival counters there and the partial sums behind it
+        if ((size_t)(ksplit - 1) * g.ncb * HLQ_CB * sizeof(float) <= (size_t)WS_COUNTER_BYTES) {
+            a.meet_slots = 1;
+            a.partial = (HLQ_GLOBAL float *)d_workspace;
+        } else {
+            a.counters = (HLQ_GLOBAL unsigned *)d_workspace;
+            a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
+        }
     }
     if (sh.narrow) return hlq_gemv_narrow_launch(&a, sizeof(a), bits, group, sh.narrow, stage_bytes, stream);
     if (sh.mfma) return hlq_gemv_mfma_launch(&a, sizeof(a), bits, group, waves, stage_bytes, stream);
@@ -877,9 +862,11 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
         a.N = problems[i].N; a.U = sh.g.U; a.NT = sh.g.NT; a.ncb = sh.g.ncb;
         a.ksplit = sh.ksplit; a.ups = sh.ups;
         a.spw = sh.wp.spw; a.nuw_max = sh.wp.nuw_max; a.wave_lds = sh.wp.wave_lds;
-        a.partial = nullptr; a.counters = nullptr;
+        a.partial = nullptr; a.counters = nullptr; a.meet_slots = 0;
         if (sh.ksplit > 1) {
-            a.counters = (HLQ_GLOBAL unsigned *)((unsigned char *)d_workspace + coff[i]);
+            // the group's workspace is its own (bound when the plan is made, zero-filled once): the slices fill and
+            // empty their slots, no counters
+            a.meet_slots = 1;
             a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + poff[i]);
         }
         a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;

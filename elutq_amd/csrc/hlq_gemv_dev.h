@@ -35,7 +35,9 @@ struct GemvArgs {
     const HLQ_GLOBAL uint16_t *x;       // fp16 [K]
     HLQ_GLOBAL uint16_t *y;             // fp16 [N]
     HLQ_GLOBAL float *partial;          // [ksplit][ncb*64]   (ksplit > 1)
-    HLQ_GLOBAL unsigned *counters;      // [ncb], zero between calls
+    HLQ_GLOBAL unsigned *counters;      // [ncb], zero between calls (meet_slots == 0)
+    int meet_slots;                     // 1: `partial` [ksplit - 1][ncb*64] is all-zero bits between calls and the slices
+                                        // meet by filling and emptying it (slices_meet); 0: arrival counters
     int N, U, NT, ncb;
     int ksplit, ups;         // slices per column block, units per slice
     int spw;                 // sub-tasks per wave (contiguous run)
@@ -328,6 +330,91 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// The K slices of a column block meet in device memory without an arrival counter.  A slot of `partial`
+// holds all-zero bits while it is empty (the workspace starts zero-filled); a slice stores its sum with an
+// agent-scope store (+0.0 goes in as -0.0, which adds the same) and leaves.  The workgroup of the last slice
+// keeps its own sum in registers, reads the other slots until none is empty, adds them in slice order and puts
+// the zeros back.  One trip through memory lies between the last store and the result (the counter needed
+// three dependent ones: store acknowledged, ticket drawn, slots read).  Who waits is fixed, so it must be
+// certain that the others run: the last slice has the highest workgroup index of its column block (slices
+// are the fastest grid dimension, and later entries of a grouped launch's tile list), hence every slice it
+// waits for was dispatched before it.  The wait is bounded all the same (SLICE_SPIN_LIMIT reads, about a
+// second): a wave that gives up returns what it has, and the kernel ends.
+constexpr int SLICE_SPIN_LIMIT = 1 << 20;
+
+// Called by one whole wave (lane = column n of the block); true in the wave that holds the complete sum.
+__device__ __forceinline__ bool slices_meet_slots(const GemvArgs &a, int slice, size_t npad, int n, float total, float &sum)
+{
+    HLQ_GLOBAL float *mine = a.partial + (size_t)slice * npad + n;
+    if (slice != a.ksplit - 1) {
+        const float v = __float_as_uint(total) == 0u ? -0.0f : total;
+        __hip_atomic_store(mine, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return false;
+    }
+    sum = 0.f;
+    const int others = a.ksplit - 1;
+    int spins = 0;
+    for (int s0 = 0; s0 < others; s0 += 8) {            // eight independent loads in flight at a time
+        float v[8];
+        for (;;) {
+            bool here = true;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int sl = min(s0 + j, others - 1);
+                v[j] = __hip_atomic_load(&a.partial[(size_t)sl * npad + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                here = here && __float_as_uint(v[j]) != 0u;
+            }
+            if (__all(here) || ++spins > SLICE_SPIN_LIMIT) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (s0 + j < others) {
+                sum += v[j];
+                __hip_atomic_store(&a.partial[(size_t)(s0 + j) * npad + n], 0.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+    }
+    sum += total;
+    return true;
+}
+
+// The same meeting with an arrival counter per column block, for launches whose slots would not fit the
+// zero-kept head of the workspace: partial sums are written and read with agent-scope atomics (they bypass the
+// per-XCD L2s' non-coherent lines), the writer waits for its stores to be acknowledged before it takes a
+// ticket, and the reader's loads depend on the ticket it drew -- so no cache write-back / invalidate is
+// needed.  The last workgroup to arrive sums in slice order.  Nothing waits for another workgroup.
+__device__ __forceinline__ bool slices_meet_ticket(const GemvArgs &a, int cb, int slice, size_t npad, int n, int lane,
+                                                   float total, float &sum)
+{
+    __hip_atomic_store(&a.partial[(size_t)slice * npad + n], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    unsigned ticket = 0;
+    if (lane == 0) ticket = __hip_atomic_fetch_add(&a.counters[cb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ticket = __builtin_amdgcn_readfirstlane(ticket);
+    if (ticket != (unsigned)a.ksplit - 1u) return false;
+    sum = 0.f;
+    for (int s0 = 0; s0 < a.ksplit; s0 += 8) {          // eight independent loads in flight at a time
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int sl = min(s0 + j, a.ksplit - 1);
+            v[j] = __hip_atomic_load(&a.partial[(size_t)sl * npad + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (s0 + j < a.ksplit) sum += v[j];
+    }
+    if (lane == 0) __hip_atomic_store(&a.counters[cb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
+__device__ __forceinline__ bool slices_meet(const GemvArgs &a, int cb, int slice, size_t npad, int n, int lane, float total,
+                                            float &sum)
+{
+    if (a.meet_slots) return slices_meet_slots(a, slice, npad, n, total, sum);
+    return slices_meet_ticket(a, cb, slice, npad, n, lane, total, sum);
 }
 
 // 1 / rms of the whole activation vector for the fused RMSNorm prologue: the workgroup sums

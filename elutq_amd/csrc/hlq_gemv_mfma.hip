@@ -270,31 +270,12 @@ __device__ __forceinline__ void mf_finish(const GemvArgs &a, int cbf, int slice,
         return;
     }
     if (wave == fin) {
-        __hip_atomic_store(&a.partial[(size_t)slice * npad + n], total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        unsigned ticket = 0;
-        if (lane == 0) ticket = __hip_atomic_fetch_add(&a.counters[cbf], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ticket = __builtin_amdgcn_readfirstlane(ticket);
-        if (ticket == (unsigned)a.ksplit - 1u) {
-            float sum = 0.f;
-            for (int s0 = 0; s0 < a.ksplit; s0 += 8) {
-                float v[8];
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    const int sl = min(s0 + j, a.ksplit - 1);
-                    v[j] = __hip_atomic_load(&a.partial[(size_t)sl * npad + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
-#pragma unroll
-                for (int j = 0; j < 8; j++)
-                    if (s0 + j < a.ksplit) sum += v[j];
-            }
-            if (n < a.N) {
-                if (a.bias) sum += (float)__builtin_bit_cast(_Float16, a.bias[n]);
-                if (residual) sum += (float)__builtin_bit_cast(_Float16, residual[n]);
-                if (extra) sum += extra[n];
-                a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
-            }
-            if (lane == 0) __hip_atomic_store(&a.counters[cbf], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        float sum;
+        if (slices_meet(a, cbf, slice, npad, n, lane, total, sum) && n < a.N) {
+            if (a.bias) sum += (float)__builtin_bit_cast(_Float16, a.bias[n]);
+            if (residual) sum += (float)__builtin_bit_cast(_Float16, residual[n]);
+            if (extra) sum += extra[n];
+            a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
         }
     }
 }

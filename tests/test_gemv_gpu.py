@@ -236,3 +236,53 @@ def test_non_finite_activations_reach_the_output(cuda, bad, ksplit, waves):
         ref = w @ x[0].astype(np.float64)
     assert not np.any(np.isfinite(ref))              # every weight of the synthetic layer is non-zero
     assert not np.any(np.isfinite(y.astype(np.float32)))
+
+
+def _tuned(m, x, ws, ksplit, waves):
+    y = torch.empty(1, m.out_features, dtype=torch.float16, device=x.device)
+    rc = _lib.lib().elutq_hlq_gemv_f16_tuned(m.planes.data_ptr(), m.scales.data_ptr(), m.zeros.data_ptr(),
+                                             m.bias.data_ptr() if m.bias is not None else None, x.data_ptr(), y.data_ptr(),
+                                             m.in_features, m.out_features, m.bits, m.group_size, ws.data_ptr(), ws.numel(),
+                                             torch.cuda.current_stream().cuda_stream, ksplit, waves)
+    _lib.check(rc, "elutq_hlq_gemv_f16_tuned")
+    torch.cuda.synchronize()
+    return y
+
+
+@pytest.mark.parametrize("n,ksplit", [(4096, 4), (8192, 4), (8192, 2)])
+def test_k_slices_meet_by_slots_or_by_tickets(cuda, n, ksplit):
+    """The K slices of a column block meet in the zero-kept first 64 KiB of the workspace where their slots fit
+    ((ksplit - 1) * ceil(N/64)*64 floats: 4096 columns x 4 slices, 8192 x 2) and through arrival counters and the
+    partial-sum area behind it where they do not (8192 x 4).  Either way: the oracle's result, the same bits on
+    every call, the head of the workspace all zero afterwards -- also when another kernel has filled the rest
+    of the workspace with its own partial sums in between."""
+    k = 512
+    L = make_layer(k, n, bits=2, group=128, seed=n + ksplit)
+    m = to_mod(L, cuda)
+    x = torch.from_numpy(L.x).to(cuda)
+    ws = torch.zeros(max(m.workspace_bytes, 1 << 22), dtype=torch.uint8, device=cuda)
+    ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, 128)
+    y0 = _tuned(m, x, ws, ksplit, 8)
+    assert O.rel_err(y0.cpu().numpy()[0], ref) <= TOL
+    assert not ws[:65536].any()
+    ws[65536:] = 0x7f                                     # what a GEMM or an attention launch may leave behind
+    for _ in range(3):
+        assert torch.equal(_tuned(m, x, ws, ksplit, 8), y0)
+        assert not ws[:65536].any()
+
+
+@pytest.mark.parametrize("ksplit", [2, 4, 7])
+def test_k_slices_whose_sums_are_zero(cuda, ksplit):
+    """A partial sum of exactly +0.0 has the bits of an empty slot: it is stored as -0.0, which adds the same.
+    x = 0 makes every partial sum zero; the output is the bias alone, at once."""
+    L = make_layer(1024, 192, bits=2, group=128, seed=77, bias=True)
+    m = to_mod(L, cuda)
+    ws = torch.zeros(m.workspace_bytes, dtype=torch.uint8, device=cuda)
+    x = torch.zeros(1, 1024, dtype=torch.float16, device=cuda)
+    for _ in range(2):
+        y = _tuned(m, x, ws, ksplit, 4)
+        assert np.array_equal(y.cpu().numpy()[0], L.bias)
+        assert not ws[:65536].any()
+    xr = torch.from_numpy(L.x).to(cuda)                   # and the slots are usable afterwards
+    ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, 128, L.bias)
+    assert O.rel_err(_tuned(m, xr, ws, ksplit, 4).cpu().numpy()[0], ref) <= TOL
