@@ -31,7 +31,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-KERNEL_TRACE_AVG_US = 6.55     # hlq_gemv_kernel<2, false, 4, true, 1> at 4096 x 14336 in the committed kernel trace
+KERNEL_TRACE_AVG_US = 6.41     # hlq_gemv_kernel<2, false, 4, true, 1> at 4096 x 14336 in the committed kernel trace
 BITS, GROUP = 2, 128
 N_LAYERS = 32
 
@@ -54,7 +54,7 @@ def parse():
                         "copy: a plain 64 MiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE; "
                         "decode / gemm: only that leg (for kernel traces); "
                         "decode-eager: three eager decode steps of a two-layer model of the same widths (for counter runs); "
-                        "shape-sweep: the small LLaMA-3-8B shapes at every K split x wave count of the tuned entry point; "
+                        "shape-sweep: the small LLaMA-3-8B shapes at every kernel, K split and wave count of the tuned entry point; "
                         "sparse: GEMVs of layers with a block-sparse extra plane beside the same layers without it")
     p.add_argument("--launches", type=int, default=256, help="launches in --mode kernel / copy")
     return p.parse_args()
@@ -386,10 +386,14 @@ def main():
             y = torch.empty(1, n, dtype=torch.float16, device=dev)
             ws = torch.zeros(max(lib.elutq_hlq_workspace_bytes(k, n, BITS, GROUP, 1), 1 << 22), dtype=torch.uint8, device=dev)
             rows = []
+            named = {_lib.GEMV_NARROW16: "narrow tiles, 16 columns", _lib.GEMV_NARROW32: "narrow tiles, 32 columns",
+                     _lib.GEMV_WIDE: "wide tiles, the library's K split"}
             for eng in ("lut", "mfma"):
                 _lib.set_gemv_engine(eng)
-                for ks in (0, 1, 2, 4, 8, 16):
+                for ks in (0, _lib.GEMV_NARROW16, _lib.GEMV_NARROW32, _lib.GEMV_WIDE, 1, 2, 4, 8, 16):
                     for wv in (0, 4, 8, 16):
+                        if ks < 0 and (wv or (eng == "mfma" and ks != _lib.GEMV_WIDE)):
+                            continue
                         slices = lib.elutq_hlq_gemv_slices(k, n, BITS, GROUP, ks, wv)
                         if slices == 0:
                             continue
@@ -403,8 +407,10 @@ def main():
                                     raise RuntimeError(f"elutq_hlq_gemv_f16_tuned: {rc}")
 
                         us = time_graph(torch, launch, 10, 2) / len(ring) * 1e6
-                        rows.append({"engine": eng, "ksplit": ks, "waves": wv, "slices": slices,
-                                     "workgroups": slices * ((n + 63) // 64), "us": round(us, 3)})
+                        ncb = (n + 63) // 64
+                        wgs = ncb * 4 if ks == _lib.GEMV_NARROW16 else ncb * 2 if ks == _lib.GEMV_NARROW32 else slices * ncb
+                        rows.append({"engine": eng, "ksplit": named.get(ks, ks), "waves": wv, "slices": slices,
+                                     "workgroups": wgs, "us": round(us, 3)})
             _lib.set_gemv_engine("auto")
             table[f"{k}x{n}"] = {"bytes": nbytes, "byte_floor_us_at_8TBps": nbytes / 8e6, "rows": rows}
             del ring

@@ -30,7 +30,9 @@
  *   - every function returns ELUTQ_OK (0) or a negative elutq_status; nothing throws;
  *   - a workspace is private to one in-flight call: calls that share a workspace
  *     must be ordered on one stream.  It must be zero-filled once after allocation
- *     (elutq_hlq_workspace_init); the kernels leave it zeroed where that matters.
+ *     (elutq_hlq_workspace_init).  Its first 64 KiB are zero between calls -- arrival counters and the
+ *     slots in which the K slices of a GEMV meet live there, and every kernel puts the zeros back --
+ *     so nothing else may write into a workspace; what lies behind the 64 KiB may hold anything.
  */
 #ifndef ELUTQ_HIP_H
 #define ELUTQ_HIP_H
@@ -223,7 +225,8 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
  * A plan holds the device-side problem list: create it once (allocates and copies; not
  * capturable), run it any number of times (one kernel launch, capturable), destroy it.
  * The workspace (elutq_hlq_gemv_group_workspace_bytes, zero-filled once) is bound at creation
- * and must not be shared with calls that may run concurrently.  Results equal those of
+ * and belongs to the plan until it is destroyed: no other call may use it (the K slices of the
+ * group's GEMVs meet in slots that are zero between runs).  Results equal those of
  * elutq_hlq_gemv_f16_tuned with the same K slicing, which the group chooses itself.
  */
 typedef struct elutq_gemv_problem {
