@@ -864,9 +864,10 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
         a.spw = sh.wp.spw; a.nuw_max = sh.wp.nuw_max; a.wave_lds = sh.wp.wave_lds;
         a.partial = nullptr; a.counters = nullptr; a.meet_slots = 0;
         if (sh.ksplit > 1) {
-            // the group's workspace is its own (bound when the plan is made, zero-filled once): the slices fill and
-            // empty their slots, no counters
-            a.meet_slots = 1;
+            // Arrival counters, not slots: in this launch a workgroup walks a list of tiles, so the workgroup a
+            // waiting one depends on can have a higher index -- and if two such launches share the GPU, neither
+            // need be resident in full.  With counters nothing ever waits for another workgroup.
+            a.counters = (HLQ_GLOBAL unsigned *)((unsigned char *)d_workspace + coff[i]);
             a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + poff[i]);
         }
         a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;

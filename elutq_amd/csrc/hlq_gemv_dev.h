@@ -339,9 +339,12 @@ __device__ __forceinline__ void lds_barrier()
 // the zeros back.  One trip through memory lies between the last store and the result (the counter needed
 // three dependent ones: store acknowledged, ticket drawn, slots read).  Who waits is fixed, so it must be
 // certain that the others run: the last slice has the highest workgroup index of its column block (slices
-// are the fastest grid dimension, and later entries of a grouped launch's tile list), hence every slice it
-// waits for was dispatched before it.  The wait is bounded all the same (SLICE_SPIN_LIMIT reads, about a
-// second): a wave that gives up returns what it has, and the kernel ends.
+// are the fastest grid dimension), and a dispatcher places workgroups in index order.  Take the lowest-indexed
+// workgroup still waiting for a place: every workgroup that holds a place ahead of it waits, if at all, for
+// ones with lower indices still -- which therefore hold their places or are done -- so places keep coming
+// free, whatever else shares the GPU.  (A launch whose workgroups walk a list of tiles cannot promise that
+// and keeps the counters.)  The wait is bounded all the same (SLICE_SPIN_LIMIT reads, about a second): a
+// wave that gives up returns what it has, and the kernel ends.
 constexpr int SLICE_SPIN_LIMIT = 1 << 20;
 
 // Called by one whole wave (lane = column n of the block); true in the wave that holds the complete sum.
@@ -381,7 +384,7 @@ __device__ __forceinline__ bool slices_meet_slots(const GemvArgs &a, int slice, 
 }
 
 // The same meeting with an arrival counter per column block, for launches whose slots would not fit the
-// zero-kept head of the workspace: partial sums are written and read with agent-scope atomics (they bypass the
+// zero-kept head of the workspace and for grouped launches: partial sums are written and read with agent-scope atomics (they bypass the
 // per-XCD L2s' non-coherent lines), the writer waits for its stores to be acknowledged before it takes a
 // ticket, and the reader's loads depend on the ticket it drew -- so no cache write-back / invalidate is
 // needed.  The last workgroup to arrive sums in slice order.  Nothing waits for another workgroup.

@@ -225,8 +225,7 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
  * A plan holds the device-side problem list: create it once (allocates and copies; not
  * capturable), run it any number of times (one kernel launch, capturable), destroy it.
  * The workspace (elutq_hlq_gemv_group_workspace_bytes, zero-filled once) is bound at creation
- * and belongs to the plan until it is destroyed: no other call may use it (the K slices of the
- * group's GEMVs meet in slots that are zero between runs).  Results equal those of
+ * and must not be shared with calls that may run concurrently.  Results equal those of
  * elutq_hlq_gemv_f16_tuned with the same K slicing, which the group chooses itself.
  */
 typedef struct elutq_gemv_problem {
