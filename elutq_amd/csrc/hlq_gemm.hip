@@ -99,7 +99,10 @@ __device__ __forceinline__ void stage_load(StageRegs<MR> &r, const GemmArgs &a, 
     // every round (two instructions per task) instead of being kept in registers for the whole kernel.
     asm volatile("" : "+v"(lane));
     const uint32_t row_bytes = (uint32_t)a.K * 2;
-    const uint32_t col_off = ((uint32_t)u * HLQ_UNIT + half * S::KS + (lane & (S::SLOTS - 1)) * 8) * 2;
+    // where K ends half way through the last unit, the slots of the absent half read the row's last slot and count as zeros
+    const uint32_t kcol = (uint32_t)u * HLQ_UNIT + half * S::KS + (lane & (S::SLOTS - 1)) * 8;
+    const bool absent = kcol >= (uint32_t)a.K;
+    const uint32_t col_off = (absent ? (uint32_t)a.K - 8u : kcol) * 2;
     const uint32_t last = (uint32_t)(a.M - 1) * row_bytes + col_off;         // rows past M read row M - 1 again
     uint32_t off = (uint32_t)(lane / S::SLOTS) * row_bytes + col_off;
 #pragma unroll
@@ -107,6 +110,10 @@ __device__ __forceinline__ void stage_load(StageRegs<MR> &r, const GemmArgs &a, 
         r.v[t] = *(const uint4 *)((const unsigned char *)a.x + (off < last ? off : last));
         off += (64 / S::SLOTS) * row_bytes;
         asm volatile("" : "+v"(off));            // one add per task: keeps the compiler from re-deriving every offset with a multiply
+    }
+    if (absent) {
+#pragma unroll
+        for (int t = 0; t < S::TPT; t++) r.v[t] = make_uint4(0u, 0u, 0u, 0u);
     }
 }
 
@@ -639,10 +646,10 @@ int hlq_gemm_chunk_with_extra(const void *d_planes, const void *d_scales, const 
     if (M < 1 || M > HLQ_GEMM_MAX_M) return ELUTQ_ERR_SHAPE;
     if (bits < 1 || bits > 4) return ELUTQ_ERR_BITS;
     if (group != 64 && group != 128) return ELUTQ_ERR_GROUP;
-    if (K < HLQ_UNIT || N < 1 || K % HLQ_UNIT != 0 || K % group != 0) return ELUTQ_ERR_SHAPE;
+    if (N < 1 || !hlq_k_ok(K, group)) return ELUTQ_ERR_SHAPE;
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
     if (kparts != 0 && kparts != HLQ_GEMM_WAVES) return ELUTQ_ERR_TUNING;
-    if (ksplit < 0 || ksplit > K / HLQ_UNIT) return ELUTQ_ERR_TUNING;
+    if (ksplit < 0 || ksplit > (K + HLQ_UNIT - 1) / HLQ_UNIT) return ELUTQ_ERR_TUNING;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     int ks = ksplit, ups;
     hlq_gemm_shape(g, M, ks, ups);

@@ -96,7 +96,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     // whose run is shorter than NSLOT re-reads its last sub-task), so the number of loads
     // behind the activations is a compile-time constant and the table build waits for the
     // activations only (vmcnt(3 * NSLOT)), with the weights still in flight.
-    const int K = a.U * HLQ_UNIT;
+    const int K = a.K;
     const size_t k0 = (size_t)(u0 + ub) * HLQ_UNIT;
     const int nchunks = nuw * 32;
     float rstd = 1.f;
@@ -118,7 +118,9 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     if (sliced) load_slice_chunk(a, K, min(tid, K / 4 - 1), sfirst);
     uint2 raw, raw2;
     // lanes past the run (and waves without one, whose k0 is the end of the slice) re-read a valid chunk
-    load_chunk<PLAIN>(a, prologue, K, hlq_x_first_k(k0, nchunks, lane), raw, raw2);
+    // (where K ends half way through the last unit, the chunks of the absent half re-read the last one and count as zeros)
+    const size_t kfirst = hlq_x_first_k(k0, nchunks, lane);
+    load_chunk<PLAIN>(a, prologue, K, hlq_x_load_k(kfirst, K), raw, raw2);
     asm volatile("" ::: "memory");      // keep both activation loads ahead of the weight loads
 
     float acc = 0.f;
@@ -133,6 +135,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                           sliced && a.x_out && blockIdx.x == 0 && blockIdx.y == 0);
     // the combined chunk replaces the base's (a wave without a run sits at the end of the slice: clamped)
     if (sliced) raw = stage[hlq_stage_first_index(k0, nchunks, lane, K)];
+    if (kfirst >= (size_t)K) raw = make_uint2(0u, 0u);
 
     // ... the tables are built as soon as the activations are in (a wave that first queued all
     // its weight loads would sit in the memory pipeline's back-pressure instead) ...
@@ -146,8 +149,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         load_slot<BITS, G64, PAIRED, d>(slot[d], here, u0, min(s_begin + d, s_last), lane);
     });
     for (int ci = lane + 64; ci < nchunks; ci += 64) {      // runs of more than two units (not the common case)
-        load_chunk<PLAIN>(a, prologue, K, k0 + (size_t)ci * 4, raw, raw2);
-        if (sliced) raw = stage[(k0 >> 2) + ci];
+        const size_t kc = k0 + (size_t)ci * 4;
+        load_chunk<PLAIN>(a, prologue, K, hlq_x_load_k(kc, K), raw, raw2);
+        if (sliced) raw = stage[hlq_stage_index(k0, ci, K)];
+        if (kc >= (size_t)K) raw = make_uint2(0u, 0u);
         build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0, lane);
     }
     HLQ_STAMP(1);
@@ -491,7 +496,7 @@ int check_shape(int K, int N, int bits, int group)
 {
     if (bits < 1 || bits > 4) return ELUTQ_ERR_BITS;
     if (group != 64 && group != 128) return ELUTQ_ERR_GROUP;
-    if (K < HLQ_UNIT || N < 1 || K % HLQ_UNIT != 0 || K % group != 0) return ELUTQ_ERR_SHAPE;
+    if (N < 1 || !hlq_k_ok(K, group)) return ELUTQ_ERR_SHAPE;
     return ELUTQ_OK;
 }
 
@@ -568,6 +573,7 @@ int plan_launch(const HlqGeo &g, int bits, int ksplit, int waves, bool allow_nar
     // tile per workgroup takes 0.5-1 us longer (its A operands cost more to build than the tables), so the
     // library's own choice is the LUT kernel throughout
     sh.mfma = g_gemv_engine == ELUTQ_GEMV_ENGINE_MFMA;
+    if (sh.mfma && g.K % HLQ_UNIT != 0) return ELUTQ_ERR_TUNING;      // the matrix-core kernel takes whole units only
     choose_shape(g, ksplit, waves);
     int ups = (g.U + ksplit - 1) / ksplit;
     if (sh.mfma) {
@@ -665,7 +671,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     a.bias = (const HLQ_GLOBAL uint16_t *)d_bias;
     a.x = (const HLQ_GLOBAL uint16_t *)d_x;
     a.y = (HLQ_GLOBAL uint16_t *)d_y;
-    a.N = N; a.U = g.U; a.NT = g.NT; a.ncb = g.ncb;
+    a.N = N; a.U = g.U; a.NT = g.NT; a.ncb = g.ncb; a.K = K;
     a.ksplit = ksplit; a.ups = ups;
     const WavePlan wp = wave_plan(ups, bits, waves);
     a.spw = wp.spw; a.nuw_max = wp.nuw_max; a.wave_lds = wp.wave_lds;
@@ -859,7 +865,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
         a.bias = (const HLQ_GLOBAL uint16_t *)problems[i].d_bias;
         a.x = (const HLQ_GLOBAL uint16_t *)problems[i].d_x;
         a.y = (HLQ_GLOBAL uint16_t *)problems[i].d_y;
-        a.N = problems[i].N; a.U = sh.g.U; a.NT = sh.g.NT; a.ncb = sh.g.ncb;
+        a.N = problems[i].N; a.U = sh.g.U; a.NT = sh.g.NT; a.ncb = sh.g.ncb; a.K = problems[i].K;
         a.ksplit = sh.ksplit; a.ups = sh.ups;
         a.spw = sh.wp.spw; a.nuw_max = sh.wp.nuw_max; a.wave_lds = sh.wp.wave_lds;
         a.partial = nullptr; a.counters = nullptr; a.meet_slots = 0;

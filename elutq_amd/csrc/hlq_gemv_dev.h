@@ -39,6 +39,7 @@ struct GemvArgs {
     int meet_slots;                     // 1: `partial` [ksplit - 1][ncb*64] is all-zero bits between calls and the slices
                                         // meet by filling and emptying it (slices_meet); 0: arrival counters
     int N, U, NT, ncb;
+    int K;                   // activations: 128 U, or 64 fewer where K ends half way through the last unit (G = 64)
     int ksplit, ups;         // slices per column block, units per slice
     int spw;                 // sub-tasks per wave (contiguous run)
     int nuw_max, wave_lds;   // units a wave's run can touch, bytes of its LDS region

@@ -99,5 +99,14 @@ HLQ_HD size_t hlq_x_first_k(size_t k0, int nchunks, int lane)
     return nchunks ? k0 + (size_t)(lane < nchunks - 1 ? lane : nchunks - 1) * 4 : 0;
 }
 
+// K may end half way through the last unit (G = 64): the chunks of the absent half are read from the last
+// chunk of x -- and counted as zeros by the caller -- in global memory and in the staged copy alike.
+HLQ_HD size_t hlq_x_load_k(size_t k, int K) { return k < (size_t)(K - 4) ? k : (size_t)(K - 4); }
+HLQ_HD int hlq_stage_index(size_t k0, int ci, int K)
+{
+    const int i = (int)(k0 >> 2) + ci;
+    return i < K / 4 - 1 ? i : K / 4 - 1;
+}
+
 // Row of the handed-over slices a fixed-count load reads for position s (rows past the count re-read the last).
 HLQ_HD int hlq_slice_row(int s, int n_slices_in) { return s < n_slices_in - 1 ? s : n_slices_in - 1; }

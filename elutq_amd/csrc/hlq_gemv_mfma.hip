@@ -295,7 +295,7 @@ __device__ __forceinline__ void mfma_tile(const GemvArgs &a, int cb, int slice, 
     const HLQ_GLOBAL float *extra = VAR == GEMV_EXTRA ? a.extra : nullptr;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int K = a.U * HLQ_UNIT;
+    const int K = a.K;                                                      // (host: whole units only)
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
     const int npairs = (nU + 1) >> 1;
     const int ppw = (npairs + nw - 1) / nw;                                 // <= MAXP (host)

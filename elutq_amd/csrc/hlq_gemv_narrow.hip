@@ -89,7 +89,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int K = a.U * HLQ_UNIT;
+    const int K = a.K;
     const int cb = blockIdx.x / UL, part = blockIdx.x % UL;
     const int col = part * CW + (lane % CW);                    // column inside the column block
     const int ul = lane / CW;                                   // this lane's unit inside a round
@@ -153,6 +153,10 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
 #pragma unroll
         for (int p = 0; p < PASSES; p++) raw[p] = stage[min(ub * 32 + p * 64 + lane, K / 4 - 1)];
     }
+    // chunks past K (the absent half of a last unit, units no wave lane owns) count as zeros
+#pragma unroll
+    for (int p = 0; p < PASSES; p++)
+        if ((ub * 32 + p * 64 + lane) * 4 >= K) raw[p] = make_uint2(0u, 0u);
 
     // the wave's own tables: chunk ci of the wave belongs to unit ci / 32, half unit ci / 16
 #pragma unroll

@@ -4,13 +4,16 @@
 // dwordx4 per lane.  Output columns are tiled in blocks of 64 (one wavefront, lane =
 // column), so a wave-wide dwordx4 load covers one unit of 64 columns = 1 KiB contiguous.
 //
-//   planes  uint4    [ncb][U][bits][64]        U = K/128, ncb = ceil(N/64)
+//   planes  uint4    [ncb][U][bits][64]        U = ceil(K/128), ncb = ceil(N/64)
 //   scales  uint32   [ncb][NT][bits][64]       one dword = fp16 scales of groups 2t, 2t+1
 //   zeros   uint32   [ncb][NT][64]             one dword = fp16 zeros  of groups 2t, 2t+1
 //
 // NT = ceil(NG/2) with NG = K/G groups per column ("task" t = the groups one meta dword
 // covers: two units at G = 128, one unit at G = 64).  Columns >= N and the odd group of
-// an odd NG are zero-filled.
+// an odd NG are zero-filled.  K is a multiple of the group size and at least 128: at G = 64 it may
+// end half way through the last unit (K % 128 == 64, which the reference accepts, arm_gemm.cpp:249);
+// the plane bits of that unit's second half are zero like the scales and zero of its absent group, and
+// the kernels read the activations of that half as zeros.
 //
 // Inside a unit, dword d holds k = 32d .. 32d+31 LSB-first (bit i <-> k = 32d + i, the
 // byte order of the reference's w_quant.bin read as little-endian dwords), rotated left
@@ -40,11 +43,18 @@ struct HlqGeo {
     int ncb;    // column blocks
 };
 
+// K >= 128, a multiple of the group size and -- except for half a unit at G = 64 -- of 128.
+static inline bool hlq_k_ok(int K, int group)
+{
+    if (K < HLQ_UNIT || (group != 64 && group != 128)) return false;
+    return K % HLQ_UNIT == 0 || (group == 64 && K % HLQ_UNIT == 64);
+}
+
 static inline HlqGeo hlq_geo(int K, int N, int bits, int group)
 {
     HlqGeo g;
     g.K = K; g.N = N; g.bits = bits; g.group = group;
-    g.U = K / HLQ_UNIT;
+    g.U = (K + HLQ_UNIT - 1) / HLQ_UNIT;
     g.NG = K / group;
     g.NT = (g.NG + 1) / 2;
     g.UPT = group == 64 ? 1 : 2;

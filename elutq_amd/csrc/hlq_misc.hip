@@ -32,7 +32,8 @@ __global__ __launch_bounds__(64) void hlq_dequant_kernel(const DequantArgs a)
         for (int i = 0; i < 4; i++) bitsw[b][i] = (d[i] >> HLQ_ROT) | (d[i] << (32 - HLQ_ROT));
     }
     uint16_t *dst = a.w + (size_t)n * a.K + (size_t)u * HLQ_UNIT;
-    for (int i = 0; i < HLQ_UNIT; i++) {
+    const int nk = min(HLQ_UNIT, a.K - u * HLQ_UNIT);             // 64 in a last unit that K ends half way through
+    for (int i = 0; i < nk; i++) {
         // group of this k and where its scale sits: task t = g / 2, half = g & 1
         const int g = a.g64 ? 2 * u + (i >> 6) : u;
         const int t = g >> 1, hi = g & 1;
@@ -55,7 +56,7 @@ const char *elutq_status_string(int status)
     switch (status) {
     case ELUTQ_OK: return "ok";
     case ELUTQ_ERR_NULL: return "a required pointer is NULL";
-    case ELUTQ_ERR_SHAPE: return "unsupported shape: need K % 128 == 0, K % group == 0, K >= 128, N >= 1, M >= 1";
+    case ELUTQ_ERR_SHAPE: return "unsupported shape: need K >= 128, K % group == 0 and K % 128 == 0 (or 64 at group 64), N >= 1, M >= 1";
     case ELUTQ_ERR_BITS: return "bits must be 1..4";
     case ELUTQ_ERR_GROUP: return "group must be 64 or 128";
     case ELUTQ_ERR_WORKSPACE: return "workspace smaller than elutq_hlq_workspace_bytes()";
@@ -76,7 +77,7 @@ int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void
 {
     if (bits < 1 || bits > 4) return ELUTQ_ERR_BITS;
     if (group != 64 && group != 128) return ELUTQ_ERR_GROUP;
-    if (K < HLQ_UNIT || N < 1 || K % HLQ_UNIT != 0 || K % group != 0) return ELUTQ_ERR_SHAPE;
+    if (N < 1 || !hlq_k_ok(K, group)) return ELUTQ_ERR_SHAPE;
     if (!d_planes || !d_scales || !d_zeros || !d_w_out) return ELUTQ_ERR_NULL;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     DequantArgs a;

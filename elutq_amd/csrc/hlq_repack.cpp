@@ -17,7 +17,7 @@ int check_shape(int K, int N, int bits, int group)
 {
     if (bits < 1 || bits > 4) return ELUTQ_ERR_BITS;
     if (group != 64 && group != 128) return ELUTQ_ERR_GROUP;
-    if (K < HLQ_UNIT || N < 1 || K % HLQ_UNIT != 0 || K % group != 0) return ELUTQ_ERR_SHAPE;
+    if (N < 1 || !hlq_k_ok(K, group)) return ELUTQ_ERR_SHAPE;
     return ELUTQ_OK;
 }
 
@@ -27,8 +27,8 @@ extern "C" {
 
 size_t elutq_hlq_planes_bytes(int K, int N, int bits)
 {
-    if (check_shape(K, N, bits, 128) != ELUTQ_OK) return 0;
-    return hlq_planes_bytes(hlq_geo(K, N, bits, 128));
+    if (check_shape(K, N, bits, 64) != ELUTQ_OK) return 0;      // (the size does not depend on the group size)
+    return hlq_planes_bytes(hlq_geo(K, N, bits, 64));
 }
 
 size_t elutq_hlq_scales_bytes(int K, int N, int bits, int group)
@@ -64,7 +64,8 @@ int elutq_hlq_repack_host(const uint8_t *w_quant, const uint16_t *w_scale, const
                     const int n = cb * HLQ_CB + lane;
                     uint32_t d[4] = {0, 0, 0, 0};
                     if (n < N) {
-                        memcpy(d, w_quant + ((size_t)b * N + n) * row_bytes + (size_t)u * 16, 16);
+                        const size_t have = row_bytes - (size_t)u * 16;          // 8 in a last unit that K ends half way through
+                        memcpy(d, w_quant + ((size_t)b * N + n) * row_bytes + (size_t)u * 16, have < 16 ? have : 16);
                         for (int i = 0; i < 4; i++) d[i] = rotl32(d[i], HLQ_ROT);
                     }
                     memcpy(dst + lane * 4, d, 16);
@@ -120,7 +121,8 @@ int elutq_hlq_unpack_host(const void *planes_in, const void *scales_in, const vo
                 uint32_t d[4];
                 memcpy(d, planes + ((((size_t)cb * g.U + u) * bits + b) * HLQ_CB + lane) * 4, 16);
                 for (int i = 0; i < 4; i++) d[i] = rotr32(d[i], HLQ_ROT);
-                memcpy(w_quant_out + ((size_t)b * N + n) * row_bytes + (size_t)u * 16, d, 16);
+                const size_t have = row_bytes - (size_t)u * 16;
+                memcpy(w_quant_out + ((size_t)b * N + n) * row_bytes + (size_t)u * 16, d, have < 16 ? have : 16);
             }
             for (int gi = 0; gi < g.NG; gi++) {
                 uint32_t v = scales[(((size_t)cb * g.NT + gi / 2) * bits + b) * HLQ_CB + lane];

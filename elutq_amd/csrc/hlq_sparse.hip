@@ -151,7 +151,7 @@ __global__ __launch_bounds__(SP_THREADS) void hlq_sparse_dequant_kernel(const Sp
 int check_sparse_call(int K, int N, int group, int nblk)
 {
     if (group != 64 && group != 128) return ELUTQ_ERR_GROUP;
-    if (K < HLQ_UNIT || N < 1 || K % HLQ_UNIT != 0 || K % group != 0 || nblk < 0) return ELUTQ_ERR_SHAPE;
+    if (N < 1 || !hlq_k_ok(K, group) || nblk < 0) return ELUTQ_ERR_SHAPE;
     return ELUTQ_OK;
 }
 

@@ -51,7 +51,7 @@ def repack_export_arrays(w_quant, w_scale, w_zero, group: int):
     zeros = np.empty(L.elutq_hlq_zeros_bytes(k, n, group), dtype=np.uint8)
     if planes.size == 0 or scales.size == 0:
         raise ValueError(f"unsupported HLQ shape K={k} N={n} bits={bits} group={group} "
-                         "(need K % 128 == 0, bits 1..4, group 64 or 128)")
+                         "(need K a multiple of 128 -- or of 64 at group 64 --, bits 1..4, group 64 or 128)")
     vp = ctypes.c_void_p
     _lib.check(L.elutq_hlq_repack_host(w_quant.ctypes.data_as(vp), w_scale.ctypes.data_as(vp),
                                        w_zero.ctypes.data_as(vp), k, n, bits, group,
@@ -122,7 +122,7 @@ class HLQLinear(nn.Module):
                                                               self.bits, self.group_size, 1)
         if self._ws_bytes == 0:
             raise ValueError(f"unsupported HLQ shape K={in_features} N={out_features} bits={bits} "
-                             f"group={group_size} (need K % 128 == 0, bits 1..4, group 64 or 128)")
+                             f"group={group_size} (need K a multiple of 128 -- or of 64 at group 64 --, bits 1..4, group 64 or 128)")
         self._ws_cache: dict = {}
         self.ksplit, self.waves = 0, 0      # 0 = library default; set for tuning
 

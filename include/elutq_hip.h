@@ -47,7 +47,7 @@ extern "C" {
 typedef enum elutq_status {
     ELUTQ_OK = 0,
     ELUTQ_ERR_NULL = -1,       /* a required pointer is NULL */
-    ELUTQ_ERR_SHAPE = -2,      /* K % 128 != 0, K % group != 0, K, N or M < 1 */
+    ELUTQ_ERR_SHAPE = -2,      /* K < 128, K % group != 0, K % 128 != 0 (at group 64: K % 128 == 64 is accepted), N or M < 1 */
     ELUTQ_ERR_BITS = -3,       /* bits outside 1..4 */
     ELUTQ_ERR_GROUP = -4,      /* group not 64 or 128 */
     ELUTQ_ERR_WORKSPACE = -5,  /* workspace smaller than elutq_hlq_workspace_bytes() */

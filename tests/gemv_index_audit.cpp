@@ -38,9 +38,10 @@ void check(bool ok, const char *what, int bits, int g64, int waves, int U, int u
 
 // One launch shape: U units of K, ncb column blocks, slices of `ups` units, `waves` waves per workgroup,
 // n_slices_in handed-over slices (0 = none), MULTI = the instances that walk runs of column blocks.
-void audit(int bits, bool g64, int waves, int U, int ups, int ncb, int n_slices_in, bool multi, bool clamp_stage)
+// `ragged`: K ends half way through the last unit (G = 64 only).
+void audit(int bits, bool g64, int waves, int U, int ups, int ncb, int n_slices_in, bool multi, bool clamp_stage, bool ragged)
 {
-    const int K = U * UNIT;
+    const int K = U * UNIT - (ragged ? UNIT / 2 : 0);
     const HlqWavePlan wp = hlq_wave_plan(ups, bits, waves);
     const size_t lds_alloc = hlq_gemv_lds_bytes(ups, bits, waves) + (n_slices_in ? (size_t)K * 2 : 0);
     if (lds_alloc > (size_t)MAX_LDS) return;                       // the launcher halves the slice or refuses
@@ -48,7 +49,7 @@ void audit(int bits, bool g64, int waves, int U, int ups, int ncb, int n_slices_
     if (multi && (wp.spw > nslot || waves != 16)) return;          // the condition of the run kernels
     const int ksplit = (U + ups - 1) / ups;
     const HlqLdsMap lm = hlq_lds_map(waves, wp.wave_lds);
-    const int NT = ((g64 ? 2 * U : U) + 1) / 2;
+    const int NT = ((g64 ? K / 64 : U) + 1) / 2;
     const size_t planes_bytes = (size_t)ncb * U * bits * CB * 16;
     const size_t scale_bytes = (size_t)ncb * NT * bits * CB * 4, zero_bytes = (size_t)ncb * NT * CB * 4;
     const size_t npad = (size_t)ncb * CB;
@@ -65,11 +66,11 @@ void audit(int bits, bool g64, int waves, int U, int ups, int ncb, int n_slices_
             for (int ci = 0; ci < nchunks; ci++) {
                 CHECK(lut + (uint32_t)ci * 64 + 64 <= xs, "lds-table");
                 CHECK(xs + (uint32_t)(ci >> 4) * 8 + 8 <= lut + (uint32_t)wp.wave_lds, "lds-half");
-                CHECK(k0 + (size_t)ci * 4 + 4 <= (size_t)K, "x");
-                if (n_slices_in && ci >= 64) CHECK(lm.stage + ((uint32_t)(k0 >> 2) + ci) * 8 + 8 <= lds_alloc, "lds-stage");
+                CHECK(hlq_x_load_k(k0 + (size_t)ci * 4, K) + 4 <= (size_t)K, "x");
+                if (n_slices_in && ci >= 64) CHECK(lm.stage + (uint32_t)hlq_stage_index(k0, ci, K) * 8 + 8 <= lm.stage + (uint32_t)K * 2, "lds-stage");
             }
             for (int lane = 0; lane < 64; lane++) {
-                CHECK(hlq_x_first_k(k0, nchunks, lane) + 4 <= (size_t)K, "x");
+                CHECK(hlq_x_load_k(hlq_x_first_k(k0, nchunks, lane), K) + 4 <= (size_t)K, "x");
                 if (n_slices_in) {
                     const int i = hlq_stage_first_index(k0, nchunks, lane, K, clamp_stage);
                     CHECK(i >= 0 && lm.stage + (uint32_t)i * 8 + 8 <= lds_alloc, "lds-stage");
@@ -130,8 +131,10 @@ int main(int argc, char **argv)
                     for (int ups = 1; ups <= U; ups++)
                         for (int nsl = 0; nsl <= HLQ_GEMV_MAX_SLICES_IN; nsl++)
                             for (int multi = 0; multi < 2; multi++) {
-                                audit(bits, g64 != 0, waves, U, ups, multi ? 448 : 3, nsl, multi != 0, clamp_stage);
-                                shapes++;
+                                for (int ragged = 0; ragged <= (g64 && U > 1 ? 1 : 0); ragged++) {
+                                    audit(bits, g64 != 0, waves, U, ups, multi ? 448 : 3, nsl, multi != 0, clamp_stage, ragged != 0);
+                                    shapes++;
+                                }
                             }
     long total = 0;
     for (auto &kv : g_viol) {

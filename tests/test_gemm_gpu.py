@@ -26,7 +26,7 @@ def gemm(L, dev, x=None):
 
 @pytest.mark.parametrize("m", [2, 5, 16, 31, 32, 33, 64, 70, 130])
 @pytest.mark.parametrize("k,n,bits,group", [(512, 128, 2, 128), (1024, 192, 3, 128), (640, 100, 2, 64),
-                                             (384, 64, 4, 64), (2048, 64, 1, 128)])
+                                             (384, 64, 4, 64), (2048, 64, 1, 128), (1216, 100, 2, 64), (192, 64, 3, 64)])
 def test_gemm_matches_oracle(cuda, m, k, n, bits, group):
     L = make_layer(k, n, bits=bits, group=group, m=m, seed=m + k + bits, bias=(bits == 3))
     _, y = gemm(L, cuda)
@@ -34,6 +34,20 @@ def test_gemm_matches_oracle(cuda, m, k, n, bits, group):
     assert y.shape == (m, n) and y.dtype == np.float16
     assert O.rel_err(y, ref) <= TOL
     assert np.max(np.abs(y.astype(np.float64) - ref)) <= 2.0 ** -9 * max(1.0, np.max(np.abs(ref)))
+
+
+@pytest.mark.parametrize("m", [3, 40])
+def test_gemm_rows_do_not_leak_where_k_ends_inside_a_unit(cuda, m):
+    """K = 64 mod 128 at group 64: the staging of a row's last unit must not take in the start of the next row.
+    A NaN at the head of row 1 stays in row 1."""
+    L = make_layer(704, 130, bits=2, group=64, m=m, seed=5)
+    x = L.x.copy()
+    x[1, :8] = np.nan
+    _, y = gemm(L, cuda, x)
+    ref = O.gemm_f64(L.x, L.w_quant, L.w_scale, L.w_zero, 64)
+    keep = np.arange(m) != 1
+    assert np.all(np.isnan(y[1].astype(np.float32))) and np.all(np.isfinite(y[keep].astype(np.float32)))
+    assert O.rel_err(y[keep], ref[keep]) <= TOL
 
 
 def test_gemm_rows_agree_with_gemv_and_are_deterministic(cuda):

@@ -19,7 +19,7 @@ def build(k, n, bits, group, seed, dev):
     return L, HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, group, L.bias, dev)
 
 
-@pytest.mark.parametrize("k,n,bits,group", [(1024, 256, 2, 128), (512, 100, 3, 64), (4096, 1024, 2, 128)])
+@pytest.mark.parametrize("k,n,bits,group", [(1024, 256, 2, 128), (512, 100, 3, 64), (4096, 1024, 2, 128), (1088, 130, 2, 64)])
 @pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 4), (2, 16), (_lib.GEMV_NARROW16, 0), (_lib.GEMV_NARROW32, 0),
                                           (_lib.GEMV_WIDE, 0)])
 def test_rmsnorm_prologue_and_residual(cuda, k, n, bits, group, ksplit, waves):
@@ -43,7 +43,7 @@ def test_rmsnorm_prologue_and_residual(cuda, k, n, bits, group, ksplit, waves):
     assert (out.float() - y_plain).abs().max() <= 2e-2 * y_plain.abs().max()
 
 
-@pytest.mark.parametrize("k,n,bits,group", [(1024, 256, 2, 128), (1536, 192, 4, 64)])
+@pytest.mark.parametrize("k,n,bits,group", [(1024, 256, 2, 128), (1536, 192, 4, 64), (960, 100, 2, 64)])
 @pytest.mark.parametrize("ksplit", [0, _lib.GEMV_NARROW16, _lib.GEMV_NARROW32, _lib.GEMV_WIDE])
 def test_silu_mul_prologue(cuda, k, n, bits, group, ksplit):
     L, mod = build(k, n, bits, group, 7, cuda)

@@ -35,6 +35,7 @@ def run(m, x, dev):
 @pytest.mark.parametrize("k,n,bits,group", [
     (256, 64, 2, 128), (512, 128, 2, 128), (1024, 256, 3, 128), (1024, 192, 2, 64),
     (384, 70, 2, 128), (128, 1, 1, 128), (640, 100, 4, 64), (2048, 512, 4, 128), (384, 64, 3, 64),
+    (192, 64, 2, 64), (832, 100, 3, 64), (4160, 256, 2, 64),        # K ends half way through the last unit of 128
 ])
 @pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 1), (1, 4), (2, 2), (3, 8), (_lib.GEMV_NARROW16, 0),
                                           (_lib.GEMV_NARROW32, 0), (_lib.GEMV_WIDE, 0)])
@@ -142,8 +143,8 @@ def test_rows_are_gemvs_and_leading_dims(cuda):
 
 
 def test_dequantize_matches_oracle(cuda):
-    for bits, group, n in ((2, 128, 64), (3, 64, 70), (4, 128, 130)):
-        L = make_layer(384, n, bits=bits, group=group, seed=61)
+    for bits, group, n, k in ((2, 128, 64, 384), (3, 64, 70, 384), (4, 128, 130, 384), (2, 64, 70, 320)):
+        L = make_layer(k, n, bits=bits, group=group, seed=61)
         w = to_mod(L, cuda).dequantize().cpu().numpy()
         planes = O.unpack_planes(L.w_quant).astype(np.float32)
         v = np.repeat(L.w_zero.astype(np.float32), group, axis=1)

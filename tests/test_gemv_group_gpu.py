@@ -28,6 +28,8 @@ def single(mod, x, ksplit):
 @pytest.mark.parametrize("bits,group", [(2, 128), (3, 128), (2, 64), (4, 64), (1, 128)])
 def test_group_equals_single_calls(cuda, bits, group):
     shapes = [(512, 128), (1024, 70), (4096, 256), (8192, 64), (128, 1), (9216, 130), (640, 192)]
+    if group == 64:
+        shapes += [(704, 100), (4160, 64)]                        # K ends half way through the last unit of 128
     layers = [make_layer(k, n, bits=bits, group=group, seed=10 * i + bits, bias=(i % 2 == 0)) for i, (k, n) in enumerate(shapes)]
     mods = [HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, L.group, L.bias, cuda) for L in layers]
     xs = [torch.from_numpy(L.x).to(cuda) for L in layers]

@@ -63,6 +63,14 @@ def test_mfma_refuses_more_than_two_pairs_per_wave(cuda):
         m(torch.from_numpy(L.x).to(cuda))
 
 
+def test_mfma_takes_whole_units_only(cuda):
+    """K that ends half way through the last unit of 128 (group 64) is the LUT kernels' business: the matrix-core
+    kernel refuses it (the tests of this file run with the engine pinned to it)."""
+    L = make_layer(320, 64, bits=2, group=64, seed=1)
+    with pytest.raises(_lib.ElutqError):
+        to_mod(L, cuda)(torch.from_numpy(L.x).to(cuda))
+
+
 @pytest.mark.parametrize("bits,group,ksplit", [(2, 128, 1), (2, 128, 2), (3, 64, 0), (4, 128, 3), (1, 64, 0)])
 def test_mfma_bit_exact_on_integer_inputs(cuda, lutref, bits, group, ksplit):
     """x in {-2..2}, power-of-two scales, quarter-integer zeros: every fp8 term, product and partial sum is exactly

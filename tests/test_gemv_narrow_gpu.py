@@ -33,6 +33,7 @@ def run(m, x, dev):
     (6400, 64, 2, 128),      # 50 units: the last wave's unit lanes partly idle
     (4224, 96, 2, 64),       # 33 units: one unit into the second round / ninth wave
     (4096, 256, 3, 128), (4096, 200, 4, 64), (5120, 70, 1, 128), (8192, 65, 3, 64), (640, 17, 2, 64),
+    (4160, 96, 2, 64), (8128, 64, 2, 64), (448, 40, 4, 64),       # K ends half way through the last unit of 128
 ])
 @pytest.mark.parametrize("ksplit", NARROW)
 def test_narrow_matches_oracle(cuda, k, n, bits, group, ksplit):

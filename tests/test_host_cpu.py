@@ -44,7 +44,12 @@ def test_size_queries_and_argument_errors():
     # columns are padded to 64, an odd number of groups to an even one
     assert L.elutq_hlq_planes_bytes(384, 70, 3) == 128 * 3 * 3 * 16 * 8 // 8
     assert L.elutq_hlq_zeros_bytes(384, 70, 128) == 128 * 2 * 4
-    assert L.elutq_hlq_planes_bytes(100, 64, 2) == 0          # K % 128
+    assert L.elutq_hlq_planes_bytes(100, 64, 2) == 0          # K % 64
+    # K may end half way through the last unit of 128 at group 64 (the reference asks for K % groupsize == 0 only,
+    # arm_gemm.cpp:249): the unit is stored whole
+    assert L.elutq_hlq_planes_bytes(320, 64, 2) == 64 * 3 * 2 * 16
+    assert L.elutq_hlq_scales_bytes(320, 64, 2, 64) == 64 * 3 * 2 * 4 and L.elutq_hlq_scales_bytes(320, 64, 2, 128) == 0
+    assert L.elutq_hlq_zeros_bytes(320, 64, 64) == 64 * 3 * 4 and L.elutq_hlq_workspace_bytes(320, 64, 2, 64, 1) >= 64 * 1024
     assert L.elutq_hlq_workspace_bytes(4096, 4096, 2, 32, 1) == 0
     assert L.elutq_hlq_workspace_bytes(4096, 4096, 2, 128, 1) >= 64 * 1024
     one = ctypes.c_void_p(1)
@@ -53,6 +58,7 @@ def test_size_queries_and_argument_errors():
     assert g(4096, 64, 2, 32) == -4
     assert g(4000, 64, 2, 128) == -2
     assert g(4096, 0, 2, 128) == -2
+    assert g(320, 64, 2, 128) == -2 and g(64, 64, 2, 64) == -2 and g(352, 64, 2, 64) == -2
     assert L.elutq_hlq_gemv_f16(None, one, one, None, one, one, 4096, 64, 2, 128, None, 0, None) == -1
     assert L.elutq_hlq_gemm_f16(one, one, one, None, one, one, 0, 4096, 64, 2, 128, None, 0, None) == -2
     assert L.elutq_hlq_repack_host(None, None, None, 128, 64, 2, 128, None, None, None) == -1
@@ -111,7 +117,7 @@ def test_decoder_defers_down_only_where_the_next_qkv_takes_the_slices():
 
 
 @pytest.mark.parametrize("k,n,bits,group", [(256, 64, 2, 128), (384, 70, 3, 128), (128, 1, 1, 64),
-                                             (512, 200, 4, 64), (1024, 128, 2, 64)])
+                                             (512, 200, 4, 64), (1024, 128, 2, 64), (192, 70, 2, 64), (1088, 64, 3, 64)])
 def test_repack_roundtrip_and_layout(k, n, bits, group):
     L = make_layer(k, n, bits=bits, group=group, seed=3)
     planes, scales, zeros = repack_export_arrays(L.w_quant, L.w_scale, L.w_zero, group)
@@ -120,15 +126,15 @@ def test_repack_roundtrip_and_layout(k, n, bits, group):
     assert np.array_equal(ws.view(np.uint16), L.w_scale.view(np.uint16))
     assert np.array_equal(wz.view(np.uint16), L.w_zero.view(np.uint16))
     # documented layout, checked independently of the library's inverse:
-    ncb, U, NG = (n + 63) // 64, k // 128, k // group
+    ncb, U, NG = (n + 63) // 64, (k + 127) // 128, k // group
     NT = (NG + 1) // 2
     p = planes.view(np.uint32).reshape(ncb, U, bits, 64, 4)
     rot = lambda v, r: ((int(v) >> r) | (int(v) << (32 - r))) & 0xFFFFFFFF
     rs = np.random.default_rng(0)
-    for _ in range(50):
+    for _ in range(80):
         col, u, b, d, i = rs.integers(n), rs.integers(U), rs.integers(bits), rs.integers(4), rs.integers(32)
         kk = u * 128 + d * 32 + i
-        want = (L.w_quant[b, col, kk // 8] >> (kk % 8)) & 1
+        want = (L.w_quant[b, col, kk // 8] >> (kk % 8)) & 1 if kk < k else 0      # past K: zero bits
         natural = rot(p[col // 64, u, b, col % 64, d], 2)          # undo the rotate-left by 2
         assert (natural >> i) & 1 == want
     s = scales.view(np.uint16).reshape(ncb, NT, bits, 64, 2)

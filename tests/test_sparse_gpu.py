@@ -38,7 +38,7 @@ def run(mod, x, dev):
 
 @pytest.mark.parametrize("k,n,bits,group,density", [
     (256, 64, 2, 128, 0.5), (512, 128, 2, 128, 0.3), (1024, 256, 3, 64, 0.2), (1024, 192, 1, 64, 1.0),
-    (2048, 512, 2, 128, 0.05), (384, 96, 4, 128, 0.5),
+    (2048, 512, 2, 128, 0.05), (384, 96, 4, 128, 0.5), (704, 128, 2, 64, 0.3),
 ])
 def test_gemv_matches_oracle(cuda, lutref, k, n, bits, group, density):
     L, sp, mod = build(k, n, bits, group, density, k + n, cuda)
@@ -193,7 +193,8 @@ def test_full_size_layer(cuda):
     assert np.array_equal((-ym).view(np.uint16), y.view(np.uint16))       # y(-x) = -y(x) exactly
 
 
-@pytest.mark.parametrize("k,n,bits,group,density", [(512, 128, 2, 128, 0.3), (1024, 256, 3, 64, 0.2), (4096, 4096, 2, 128, 0.1)])
+@pytest.mark.parametrize("k,n,bits,group,density", [(512, 128, 2, 128, 0.3), (1024, 256, 3, 64, 0.2), (4096, 4096, 2, 128, 0.1),
+                                                     (832, 128, 2, 64, 0.3)])
 def test_dense_form_matches_oracle(cuda, k, n, bits, group, density):
     """The default way to hold the plane on this GPU: one more dense plane, every dense kernel as it is."""
     L, sp, mod = build(k, n, bits, group, density, k + n + 1, cuda, m=3, mode="dense")

@@ -20,7 +20,7 @@ def build(k, n, seed, dev, bits=2, group=128):
 
 @pytest.mark.parametrize("ffn,hidden,n_next,bits,group", [(1024, 512, 768, 2, 128), (14336, 4096, 6144, 2, 128),
                                                           (1024, 512, 768, 3, 64), (1024, 512, 768, 4, 128),
-                                                          (2048, 1024, 1536, 2, 64)])
+                                                          (2048, 1024, 1536, 2, 64), (1088, 576, 768, 2, 64)])
 @pytest.mark.parametrize("consumer", [_lib.GEMV_WIDE, 0, _lib.GEMV_NARROW32])
 def test_consumer_sees_what_the_producer_would_have_written(cuda, ffn, hidden, n_next, bits, group, consumer):
     """down (SiLU*up prologue, K slices) -> next q|k|v (RMSNorm prologue), at the shapes of the small test
