@@ -546,6 +546,28 @@ def main():
                                     "bytes": nbytes, "ring_sets": len(ring)}}
         del ring
         torch.cuda.empty_cache()
+        # ---- the same lm_head unquantized: the dense fp16 GEMV of the decode step (two weight sets of 1.05 GB),
+        # beside the hipBLASLt call it replaced
+        wsets = [(torch.randn(n, k, device=dev) * 0.02).to(torch.float16) for _ in range(2)]
+        yb = torch.empty(1, n, dtype=torch.float16, device=dev)
+
+        def launch_dense(stream):
+            for w in wsets:
+                rc = lib.elutq_fp16_gemv_f16(w.data_ptr(), None, xs[k].data_ptr(), yb.data_ptr(), k, n, None, 0.0, stream)
+                if rc:
+                    raise RuntimeError(f"elutq_fp16_gemv_f16 failed: {rc}")
+
+        def launch_blas(stream):
+            for w in wsets:
+                torch.mm(xs[k], w.t(), out=yb)
+
+        fbytes = 2 * n * k + 2 * k + 2 * n
+        sec = time_graph(torch, launch_dense, max(3, min(a.steps, 10)), 2) / len(wsets)
+        secb = time_graph(torch, launch_blas, max(3, min(a.steps, 10)), 2) / len(wsets)
+        large_shape[f"fp16_{k}x{n}"] = {"us": sec * 1e6, "GBps": fbytes / sec / 1e9, "frac_hbm_peak": fbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                                        "bytes": fbytes, "ring_sets": len(wsets), "hipblaslt_us": secb * 1e6}
+        del wsets
+        torch.cuda.empty_cache()
 
     dom = per_shape["4096x14336"]
     roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",

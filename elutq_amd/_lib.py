@@ -40,6 +40,7 @@ SIGNATURES = {
     "elutq_decode_rope_attn_sliced_f16": (_ci, [_vp, _ci, _ci, _vp, _vp, _vp, _vp] + [_ci] * 4 + [ctypes.c_float, _ci, _vp, _sz, _vp]),
     "elutq_decode_embed_f16": (_ci, [_vp] * 3 + [_ci, _ci, _vp]),
     "elutq_decode_rmsnorm_f16": (_ci, [_vp] * 3 + [_ci, ctypes.c_float, _vp]),
+    "elutq_fp16_gemv_f16": (_ci, [_vp] * 4 + [_ci, _ci, _vp, ctypes.c_float, _vp]),
     "elutq_decode_argmax_f16": (_ci, [_vp, _ci, _vp, _vp, _vp]),
     "elutq_decode_argmax_ws_f16": (_ci, [_vp, _ci, _vp, _vp, _vp, _sz, _vp]),
     "elutq_hlq_gemv_group_workspace_bytes": (_sz, [_vp, _ci, _ci, _ci]),

@@ -18,7 +18,7 @@ CSRC = os.path.join(_PKG, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(_PKG, "libelutq_hip.so")
 SOURCES = ["hlq_gemv.hip", "hlq_gemm.hip", "hlq_misc.hip", "hlq_sparse.hip", "decode_ops.hip", "hlq_repack.cpp",
-           "hlq_static.hip", "hlq_gemv_mfma.hip", "hlq_gemv_narrow.hip"]
+           "hlq_static.hip", "hlq_gemv_mfma.hip", "hlq_gemv_narrow.hip", "fp16_gemv.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -406,6 +406,12 @@ class LlamaDecoder(nn.Module):
             if self.lm_head_q is not None:       # the final norm rides in the GEMV's prologue
                 logits = self.lm_head_q.gemv_fused(x, b.logits, b.ws, prologue=1, norm_weight=self.norm,
                                                    eps=self.s.rms_eps)
+            elif self.s.hidden % 8 == 0 and self.s.hidden <= 32768 and self.lm_head.data_ptr() % 16 == 0:
+                # the unquantized lm_head: the library's dense fp16 GEMV, the final norm in the same launch
+                logits = b.logits
+                _lib.check(L.elutq_fp16_gemv_f16(self.lm_head.data_ptr(), None, x.data_ptr(), logits.data_ptr(), self.s.hidden,
+                                                 self.s.vocab, self.norm.data_ptr(), self.s.rms_eps, stream),
+                           "elutq_fp16_gemv_f16")
             else:
                 _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), free.data_ptr(),
                                                       self.s.hidden, self.s.rms_eps, stream), "elutq_decode_rmsnorm_f16")
@@ -477,7 +483,7 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
             "glue": ("5 launches per layer (rmsnorm+qkv | rope+cache+attention | o+residual | rmsnorm+gate|up | "
                      "silu*up+down+residual; the K slices of q|k|v and of down are summed by the launch that reads "
                      "them), " if impl == "hip" else "PyTorch-ROCm ops around the HLQ GEMVs, ")
-                    + ("own embedding gather, final norm and argmax kernels, "
-                       + ("HLQ GEMV lm_head, " if hlq_lm_head else "hipBLASLt fp16 lm_head, ")
+                    + ("own embedding gather and argmax kernels, "
+                       + ("HLQ GEMV lm_head, " if hlq_lm_head else "own dense fp16 GEMV lm_head, ") + "the final norm inside the lm_head launch, "
                        if impl == "hip" else "torch embedding / final norm / hipBLASLt fp16 lm_head / argmax, ")
                     + "one HIP graph per token"}

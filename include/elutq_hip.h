@@ -316,6 +316,18 @@ int elutq_decode_rope_attn_sliced_f16(const void *d_qkv_slices, int n_slices, in
  * fp16 logits (arm_argmax_last, C++/ops/src/arm/arm_argmax.cpp:3-30; NaNs never win), and, if
  * d_pos is not NULL, *d_pos (DEVICE int64) += 1 -- so a captured graph advances its own state.
  */
+/*
+ * Dense fp16 GEMV, y[n] = fp16(sum_k W[n][k] x[k] + bias[n]) with W fp16 [N][K] row-major: the bit == 16
+ * branch of arm_gemm (C++/ops/src/arm/arm_gemm.cpp:883-886, MultiThreadGemvFP::Run :586-626), which a decode
+ * step runs for an lm_head that was exported unquantized (lm_head.bin, C++/examples/models/llama.cpp:78).
+ * Products and sums in fp32, one rounding (the reference accumulates in fp16).  d_norm_weight not NULL:
+ * x <- fp16(x * rsqrt(mean(x^2) + eps) * norm_weight) first, i.e. the final launch_pre_rms_norm of the step
+ * (C++/ops/src/arm/arm_rmsnorm.cpp:25-84) in the same launch.  d_bias may be NULL.  K % 8 == 0, 8 <= K <= 32768,
+ * d_weight 16-byte aligned; no workspace.
+ */
+int elutq_fp16_gemv_f16(const void *d_weight, const void *d_bias, const void *d_x, void *d_y, int K, int N,
+                        const void *d_norm_weight, float eps, void *stream);
+
 /* Head of a decode step: out[0:hidden] = embed[*d_token][0:hidden], fp16 (arm_embedding,
  * C++/ops/src/arm/arm_embedding.cpp:4-20).  d_token is a DEVICE int64, so a captured graph follows the
  * token the previous step picked; a token outside [0, vocab) gives a zero row (the reference would read
