@@ -287,3 +287,41 @@ def test_k_slices_whose_sums_are_zero(cuda, ksplit):
     xr = torch.from_numpy(L.x).to(cuda)                   # and the slots are usable afterwards
     ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, 128, L.bias)
     assert O.rel_err(_tuned(m, xr, ws, ksplit, 4).cpu().numpy()[0], ref) <= TOL
+
+
+def test_k_sliced_launches_in_a_replayed_graph(cuda):
+    """Three K-sliced GEMVs of different shapes share one workspace inside one HIP graph (the slots of one launch are
+    the slots of the next): every replay, with eager work of the same kind in between, gives the eager result."""
+    shapes = [(2048, 512, 4), (1024, 4096, 4), (4096, 192, 3)]
+    layers = [make_layer(k, n, bits=2, group=128, seed=90 + i) for i, (k, n, _) in enumerate(shapes)]
+    mods = [to_mod(L, cuda) for L in layers]
+    xs = [torch.from_numpy(L.x).to(cuda) for L in layers]
+    ws = torch.zeros(max(m.workspace_bytes for m in mods), dtype=torch.uint8, device=cuda)
+    eager = [_tuned(m, x, ws, ks, 8).clone() for m, x, (_, _, ks) in zip(mods, xs, shapes)]
+    for y, L in zip(eager, layers):
+        assert O.rel_err(y.cpu().numpy()[0], O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, 128)) <= TOL
+    lib = _lib.lib()
+    ys = [torch.zeros_like(y) for y in eager]
+    s = torch.cuda.Stream()
+
+    def launch(stream):
+        for m, x, y, (_, _, ks) in zip(mods, xs, ys, shapes):
+            rc = lib.elutq_hlq_gemv_f16_tuned(m.planes.data_ptr(), m.scales.data_ptr(), m.zeros.data_ptr(), None, x.data_ptr(),
+                                              y.data_ptr(), m.in_features, m.out_features, 2, 128, ws.data_ptr(), ws.numel(),
+                                              stream, ks, 8)
+            assert rc == 0
+
+    with torch.cuda.stream(s):
+        launch(s.cuda_stream)
+    s.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        launch(torch.cuda.current_stream().cuda_stream)
+    for rep in range(5):
+        for y in ys:
+            y.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(y, e) for y, e in zip(ys, eager)), rep
+        assert not ws[:65536].any()
+        assert torch.equal(_tuned(mods[rep % 3], xs[rep % 3], ws, shapes[rep % 3][2], 8), eager[rep % 3])    # eager work in between
