@@ -658,7 +658,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     LaunchShape sh;
-    const bool allow_narrow = !d_extra && !(fusion && fusion->d_slices_out);
+    const bool allow_narrow = !(fusion && fusion->d_slices_out);
     rc = plan_launch(g, bits, ksplit, waves, allow_narrow, sh);
     if (rc != ELUTQ_OK) return rc;
     ksplit = sh.ksplit; waves = sh.waves;

@@ -87,6 +87,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     extern __shared__ __align__(256) unsigned char smem[];
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
+    const HLQ_GLOBAL float *extra = PLAIN ? nullptr : a.extra;      // fp32 term added before the rounding (a sparse extra plane)
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int K = a.K;
@@ -192,6 +193,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
         if (lane < CW && n_out < a.N) {
             if (a.bias) total += (float)__builtin_bit_cast(_Float16, pre_bias);
             if (residual) total += (float)__builtin_bit_cast(_Float16, pre_res);
+            if (extra) total += extra[n_out];
             a.y[n_out] = __builtin_bit_cast(uint16_t, (_Float16)total);
         }
     }
@@ -223,7 +225,7 @@ int launch_narrow_v(const GemvArgs &a, size_t stage_bytes, hipStream_t stream)
 template <int BITS, bool G64, int CW, int R>
 int launch_narrow_r(const GemvArgs &a, size_t stage_bytes, hipStream_t stream)
 {
-    if (a.prologue == 0 && !a.residual) return launch_narrow_v<BITS, G64, CW, R, true>(a, stage_bytes, stream);
+    if (a.prologue == 0 && !a.residual && !a.extra) return launch_narrow_v<BITS, G64, CW, R, true>(a, stage_bytes, stream);
     return launch_narrow_v<BITS, G64, CW, R, false>(a, stage_bytes, stream);
 }
 
@@ -260,7 +262,8 @@ int hlq_gemv_narrow_launch(const void *gemv_args, size_t args_bytes, int bits, i
 {
     if (args_bytes != sizeof(GemvArgs)) return ELUTQ_ERR_HIP;
     const GemvArgs &a = *(const GemvArgs *)gemv_args;
-    if (a.extra || a.defer) return ELUTQ_ERR_TUNING;      // the wide-tile kernel's
+    if (a.defer) return ELUTQ_ERR_TUNING;                 // slices are left behind by the wide-tile kernel only
+    if (a.extra && (a.prologue != 0 || a.residual)) return ELUTQ_ERR_TUNING;      // as on wide tiles: not both
     const bool g64 = group == 64;
     hipStream_t st = (hipStream_t)stream;
     switch (bits) {

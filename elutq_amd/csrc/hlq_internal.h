@@ -34,7 +34,7 @@ HLQ_INTERNAL size_t hlq_gemv_mfma_lds_bytes(int ups, int waves);
 // kernel has no instance for it (its tables of all of K must fit the LDS of one workgroup);
 // hlq_gemv_narrow_lds_bytes: dynamic LDS of a launch without staged activations (0: no instance).  The launch
 // takes the launcher's argument block like hlq_gemv_mfma_launch; prologues, bias, residual and handed-over
-// slices (n_slices_in, with `stage_bytes` = 2 K) as the wide-tile kernel, no extra term and no slices left
+// slices (n_slices_in, with `stage_bytes` = 2 K) and the extra term as the wide-tile kernel, no slices left
 // to the next launch (ELUTQ_ERR_TUNING).
 HLQ_INTERNAL int hlq_gemv_narrow_rounds(int U, int cw);
 HLQ_INTERNAL size_t hlq_gemv_narrow_lds_bytes(int U, int cw);

@@ -148,7 +148,7 @@ int elutq_hlq_gemv_f16_static(const void *d_planes, const void *d_scales, const 
  * without K slices; K <= 8192, else ELUTQ_ERR_TUNING.  With ksplit = waves = 0 the library takes it
  * where the layer has at most 64 / 128 column blocks of 64; ksplit = ELUTQ_GEMV_WIDE keeps it on the
  * wide-tile kernel (64 columns per wavefront) with the library's own K slicing -- the kernel a call with
- * slices to hand over (elutq_gemv_fusion.d_slices_out) or an extra term always runs on.
+ * slices to hand over (elutq_gemv_fusion.d_slices_out) always runs on.
  */
 #define ELUTQ_GEMV_NARROW16 (-16)
 #define ELUTQ_GEMV_NARROW32 (-32)
