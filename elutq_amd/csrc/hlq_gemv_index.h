@@ -110,3 +110,29 @@ HLQ_HD int hlq_stage_index(size_t k0, int ci, int K)
 
 // Row of the handed-over slices a fixed-count load reads for position s (rows past the count re-read the last).
 HLQ_HD int hlq_slice_row(int s, int n_slices_in) { return s < n_slices_in - 1 ? s : n_slices_in - 1; }
+
+// ---- narrow tiles (hlq_gemv_narrow.hip): a wave instruction covers cw = 16 / 32 columns of 64 / cw units ----------
+// LDS of one wave: the tables of its nu = (64 / cw) * rounds units, one spare table behind each unit's 32 (so that
+// units looked up side by side start 16 banks apart), then float2 [2 * nu] half-unit records; rounded up to 256 bytes.
+#define HLQ_NARROW_UNIT_STRIDE (HLQ_UNIT_LUT_BYTES + HLQ_TBL_BYTES)
+HLQ_HD int hlq_narrow_wave_lds(int nu) { return (nu * HLQ_NARROW_UNIT_STRIDE + 2 * nu * 8 + 255) & ~255; }
+// Dynamic LDS of a workgroup: [waves][wave_lds] | float [waves][64] cross-wave sums | float [HLQ_RSTD_SCRATCH] | gap |
+// fp16 [K] staged activations (launches that take handed-over slices only).
+struct HlqNarrowLds {
+    uint32_t red, rstd, stage;      // byte offsets; `stage` == what a launch without staging allocates
+};
+HLQ_HD HlqNarrowLds hlq_narrow_lds(int nu, int waves)
+{
+    HlqNarrowLds m;
+    m.red = (uint32_t)waves * (uint32_t)hlq_narrow_wave_lds(nu);
+    m.rstd = m.red + (uint32_t)waves * 64u * 4u;
+    m.stage = m.rstd + (HLQ_RSTD_SCRATCH + HLQ_STAGE_GAP) * 4u;
+    return m;
+}
+// Chunk `ci` (0 .. 32 nu) of a wave: byte offset of its table inside the wave's region, index of its half-unit record.
+HLQ_HD uint32_t hlq_narrow_table_off(int ci) { return (uint32_t)(ci >> 5) * HLQ_NARROW_UNIT_STRIDE + (uint32_t)(ci & 31) * HLQ_TBL_BYTES; }
+HLQ_HD int hlq_narrow_half_index(int ci) { return ci >> 4; }
+// Global chunk index of x a lane loads for chunk `ci` of its wave (first unit `ub`), clamped to the last chunk of x.
+HLQ_HD int hlq_narrow_x_chunk(int ub, int ci, int K) { const int c = ub * 32 + ci; return c < K / 4 - 1 ? c : K / 4 - 1; }
+// Unit whose weights a lane loads in round r (clamped to the last unit; past it the lane's sum is masked).
+HLQ_HD int hlq_narrow_unit(int ub, int r, int ul_count, int ul, int U) { const int u = ub + r * ul_count + ul; return u < U - 1 ? u : U - 1; }

@@ -22,23 +22,24 @@
 
 namespace {
 
-constexpr int UNIT_STRIDE = UNIT_LUT_BYTES + TBL_BYTES;       // tables of a unit plus the spare one
+constexpr int UNIT_STRIDE = HLQ_NARROW_UNIT_STRIDE;           // tables of a unit plus the spare one
 
 template <int CW, int R>
 struct NarrowGeo {
     static constexpr int UL = 64 / CW;           // units one wave instruction covers (unit lanes)
     static constexpr int NU = UL * R;            // units of a wave: R rounds
     static constexpr int PASSES = NU / 2;        // table-build passes of 64 chunks
-    // tables [NU][33][16] int32, then the half-unit records float2 [2 * NU]
+    // tables [NU][33][16] int32, then the half-unit records float2 [2 * NU] (hlq_narrow_wave_lds)
     static constexpr int WAVE_LDS = (NU * UNIT_STRIDE + 2 * NU * 8 + 255) & ~255;
 };
 
 // dynamic LDS: [waves][WAVE_LDS] | float [waves][64] cross-wave sums | float [HLQ_RSTD_SCRATCH] | gap |
 // fp16 [K] staged activations (launches that take handed-over slices only)
 template <int CW, int R>
-constexpr size_t narrow_lds_bytes(int waves)
+size_t narrow_lds_bytes(int waves)
 {
-    return (size_t)waves * NarrowGeo<CW, R>::WAVE_LDS + (size_t)waves * 64 * 4 + (HLQ_RSTD_SCRATCH + HLQ_STAGE_GAP) * 4;
+    static_assert(NarrowGeo<CW, R>::WAVE_LDS == (NarrowGeo<CW, R>::NU * HLQ_NARROW_UNIT_STRIDE + 2 * NarrowGeo<CW, R>::NU * 8 + 255) / 256 * 256, "");
+    return hlq_narrow_lds(NarrowGeo<CW, R>::NU, waves).stage;
 }
 
 // The lookups of one sub-task (128 k of one plane) where every lane has its own unit: `ub` is the LDS
@@ -98,8 +99,9 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
 
     unsigned char *lut = smem + (size_t)wave * Geo::WAVE_LDS;
     float2 *xs_inv = (float2 *)(lut + NU * UNIT_STRIDE);
-    float *red = (float *)(smem + (size_t)nw * Geo::WAVE_LDS);  // [nw][64]
-    float *rstd_scratch = red + nw * 64;
+    const HlqNarrowLds lm = hlq_narrow_lds(NU, nw);
+    float *red = (float *)(smem + lm.red);                      // [nw][64]
+    float *rstd_scratch = (float *)(smem + lm.rstd);
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
     // what the last step adds to the output, fetched first so that its latency is not left at the end
@@ -116,13 +118,12 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     // block_rstd forms every chunk once, into `stage`
     const bool sliced = !PLAIN && a.n_slices_in > 0;
     SliceChunk sfirst = {};
-    uint2 *stage = (uint2 *)(rstd_scratch + HLQ_RSTD_SCRATCH + HLQ_STAGE_GAP);
+    uint2 *stage = (uint2 *)(smem + lm.stage);
     if (sliced) load_slice_chunk(a, K, min(tid, K / 4 - 1), sfirst);
     uint2 raw[PASSES], raw2[PASSES];
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
-        const int ci = ub * 32 + p * 64 + lane;
-        load_chunk<PLAIN>(a, prologue, K, (size_t)min(ci, K / 4 - 1) * 4, raw[p], raw2[p]);
+        load_chunk<PLAIN>(a, prologue, K, (size_t)hlq_narrow_x_chunk(ub, p * 64 + lane, K) * 4, raw[p], raw2[p]);
     }
     asm volatile("" ::: "memory");      // the activation loads stay ahead of the weight loads
 
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     const HLQ_GLOBAL unsigned char *pz = (const HLQ_GLOBAL unsigned char *)a.zeros + (size_t)cb * a.NT * (size_t)(HLQ_CB * 4);
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const uint32_t u = (uint32_t)min(ub + r * UL + ul, a.U - 1);
+        const uint32_t u = (uint32_t)hlq_narrow_unit(ub, r, UL, ul, a.U);
         const uint32_t row = G64 ? u : (u >> 1);
 #pragma unroll
         for (int b = 0; b < BITS; b++) {
@@ -152,7 +153,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
         rstd = block_rstd(a, K, rstd_scratch, tid, blockDim.x, rfirst, sfirst, sliced, stage, sliced && a.x_out && blockIdx.x == 0);
     if (sliced) {
 #pragma unroll
-        for (int p = 0; p < PASSES; p++) raw[p] = stage[min(ub * 32 + p * 64 + lane, K / 4 - 1)];
+        for (int p = 0; p < PASSES; p++) raw[p] = stage[hlq_narrow_x_chunk(ub, p * 64 + lane, K)];
     }
     // chunks past K (the absent half of a last unit, units no wave lane owns) count as zeros
 #pragma unroll
@@ -163,8 +164,8 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
         const int ci = p * 64 + lane;
-        build_chunk(prologue, raw[p], raw2[p], rstd, lut + (ci >> 5) * UNIT_STRIDE + (ci & 31) * TBL_BYTES,
-                    xs_inv + (ci >> 4), (lane & 15) == 0, lane);
+        build_chunk(prologue, raw[p], raw2[p], rstd, lut + hlq_narrow_table_off(ci), xs_inv + hlq_narrow_half_index(ci),
+                    (lane & 15) == 0, lane);
     }
     // written by this wave, read by this wave: LDS executes a wave's operations in order
     asm volatile("" ::: "memory");

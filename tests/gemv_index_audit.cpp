@@ -1,5 +1,5 @@
-// CPU audit of the index arithmetic of the batch-1 GEMV tile (elutq_amd/csrc/hlq_gemv.hip: gemv_tile,
-// block_rstd, load_slice_chunk).  The kernel computes its run boundaries, LDS offsets and staging indices
+// CPU audit of the index arithmetic of the batch-1 GEMV tiles (elutq_amd/csrc/hlq_gemv.hip: gemv_tile,
+// block_rstd, load_slice_chunk; elutq_amd/csrc/hlq_gemv_narrow.hip: the narrow-tile kernel).  The kernel computes its run boundaries, LDS offsets and staging indices
 // with the functions of elutq_amd/csrc/hlq_gemv_index.h; this program replays them for every slice and
 // every wave -- waves without a run included -- of a superset of the launch shapes the library can choose,
 // and checks the highest byte each access can touch against what the launcher allocates (dynamic LDS =
@@ -116,6 +116,53 @@ void audit(int bits, bool g64, int waves, int U, int ups, int ncb, int n_slices_
 #undef CHECK
 }
 
+// The narrow-tile kernel (hlq_gemv_narrow.hip): workgroups of cw = 16 / 32 columns over all of K, `rounds` units per
+// unit lane of a wave, waves = ceil(U / nu).  Every wave and lane: table stores and half-unit records inside the wave's
+// region, lookups inside the unit's tables, activation chunks inside x and the staged copy, weight / scale / zero loads
+// inside the layer's buffers, cross-wave sums and reduction scratch inside the allocation.
+void audit_narrow(int bits, bool g64, int cw, int rounds, int U, int ncb, bool ragged, bool staged)
+{
+    const int K = U * UNIT - (ragged ? UNIT / 2 : 0);
+    const int ul_count = 64 / cw, nu = ul_count * rounds, waves = (U + nu - 1) / nu;
+    if (waves > 16) return;
+    const HlqNarrowLds lm = hlq_narrow_lds(nu, waves);
+    const size_t lds_alloc = lm.stage + (staged ? (size_t)K * 2 : 0);
+    if (lds_alloc > (size_t)MAX_LDS) return;
+    const int wave_lds = hlq_narrow_wave_lds(nu);
+    const int NT = ((g64 ? K / 64 : U) + 1) / 2;
+    const size_t planes_bytes = (size_t)ncb * U * bits * CB * 16;
+    const size_t scale_bytes = (size_t)ncb * NT * bits * CB * 4, zero_bytes = (size_t)ncb * NT * CB * 4;
+    const int slice = 0, n_slices_in = staged ? 4 : 0, multi = 0, ups = U;
+#define CHECK(ok, what) check((ok), what, bits, g64, waves, U, ups, slice, wave, n_slices_in, multi)
+    for (int wave = 0; wave < waves; wave++) {
+        const uint32_t lut = (uint32_t)wave * wave_lds, xs = lut + (uint32_t)nu * HLQ_NARROW_UNIT_STRIDE;
+        const int ub = wave * nu;
+        for (int ci = 0; ci < 32 * nu; ci++) {
+            CHECK(lut + hlq_narrow_table_off(ci) + 64 <= xs, "n-lds-table");
+            CHECK(xs + (uint32_t)hlq_narrow_half_index(ci) * 8 + 8 <= lut + (uint32_t)wave_lds, "n-lds-half");
+            const int xc = hlq_narrow_x_chunk(ub, ci, K);
+            CHECK(xc >= 0 && (size_t)xc * 4 + 4 <= (size_t)K, "n-x");
+            if (staged) CHECK(lm.stage + (uint32_t)xc * 8 + 8 <= lds_alloc, "n-lds-stage");
+        }
+        for (int r = 0; r < rounds; r++)
+            for (int ul = 0; ul < ul_count; ul++) {
+                const int lu = r * ul_count + ul;
+                CHECK(lut + (uint32_t)lu * HLQ_NARROW_UNIT_STRIDE + 3 * 8 * 64 + 7 * 64 + 60 + 4 <= xs, "n-lds-lookup");
+                CHECK(xs + (uint32_t)(2 * lu + 1) * 8 + 8 <= lut + (uint32_t)wave_lds, "n-lds-half");
+                const int u = hlq_narrow_unit(ub, r, ul_count, ul, U), row = g64 ? u : (u >> 1);
+                for (int cb = 0; cb < ncb; cb += (ncb > 1 ? ncb - 1 : 1))
+                    for (int b = 0; b < bits; b++) {
+                        CHECK(u >= 0 && (((size_t)cb * U + u) * bits + b) * (CB * 16) + 63 * 16 + 16 <= planes_bytes, "n-planes");
+                        CHECK(row < NT && ((size_t)cb * NT * bits + (size_t)row * bits + b) * (CB * 4) + 63 * 4 + 4 <= scale_bytes, "n-scales");
+                        CHECK(((size_t)cb * NT + row) * (CB * 4) + 63 * 4 + 4 <= zero_bytes, "n-zeros");
+                    }
+            }
+        CHECK(lm.red + ((uint32_t)wave * 64 + 63) * 4 + 4 <= lm.rstd, "n-lds-red");
+        CHECK(lm.rstd + (uint32_t)((waves * 64 - 1) >> 4) * 4 + 4 <= lm.rstd + 64 * 4 && lm.rstd + 64 * 4 + 4 <= lm.stage, "n-lds-rstd");
+    }
+#undef CHECK
+}
+
 }  // namespace
 
 int main(int argc, char **argv)
@@ -136,6 +183,17 @@ int main(int argc, char **argv)
                                     shapes++;
                                 }
                             }
+    // narrow tiles: the instances the launcher has (16 columns x 1 round, 32 x 1, 32 x 2), every unit count they take
+    const int narrow[3][2] = {{16, 1}, {32, 1}, {32, 2}};
+    for (int bits = 1; bits <= 4; bits++)
+        for (int g64 = 0; g64 < 2; g64++)
+            for (auto &cr : narrow)
+                for (int U = 1; U <= 64; U++)
+                    for (int ragged = 0; ragged <= (g64 && U > 1 ? 1 : 0); ragged++)
+                        for (int staged = 0; staged < 2; staged++) {
+                            audit_narrow(bits, g64 != 0, cr[0], cr[1], U, 3, ragged != 0, staged != 0);
+                            shapes++;
+                        }
     long total = 0;
     for (auto &kv : g_viol) {
         std::printf("category %s %ld\n", kv.first.c_str(), kv.second);
