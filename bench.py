@@ -8,7 +8,8 @@ One "step" streams the seven projections (q, k, v, o, gate, up, down) of all 32 
 224 GEMVs over 224 distinct random weight sets, 2.07 GB of packed planes + scales + zeros,
 far more than the 256 MB Infinity Cache, so every step reads its weights from HBM.  Inputs
 are resident in HBM before the timed region.  The step is captured once in a HIP graph and
-replayed, so the figure is GPU throughput, not Python launch rate.
+replayed, so the figure is GPU throughput, not Python launch rate.  Defaults: K = 4000 timed steps after
+W = 10 (about four seconds of continuous GPU work per leg; the whole run takes about a minute).
 
 Prints ONE JSON line.  `value` is algorithmic bytes per step / time per step in GB/s
 (bytes = planes + fp16 scales + fp16 zeros + x + y per GEMV).  `per_shape` holds the
@@ -39,8 +40,9 @@ N_LAYERS = 32
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=50)
-    p.add_argument("--warmup", type=int, default=5)
+    # default: a timed region of a few seconds per leg, long enough for a once-every-few-seconds GPU-busy sampler to see it
+    p.add_argument("--steps", type=int, default=4000)
+    p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     p.add_argument("--no-decode", action="store_true", help="skip the decode tokens/s leg")
     p.add_argument("--no-gemm", action="store_true", help="skip the small-batch GEMM leg")
