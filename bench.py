@@ -180,7 +180,7 @@ def gemm_leg(torch, lib, dev, steps):
                     if rc:
                         raise RuntimeError(f"elutq_hlq_gemm_f16 failed: {rc}")
 
-            sec = time_graph(torch, launch, max(3, min(steps, 10)), 1) / nsets
+            sec = time_graph(torch, launch, max(3, min(steps, 200)), 2) / nsets
             flops, nbytes = 2.0 * m * k * n, algorithmic_bytes(k, n, BITS, GROUP, m)
             out[f"{k}x{n}_M{m}"] = {"us": sec * 1e6, "TFLOPs": flops / sec / 1e12,
                                     "frac_mfma_peak": flops / sec / 1e12 / MFMA_PEAK_TFLOPS,
@@ -500,7 +500,7 @@ def main():
             for _ in range(64):
                 hot(stream)
 
-        sec_hot = time_graph(torch, launch_hot, max(3, min(a.steps, 10)), 2) / 64
+        sec_hot = time_graph(torch, launch_hot, max(3, min(a.steps, 500)), 2) / 64
         per_shape[f"{k}x{n}"] = {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
                                  "bytes": nbytes, "ring_sets": len(ring),
                                  "cache_resident_us": sec_hot * 1e6, "cache_resident_GBps": nbytes / sec_hot / 1e9}
@@ -543,7 +543,7 @@ def main():
             for c in ring:
                 c(stream)
 
-        sec = time_graph(torch, launch_big, max(3, min(a.steps, 10)), 2) / len(ring)
+        sec = time_graph(torch, launch_big, max(3, min(a.steps, 2000)), 5) / len(ring)
         large_shape = {f"{k}x{n}": {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
                                     "bytes": nbytes, "ring_sets": len(ring)}}
         del ring
@@ -564,8 +564,8 @@ def main():
                 torch.mm(xs[k], w.t(), out=yb)
 
         fbytes = 2 * n * k + 2 * k + 2 * n
-        sec = time_graph(torch, launch_dense, max(3, min(a.steps, 10)), 2) / len(wsets)
-        secb = time_graph(torch, launch_blas, max(3, min(a.steps, 10)), 2) / len(wsets)
+        sec = time_graph(torch, launch_dense, max(3, min(a.steps, 1000)), 5) / len(wsets)
+        secb = time_graph(torch, launch_blas, max(3, min(a.steps, 1000)), 5) / len(wsets)
         large_shape[f"fp16_{k}x{n}"] = {"us": sec * 1e6, "GBps": fbytes / sec / 1e9, "frac_hbm_peak": fbytes / sec / 1e9 / HBM_PEAK_GBPS,
                                         "bytes": fbytes, "ring_sets": len(wsets), "hipblaslt_us": secb * 1e6}
         del wsets
