@@ -233,6 +233,22 @@ def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
 
         t_sp = time_graph(torch, launch_sparse, steps, warmup) / ring_len
         t_de = time_graph(torch, launch_dense, steps, warmup) / ring_len
+        # inside a decode step: RMSNorm in front of the projection (formed by both launches), residual behind
+        from elutq_amd.hlq_linear import HLQLinear
+        fused = [HLQLinear(k, n, BITS, GROUP, mod.planes, mod.scales, mod.zeros, None, (blocks, scales, index))
+                 for mod, blocks, scales in ring]
+        norm_w = torch.ones(k, dtype=torch.float16, device=dev)
+        res = torch.randn(1, n, device=dev).to(torch.float16)
+
+        def launch_fused(stream, mods=fused):       # (time_graph makes `stream` the current one)
+            for m in mods:
+                m.gemv_fused(x, y, ws, prologue=1, norm_weight=norm_w, eps=1e-5, residual=res)
+
+        def launch_fused_dense(stream):
+            launch_fused(stream, [mod for mod, _, _ in ring])
+
+        t_fu = time_graph(torch, launch_fused, steps, warmup) / ring_len
+        t_fd = time_graph(torch, launch_fused_dense, steps, warmup) / ring_len
         # the plane written out as one more dense plane (scale 0 where no block exists): what the loader does
         # by default -- it costs what any layer with one more plane costs
         wide = [Gemv(lib, make_device_layer(k, n, BITS + 1, GROUP, seed=100 + i, device=dev), x, y, ws) for i in range(ring_len)]
@@ -245,8 +261,43 @@ def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
         sparse_bytes = nblk * (32 * GROUP // 8 + 64 + 4) + 4 * (n // 32 + 1) + 8 * n      # blocks, scales, index, fp32 term out and in
         out[f"{k}x{n}"] = {"blocks": nblk, "density": density, "sparse_layer_us": t_sp * 1e6, "dense_layer_us": t_de * 1e6,
                            "as_one_more_dense_plane_us": t_wi * 1e6,
+                           "rmsnorm_residual_sparse_layer_us": t_fu * 1e6, "rmsnorm_residual_dense_layer_us": t_fd * 1e6,
                            "sparse_plane_bytes": sparse_bytes, "dense_bytes": algorithmic_bytes(k, n, BITS, GROUP)}
+    out["decode"] = sparse_decode_leg(torch, dev, density)
     return out
+
+
+def sparse_decode_leg(torch, dev, density, n_ctx=512, n_gen=50):
+    """Decode tokens/s of the LLaMA-3-8B-shaped w2g128 model whose every projection carries a sparse extra plane on
+    `density` of its blocks, held as blocks: the fused step with one launch of the plane in front of each projection."""
+    from elutq_amd.llama_decode import LlamaDecoder, LlamaShape, random_parts
+    from elutq_amd.synth import with_device_sparse_plane
+    s = LlamaShape()
+    parts = random_parts(s, dev, 0)
+    seed, nblk = 1, 0
+    for lin, _ in parts["layers"]:
+        for name in list(lin):
+            lin[name] = with_device_sparse_plane(lin[name], density, seed)
+            nblk += lin[name].sparse_count
+            seed += 1
+    model = LlamaDecoder(s, device=dev, seed=0, impl="hip", parts=parts)
+    model.fill_cache(n_ctx)
+    model.token.fill_(1)
+    model.capture()
+    for _ in range(n_gen):                       # untimed pass over the same tokens, then the timed one
+        model.replay()
+    model.pos.fill_(n_ctx)
+    model.token.fill_(1)
+    model.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n_gen - 1):
+        model.replay()
+    torch.cuda.synchronize()
+    sec = time.perf_counter() - t0
+    return {"tokens_per_s": (n_gen - 1) / sec, "ms_per_token": sec / (n_gen - 1) * 1e3, "blocks": nblk, "density": density,
+            "model": "LLaMA-3-8B-shaped random init, 32 layers, HLQ w2g128 + sparse extra plane held as blocks on every "
+                     "projection, fp16 lm_head", "n_ctx": n_ctx, "n_gen": n_gen}
 
 
 def counter_mode(a, torch, lib, dev):

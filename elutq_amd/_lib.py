@@ -55,6 +55,7 @@ SIGNATURES = {
     "elutq_hlq_sparse_workspace_bytes": (_sz, [_ci] * 5),
     "elutq_hlq_sparse_gemv_f16": (_ci, [_vp] * 7 + [_ci] + [_vp] * 2 + [_ci] * 4 + [_vp, _sz, _vp]),
     "elutq_hlq_sparse_gemm_f16": (_ci, [_vp] * 7 + [_ci] + [_vp] * 2 + [_ci] * 5 + [_vp, _sz, _vp]),
+    "elutq_hlq_sparse_gemv_fused_f16": (_ci, [_vp] * 7 + [_ci] + [_vp] * 2 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
     "elutq_hlq_sparse_dequant_add_f16": (_ci, [_vp] * 3 + [_ci, _vp] + [_ci] * 3 + [_vp]),
 }
 

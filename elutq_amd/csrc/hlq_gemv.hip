@@ -58,9 +58,9 @@ constexpr int depth_of(int bits) { return bits == 3 ? 6 : (bits == 4 ? 8 : 4); }
 // consumed is refilled with the same sub-task of the next block, so the weight stream never
 // stops between blocks.  Needs runs of at most NSLOT sub-tasks per wave.
 // VAR: which optional inputs the instance reads, known when the kernel is compiled.
-//   GEMV_FUSED  prologue and residual as `a` says (the decode step's launches)
+//   GEMV_FUSED  prologue, residual and the fp32 term `a.extra` as `a` says (the decode step's launches)
 //   GEMV_PLAIN  none of them (their fields of `a` are not read)
-//   GEMV_EXTRA  plain, plus the fp32 term `a.extra` added before the output is rounded
+//   GEMV_EXTRA  plain, plus `a.extra`, added before the output is rounded
 template <int BITS, bool G64, int NSLOT, bool MULTI, int VAR, bool PAIRED>
 __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, int ncb_run, unsigned char *smem, int &red_sel)
 {
@@ -72,7 +72,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     constexpr bool PLAIN = VAR != GEMV_FUSED;
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
-    const HLQ_GLOBAL float *extra = VAR == GEMV_EXTRA ? a.extra : nullptr;
+    const HLQ_GLOBAL float *extra = VAR == GEMV_PLAIN ? nullptr : a.extra;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
@@ -103,9 +103,11 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     // what the last step adds to the output is fetched first of all, so that its latency is not
     // left at the end of the kernel (wave 0 finishes a tile; a run of column blocks loads it there)
     uint16_t pre_bias = 0, pre_res = 0;
+    float pre_extra = 0.f;
     if (!MULTI && wave == 0 && cb * HLQ_CB + lane < a.N) {
         if (a.bias) pre_bias = a.bias[cb * HLQ_CB + lane];
         if (residual) pre_res = residual[cb * HLQ_CB + lane];
+        if (extra) pre_extra = extra[cb * HLQ_CB + lane];
     }
     uint2 rfirst = make_uint2(0, 0);
     if (prologue == 1) rfirst = rstd_first_load(a, K, tid);
@@ -186,7 +188,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
             if (wave == fin && n < a.N) {
                 if (a.bias) total += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
                 if (residual) total += (float)__builtin_bit_cast(_Float16, MULTI ? residual[n] : pre_res);
-                if (extra) total += extra[n];
+                if (extra) total += MULTI ? extra[n] : pre_extra;
                 a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)total);
             }
             return;
@@ -206,7 +208,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                 if (n < a.N) {
                     if (a.bias) sum += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
                     if (residual) sum += (float)__builtin_bit_cast(_Float16, MULTI ? residual[n] : pre_res);
-                    if (extra) sum += extra[n];
+                    if (extra) sum += MULTI ? extra[n] : pre_extra;
                     a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
                 }
                 HLQ_STAMP(7);
@@ -355,7 +357,7 @@ int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
     if (!allow_big_lds((const void *)kern, lds, MAX_LDS, big_lds_done)) return ELUTQ_ERR_HIP;
     // more tiles than CUs and runs that fit the slots: runs of column blocks, one workgroup per CU
     const int run = (a.ncb * a.ksplit + NUM_CU_RUN - 1) / NUM_CU_RUN;
-    if (VAR != GEMV_EXTRA && run > 1 && a.spw <= NSLOT && waves == 16) {       // (the extra term has no run instances)
+    if (VAR != GEMV_EXTRA && run > 1 && a.spw <= NSLOT && waves == 16) {       // (plain plus extra term: no run instances)
         auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT, PAIRED, PLAIN>;
         static bool big_lds_run_done[64] = {};
         if (!allow_big_lds((const void *)kern_run, lds, MAX_LDS, big_lds_run_done)) return ELUTQ_ERR_HIP;
@@ -370,11 +372,9 @@ int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 template <int BITS, bool G64, int NSLOT, bool PAIRED>
 int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
-    if (a.extra) {
-        if (a.prologue != 0 || a.residual) return ELUTQ_ERR_TUNING;     // no instance reads both
+    if (a.extra && a.prologue == 0 && !a.residual)
         return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_EXTRA>(a, waves, lds, stream);
-    }
-    if (a.prologue == 0 && !a.residual && !a.defer && a.n_slices_in == 0)      // the plain instances read none of these fields
+    if (a.prologue == 0 && !a.residual && !a.extra && !a.defer && a.n_slices_in == 0)      // the plain instances read none of these fields
         return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_PLAIN>(a, waves, lds, stream);
     return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_FUSED>(a, waves, lds, stream);
 }

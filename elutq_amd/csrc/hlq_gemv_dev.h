@@ -258,18 +258,21 @@ __device__ __forceinline__ float op_max(float a, float b) { return fmaxf(a, b); 
 // exactly representable in fp16 (the fused ops round to fp16 where the unfused pipeline
 // would have stored fp16: RMSNorm output, arm_rmsnorm.cpp:25-84; SiLU(gate)*up,
 // arm_activation.cpp:36-49).
+__device__ __forceinline__ float prologue_value(int prologue, float v, float w, float rstd)
+{
+    float t;
+    if (prologue == 1) t = v * rstd * w;
+    else t = v / (1.0f + __expf(-v)) * w;
+    return (float)(_Float16)t;
+}
+
 __device__ __forceinline__ void chunk_values(int prologue, uint2 raw, uint2 raw2, float rstd, float (&v)[4])
 {
     v[0] = h2f_lo(raw.x); v[1] = h2f_hi(raw.x); v[2] = h2f_lo(raw.y); v[3] = h2f_hi(raw.y);
     if (prologue == 0) return;
     const float w[4] = {h2f_lo(raw2.x), h2f_hi(raw2.x), h2f_lo(raw2.y), h2f_hi(raw2.y)};
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        float t;
-        if (prologue == 1) t = v[i] * rstd * w[i];
-        else t = v[i] / (1.0f + __expf(-v[i])) * w[i];
-        v[i] = (float)(_Float16)t;
-    }
+    for (int i = 0; i < 4; i++) v[i] = prologue_value(prologue, v[i], w[i], rstd);
 }
 
 // Always two loads (without a prologue the second one re-reads the chunk): a fixed number
@@ -516,7 +519,7 @@ __device__ __forceinline__ void progress_prio(int done, int total)
 }
 
 // Which optional inputs a kernel instance reads, known when it is compiled:
-//   GEMV_FUSED  prologue and residual as the argument block says (the decode step's launches)
+//   GEMV_FUSED  prologue, residual and the fp32 term `extra` as the argument block says (the decode step's launches)
 //   GEMV_PLAIN  none of them (their fields are not read)
 //   GEMV_EXTRA  plain, plus the fp32 term `extra` added before the output is rounded
 enum { GEMV_FUSED = 0, GEMV_PLAIN = 1, GEMV_EXTRA = 2 };

@@ -107,9 +107,11 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     // what the last step adds to the output, fetched first so that its latency is not left at the end
     const int n_out = cb * HLQ_CB + part * CW + lane;           // lanes < CW of wave 0 store
     uint16_t pre_bias = 0, pre_res = 0;
+    float pre_extra = 0.f;
     if (wave == 0 && lane < CW && n_out < a.N) {
         if (a.bias) pre_bias = a.bias[n_out];
         if (residual) pre_res = residual[n_out];
+        if (extra) pre_extra = extra[n_out];
     }
     // activations: chunk p * 64 + lane of the wave's NU units (clamped to K: units past the end are masked below)
     uint2 rfirst = make_uint2(0, 0);
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
         if (lane < CW && n_out < a.N) {
             if (a.bias) total += (float)__builtin_bit_cast(_Float16, pre_bias);
             if (residual) total += (float)__builtin_bit_cast(_Float16, pre_res);
-            if (extra) total += extra[n_out];
+            if (extra) total += pre_extra;
             a.y[n_out] = __builtin_bit_cast(uint16_t, (_Float16)total);
         }
     }
@@ -264,7 +266,6 @@ int hlq_gemv_narrow_launch(const void *gemv_args, size_t args_bytes, int bits, i
     if (args_bytes != sizeof(GemvArgs)) return ELUTQ_ERR_HIP;
     const GemvArgs &a = *(const GemvArgs *)gemv_args;
     if (a.defer) return ELUTQ_ERR_TUNING;                 // slices are left behind by the wide-tile kernel only
-    if (a.extra && (a.prologue != 0 || a.residual)) return ELUTQ_ERR_TUNING;      // as on wide tiles: not both
     const bool g64 = group == 64;
     hipStream_t st = (hipStream_t)stream;
     switch (bits) {

@@ -7,8 +7,9 @@
 #define HLQ_INTERNAL __attribute__((visibility("hidden")))
 
 // elutq_hlq_gemv_fused_f16 with an fp32 vector [N] (device) added to every output before it is
-// rounded to fp16; d_extra may be null.  No kernel instance reads both the extra term and a
-// prologue / residual: such a call returns ELUTQ_ERR_TUNING.
+// rounded to fp16; d_extra may be null.  The matrix-core kernel has no instance that reads both the
+// extra term and a prologue / residual (ELUTQ_ERR_TUNING where that engine is selected); no kernel
+// leaves K slices to the next launch with an extra term due.
 HLQ_INTERNAL int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
                                      const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
                                      size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,

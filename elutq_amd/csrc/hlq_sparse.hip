@@ -13,6 +13,10 @@
 // dense GEMV / GEMM kernel then adds it to its own fp32 sum before the one rounding to fp16, so a
 // sparse layer's output is as exact as a dense layer's.
 //
+// In a decode step the projection's input may only exist inside the launch that reads it (the fused GEMV forms
+// RMSNorm(x) or SiLU(gate) * up in its prologue): the batch-1 plane kernel then forms the same values itself, with
+// the same operations (prologue_value), from the same stored vectors.
+//
 // The block bits and scales stay exactly as the files hold them -- [block][32 channels][G/8
 // bytes] is already what a wave wants: 8 consecutive lanes own the 8 k-eighths of one channel, so a
 // block is one contiguous 32*G/8-byte read -- and the pair list becomes an index by channel tile.
@@ -22,12 +26,14 @@
 #include "../../include/elutq_hip.h"
 #include "hlq_layout.h"
 #include "hlq_internal.h"
+#include "hlq_gemv_dev.h"
 
 namespace {
 
 constexpr int SP_TILE = 32;        // channels per block
 constexpr int SP_PARTS = 8;        // lanes that share a channel: each owns G/8 consecutive k
 constexpr int SP_THREADS = SP_TILE * SP_PARTS;
+constexpr int SP_HEAD = 16;        // k starts per tile that the batch-1 kernel finds without knowing the tile's block range
 
 inline int sp_tiles(int N) { return (N + SP_TILE - 1) / SP_TILE; }
 
@@ -36,10 +42,15 @@ struct SparseArgs {
     const uint16_t *blk_scales;    // fp16 [nblk][32]
     const int32_t *tile_ptr;       // [tiles + 1]: blocks of tile t are tile_ptr[t] .. tile_ptr[t+1]-1
     const int32_t *blk_k;          // [nblk] k start
+    const int32_t *head;           // [tiles][SP_HEAD]: k starts of a tile's first SP_HEAD blocks again (-1: no such block)
     const uint16_t *x;             // fp16 [M][K]
     float *extra;                  // fp32 [M][N], written for every (m, n)
     uint16_t *w;                   // fp16 [N][K] (dequantisation only)
     int M, K, N, nblk;
+    // M == 1 only: the activations pass through the prologue of the fused GEMV first
+    int prologue;                  // 0: x as is; 1: rmsnorm(x) * norm_w; 2: silu(x[0:K]) * x[K:2K]
+    float eps;
+    const uint16_t *norm_w;        // fp16 [K] (prologue 1)
 };
 
 __device__ __forceinline__ float hf(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
@@ -123,6 +134,146 @@ __global__ __launch_bounds__(SP_THREADS) void hlq_sparse_plane_kernel(const Spar
     }
 }
 
+// Batch 1: one workgroup of sixteen waves per channel tile; wave w takes the tile's blocks w, w + 16, ... and works
+// on a block alone (a tile's blocks cost a chain of dependent memory round trips -- block range, k starts,
+// activations -- whatever their number, so as many as possible go through it side by side).  The G activations of a block are the same for its 32 channels, so the wave forms them once
+// (two per lane, through the prologue if there is one), parks them in LDS as fp32 and every lane (channel, half of
+// the block's k) adds up the ones its bits select: LDS reads of one address per half, no bank conflicts.  NB
+// blocks of a wave are in flight at a time (their k starts, bits, scales and activations depend on each other only
+// through addresses).  The waves' sums meet in LDS in wave order: the result does not depend on timing.
+// v where bit `pos` of `bits` is set, else +0.
+__device__ __forceinline__ float bit_select(float v, uint32_t bits, int pos)
+{
+    const uint32_t mask = (uint32_t)__builtin_amdgcn_sbfe((int)bits, pos, 1);      // the bit, sign-extended
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) & mask);
+}
+
+constexpr int SPV_WAVES = 16;                    // at most; the launch decides (blockDim.x / 64)
+
+template <int G, bool PRO, int NB>
+__global__ __launch_bounds__(SPV_WAVES * 64) void hlq_sparse_plane_gemv_kernel(const SparseArgs a)
+{
+    constexpr int HALF = G / 2;                      // k per lane and block
+    __shared__ __align__(16) float xs[SPV_WAVES][NB][G];
+    __shared__ float red[SPV_WAVES][SP_TILE];
+    __shared__ float part_ssq[SPV_WAVES];
+    const int tile = blockIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), nw = blockDim.x >> 6;
+    const int ch = lane >> 1, part = lane & 1;
+    const int prologue = PRO ? a.prologue : 0;
+    // block `wave` of the tile is this wave's first: its k start comes in with the tile's block range, not after it
+    // (one memory round trip fewer in front of the activations)
+    const int k_head = a.head[(size_t)tile * SP_HEAD + wave];
+    const int b0 = a.tile_ptr[tile], b1 = a.tile_ptr[tile + 1];
+    const int n = tile * SP_TILE + ch;
+    if (b0 >= b1) {                                  // the same for every thread of the workgroup
+        if (wave == 0 && part == 0 && n < a.N) a.extra[n] = 0.f;
+        return;
+    }
+    const uint16_t *second = prologue == 1 ? a.norm_w : (prologue == 2 ? a.x + a.K : a.x);
+    const int xl = G == 128 ? lane : (lane & 31);    // the pair of activations this lane forms (G = 64: both halves of the wave the same)
+    int k0[NB];
+    uint32_t raw[NB], raw2[NB], bits[NB][HALF / 32];
+    float s[NB];
+    // everything a round of NB blocks reads from memory (nothing of it depends on 1 / rms): first what depends on
+    // the block numbers alone, then the activations at the k starts that came in
+    auto load_meta = [&](int base, bool first) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const int blk = base + i * nw;
+            const int blkc = min(blk, b1 - 1);       // past the end: the last block again, its result dropped
+            k0[i] = first && i == 0 ? k_head : a.blk_k[blkc];
+            const uint32_t *bp = (const uint32_t *)(a.blocks + ((size_t)blkc * SP_TILE + ch) * (G / 8) + part * (HALF / 8));
+#pragma unroll
+            for (int q = 0; q < HALF / 32; q++) bits[i][q] = bp[q];
+            s[i] = hf(a.blk_scales[(size_t)blkc * SP_TILE + ch]);
+            // the index is validated on the host; a bad k start still never reads outside x
+            if (!(blk < b1 && k0[i] >= 0 && k0[i] + G <= a.K)) {
+                k0[i] = 0; s[i] = 0.f;
+#pragma unroll
+                for (int q = 0; q < HALF / 32; q++) bits[i][q] = 0;
+            }
+        }
+    };
+    auto load_x = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            raw[i] = *(const uint32_t *)(a.x + k0[i] + 2 * xl);          // k0 % 4 == 0: 4-byte aligned
+            raw2[i] = PRO ? *(const uint32_t *)(second + k0[i] + 2 * xl) : raw[i];
+        }
+    };
+    load_meta(b0 + wave, true);                      // in flight while the workgroup sums the squares
+    float rstd = 1.f;
+    if (PRO && prologue == 1) {
+        float ssq = 0.f;
+        for (int i = tid; i < a.K / 4; i += nw * 64) {
+            const uint2 r = *(const uint2 *)(a.x + (size_t)i * 4);
+            const float x0 = h2f_lo(r.x), x1 = h2f_hi(r.x), x2 = h2f_lo(r.y), x3 = h2f_hi(r.y);
+            ssq += (x0 * x0 + x1 * x1) + (x2 * x2 + x3 * x3);
+        }
+        load_x();
+#pragma unroll
+        for (int d = 1; d < 64; d *= 2) ssq += __shfl_xor(ssq, d, 64);
+        if (lane == 0) part_ssq[wave] = ssq;
+        __syncthreads();
+        float all = 0.f;
+        for (int w = 0; w < nw; w++) all += part_ssq[w];
+        rstd = rsqrtf(all / (float)a.K + a.eps);
+    } else {
+        load_x();
+    }
+    float tot = 0.f;
+    for (int base = b0 + wave; base < b1; base += nw * NB) {
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            float v0 = h2f_lo(raw[i]), v1 = h2f_hi(raw[i]);
+            if (PRO && prologue != 0) {
+                v0 = prologue_value(prologue, v0, h2f_lo(raw2[i]), rstd);
+                v1 = prologue_value(prologue, v1, h2f_hi(raw2[i]), rstd);
+            }
+            if (G == 128 || lane < 32) *(float2 *)&xs[wave][i][2 * xl] = make_float2(v0, v1);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");          // this wave's LDS stores before its loads below
+        __builtin_amdgcn_wave_barrier();
+        float sums[NB];
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            sums[i] = 0.f;
+            if (base + i * nw >= b1) continue;       // no such block (the same for the whole wave)
+            const float4 *xp = (const float4 *)&xs[wave][i][part * HALF];
+            float sum = 0.f;
+#pragma unroll
+            for (int q = 0; q < HALF / 4; q++) {
+                // an activation or +0, chosen by an all-ones / all-zeros mask made of its bit: no branches, and the
+                // reads of a block go out together
+                const float4 v = xp[q];
+                const uint32_t w = bits[i][q / 8];
+                sum += bit_select(v.x, w, 4 * (q % 8));
+                sum += bit_select(v.y, w, 4 * (q % 8) + 1);
+                sum += bit_select(v.z, w, 4 * (q % 8) + 2);
+                sum += bit_select(v.w, w, 4 * (q % 8) + 3);
+            }
+            sums[i] = sum + __shfl_xor(sum, 1, 64);  // the two halves of a channel sit in neighbouring lanes
+        }
+#pragma unroll
+        for (int i = 0; i < NB; i++) tot = fmaf(s[i], sums[i], tot);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");          // ... and those loads before the next round's stores
+        __builtin_amdgcn_wave_barrier();
+        if (base + nw * NB < b1) {
+            load_meta(base + nw * NB, false);
+            load_x();
+        }
+    }
+    if (part == 0) red[wave][ch] = tot;
+    __syncthreads();
+    if (wave == 0 && part == 0 && n < a.N) {
+        float sum = red[0][ch];
+        for (int w = 1; w < nw; w++) sum += red[w][ch];
+        a.extra[n] = sum;
+    }
+}
+
 // W[c0 + ch][k0 + j] += scale[blk][ch] where the block's bit is set.  One workgroup per channel
 // tile walks the tile's blocks in list order with a barrier between them, so blocks that overlap in
 // k (the format does not forbid it) add up as they do in the GEMV.
@@ -162,6 +313,7 @@ SparseArgs sparse_args(const void *d_blocks, const void *d_blk_scales, const voi
     a.blk_scales = (const uint16_t *)d_blk_scales;
     a.tile_ptr = (const int32_t *)d_index;
     a.blk_k = a.tile_ptr + sp_tiles(N) + 1;
+    a.head = a.blk_k + nblk;
     a.K = K; a.N = N; a.nblk = nblk;
     return a;
 }
@@ -172,12 +324,21 @@ int launch_sparse_plane(SparseArgs a, const void *d_x, float *d_extra, int M, in
     a.x = (const uint16_t *)d_x;
     a.extra = d_extra;
     a.M = M;
-    const int rows = M == 1 ? 1 : 4;
-    const dim3 grid(sp_tiles(a.N), (M + rows - 1) / rows);
     if (M == 1) {
-        if (group == 64) hipLaunchKernelGGL((hlq_sparse_plane_kernel<64, 1, 4>), grid, dim3(SP_THREADS), 0, stream, a);
-        else hipLaunchKernelGGL((hlq_sparse_plane_kernel<128, 1, 4>), grid, dim3(SP_THREADS), 0, stream, a);
+        // as many waves per tile as leave all tiles resident at once (32 waves per compute unit)
+        const int tiles = sp_tiles(a.N);
+        const int waves = tiles * 16 <= HLQ_NUM_CU * 32 ? 16 : (tiles * 8 <= HLQ_NUM_CU * 32 ? 8 : 4);
+        const dim3 grid(tiles), block(waves * 64);
+        if (a.prologue != 0) {
+            if (group == 64) hipLaunchKernelGGL((hlq_sparse_plane_gemv_kernel<64, true, 2>), grid, block, 0, stream, a);
+            else hipLaunchKernelGGL((hlq_sparse_plane_gemv_kernel<128, true, 2>), grid, block, 0, stream, a);
+        } else {
+            if (group == 64) hipLaunchKernelGGL((hlq_sparse_plane_gemv_kernel<64, false, 2>), grid, block, 0, stream, a);
+            else hipLaunchKernelGGL((hlq_sparse_plane_gemv_kernel<128, false, 2>), grid, block, 0, stream, a);
+        }
     } else {
+        if (a.prologue != 0) return ELUTQ_ERR_TUNING;
+        const dim3 grid(sp_tiles(a.N), (M + 3) / 4);
         if (group == 64) hipLaunchKernelGGL((hlq_sparse_plane_kernel<64, 4, 2>), grid, dim3(SP_THREADS), 0, stream, a);
         else hipLaunchKernelGGL((hlq_sparse_plane_kernel<128, 4, 2>), grid, dim3(SP_THREADS), 0, stream, a);
     }
@@ -193,7 +354,7 @@ extern "C" {
 size_t elutq_hlq_sparse_index_bytes(int N, int nblk)
 {
     if (N < 1 || nblk < 0) return 0;
-    return sizeof(int32_t) * ((size_t)sp_tiles(N) + 1 + (size_t)nblk);
+    return sizeof(int32_t) * ((size_t)sp_tiles(N) + 1 + (size_t)nblk + (size_t)sp_tiles(N) * SP_HEAD);
 }
 
 int elutq_hlq_sparse_index_host(const uint32_t *h_mask, int mask_len, int K, int N, int group, void *h_index_out)
@@ -216,6 +377,10 @@ int elutq_hlq_sparse_index_host(const uint32_t *h_mask, int mask_len, int K, int
         blk_k[i] = (int32_t)k;
     }
     for (int t = 0; t < tiles; t++) tile_ptr[t + 1] += tile_ptr[t];
+    int32_t *head = blk_k + nblk;
+    for (int t = 0; t < tiles; t++)
+        for (int j = 0; j < SP_HEAD; j++)
+            head[(size_t)t * SP_HEAD + j] = tile_ptr[t] + j < tile_ptr[t + 1] ? blk_k[tile_ptr[t] + j] : -1;
     return ELUTQ_OK;
 }
 
@@ -260,6 +425,36 @@ int elutq_hlq_sparse_gemm_f16(const void *d_planes, const void *d_scales, const 
         m0 += mc;
     }
     return ELUTQ_OK;
+}
+
+int elutq_hlq_sparse_gemv_fused_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                                    const void *d_blocks, const void *d_blk_scales, const void *d_index, int nblk,
+                                    const void *d_x, void *d_y, int K, int N, int bits, int group,
+                                    void *d_workspace, size_t workspace_bytes, void *stream,
+                                    const elutq_gemv_fusion *fusion, int ksplit, int waves)
+{
+    int rc = check_sparse_call(K, N, group, nblk);
+    if (rc != ELUTQ_OK) return rc;
+    if (!d_index || !d_x || !d_y || !d_workspace || (nblk && (!d_blocks || !d_blk_scales))) return ELUTQ_ERR_NULL;
+    const size_t dense = elutq_hlq_workspace_bytes(K, N, bits, group, 1);
+    if (!dense) return bits < 1 || bits > 4 ? ELUTQ_ERR_BITS : ELUTQ_ERR_SHAPE;
+    if (workspace_bytes < elutq_hlq_sparse_workspace_bytes(K, N, bits, group, 1)) return ELUTQ_ERR_WORKSPACE;
+    SparseArgs a = sparse_args(d_blocks, d_blk_scales, d_index, nblk, K, N);
+    if (fusion) {
+        // the plane reads the projection's input from the vectors the call names: K slices handed over by another
+        // launch, or left to one, are not among them
+        if (fusion->d_slices_out || fusion->n_slices_in != 0 || fusion->d_slices_in) return ELUTQ_ERR_TUNING;
+        if (fusion->prologue < 0 || fusion->prologue > 2) return ELUTQ_ERR_TUNING;
+        if (fusion->prologue == 1 && !fusion->d_norm_weight) return ELUTQ_ERR_NULL;
+        a.prologue = fusion->prologue;
+        a.eps = fusion->eps;
+        a.norm_w = (const uint16_t *)fusion->d_norm_weight;
+    }
+    float *extra = (float *)((unsigned char *)d_workspace + align256(dense));
+    rc = launch_sparse_plane(a, d_x, extra, 1, group, (hipStream_t)stream);
+    if (rc != ELUTQ_OK) return rc;
+    return hlq_gemv_with_extra(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace, dense,
+                               stream, fusion, ksplit, waves, extra);
 }
 
 int elutq_hlq_sparse_gemv_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,

@@ -126,6 +126,15 @@ class HLQLinear(nn.Module):
         self._ws_cache: dict = {}
         self.ksplit, self.waves = 0, 0      # 0 = library default; set for tuning
 
+    def sparse_pairs(self) -> np.ndarray:
+        """uint32 [nblk, 2]: the (channel start, k start) pairs of the sparse extra plane's blocks, in list order
+        (the contents of weight_mask.bin), read back from the index the kernels use."""
+        tiles = (self.out_features + 31) // 32
+        idx = self.sparse_index.cpu().numpy()
+        counts = np.diff(idx[:tiles + 1])
+        return np.stack([np.repeat(np.arange(tiles, dtype=np.int64) * 32, counts),
+                         idx[tiles + 1:tiles + 1 + self.sparse_count]], 1).astype(np.uint32)
+
     def _ws_bytes_for(self, m: int) -> int:
         key = 64 if m > 32 else 32
         if key not in self._ws_cache:
@@ -204,7 +213,7 @@ class HLQLinear(nn.Module):
         Lets layers of different depth share a launch (q|k|v where only one of them carries an extra plane)."""
         if bits == self.bits:
             return self
-        if bits < self.bits or bits > 4 or self.sparse_count:
+        if bits < self.bits or bits > 4:
             raise ValueError(f"cannot turn a {self.bits}-plane layer into a {bits}-plane one")
         ncb = (self.out_features + 63) // 64
         add = bits - self.bits
@@ -214,8 +223,9 @@ class HLQLinear(nn.Module):
             z = torch.zeros(ncb, v.shape[1], add, 64 * unit_bytes, dtype=buf.dtype, device=buf.device)
             return torch.cat([v, z], 2).reshape(-1)
 
+        sparse = (self.sparse_blocks, self.sparse_scales, self.sparse_index) if self.sparse_count else None
         return HLQLinear(self.in_features, self.out_features, bits, self.group_size, widen(self.planes, 16),
-                         widen(self.scales, 4), self.zeros, self.bias)
+                         widen(self.scales, 4), self.zeros, self.bias, sparse)
 
     # -- compute -----------------------------------------------------------------------
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -274,10 +284,11 @@ class HLQLinear(nn.Module):
         not written; `slices_in` (fp32 [S, K], prologue 1): x is the sum of those slices plus `x`,
         rounded to fp16 (what the producer would have written with residual = x), and `x_out`
         receives it.
-        A layer with a sparse extra plane cannot be fused (the plane reads the projection's own
-        input, which a prologue only forms inside the kernel): use forward()."""
-        if self.sparse_count:
-            raise NotImplementedError("a layer with a sparse extra plane has no fused GEMV; call forward()")
+        A layer with a sparse extra plane held as blocks takes two launches (the plane's fp32 term with
+        the same prologue, then the dense kernel, elutq_hlq_sparse_gemv_fused_f16), `ws` of
+        self.workspace_bytes, and no slices in either direction."""
+        if self.sparse_count and (slices_out is not None or slices_in is not None):
+            raise ValueError("a layer with a sparse extra plane held as blocks neither takes nor leaves K slices")
         f = _lib.GemvFusion(prologue, eps, norm_weight.data_ptr() if norm_weight is not None else None,
                             residual.data_ptr() if residual is not None else None,
                             slices_out.data_ptr() if slices_out is not None else None,
@@ -289,6 +300,15 @@ class HLQLinear(nn.Module):
         if slices_in is not None and (slices_in.dtype != torch.float32 or slices_in.dim() != 2
                                       or slices_in.shape[1] != self.in_features or not slices_in.is_contiguous()):
             raise ValueError("slices_in must be contiguous fp32 [S, in_features]")
+        if self.sparse_count:
+            rc = _lib.lib().elutq_hlq_sparse_gemv_fused_f16(
+                self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
+                self.bias.data_ptr() if self.bias is not None else None, self.sparse_blocks.data_ptr(),
+                self.sparse_scales.data_ptr(), self.sparse_index.data_ptr(), self.sparse_count, x.data_ptr(), out.data_ptr(),
+                self.in_features, self.out_features, self.bits, self.group_size, ws.data_ptr(), ws.numel(),
+                torch.cuda.current_stream(x.device).cuda_stream, ctypes.byref(f), self.ksplit, self.waves)
+            _lib.check(rc, "elutq_hlq_sparse_gemv_fused_f16")
+            return out
         rc = _lib.lib().elutq_hlq_gemv_fused_f16(
             self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
             self.bias.data_ptr() if self.bias is not None else None, x.data_ptr(), out.data_ptr(),
@@ -299,6 +319,10 @@ class HLQLinear(nn.Module):
 
     @property
     def workspace_bytes(self) -> int:
+        """Workspace of a batch-1 call (with a sparse extra plane held as blocks: its fp32 term behind the dense part)."""
+        if self.sparse_count:
+            return _lib.lib().elutq_hlq_sparse_workspace_bytes(self.in_features, self.out_features, self.bits,
+                                                               self.group_size, 1)
         return self._ws_bytes
 
     @property

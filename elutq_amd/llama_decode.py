@@ -55,9 +55,6 @@ def fuse_along_n(mods: list[HLQLinear]) -> HLQLinear:
     """One HLQLinear computing the concatenation of the outputs.  The kernel layout is
     column-block major, so this is a concatenation of the packed buffers (every N but the
     last must be a multiple of 64)."""
-    if any(m.sparse_count for m in mods):
-        raise NotImplementedError("layers whose sparse extra plane is held as blocks cannot be concatenated: load "
-                                  "them with sparse_mode='dense', or build the decoder with fuse=False, impl='torch'")
     k, group = mods[0].in_features, mods[0].group_size
     bits = max(m.bits for m in mods)                 # a layer that carries an extra plane lifts the others
     mods = [m.with_bits(bits) for m in mods]
@@ -71,7 +68,31 @@ def fuse_along_n(mods: list[HLQLinear]) -> HLQLinear:
                           torch.zeros(m.out_features, dtype=torch.float16, device=m.planes.device) for m in mods])
     return HLQLinear(k, sum(m.out_features for m in mods), bits, group,
                      torch.cat([m.planes for m in mods]), torch.cat([m.scales for m in mods]),
-                     torch.cat([m.zeros for m in mods]), bias)
+                     torch.cat([m.zeros for m in mods]), bias, concat_sparse(mods))
+
+
+def concat_sparse(mods: list[HLQLinear]):
+    """The sparse extra planes (held as blocks) of layers concatenated along N as one plane: the block
+    lists one after the other, every layer's channels behind those of the layers before it; the index is
+    made anew from the (channel start, k start) pairs."""
+    if not any(m.sparse_count for m in mods):
+        return None
+    import numpy as np
+
+    from .hlq_linear import sparse_index
+    dev = mods[0].planes.device
+    k, group = mods[0].in_features, mods[0].group_size
+    blocks, scales, pairs = [], [], []
+    n0 = 0
+    for m in mods:
+        if m.sparse_count:
+            blocks.append(m.sparse_blocks.reshape(-1))
+            scales.append(m.sparse_scales)
+            pairs.append(m.sparse_pairs() + np.array([[n0, 0]], dtype=np.uint32))
+        n0 += m.out_features
+    nblk = sum(p.shape[0] for p in pairs)
+    index = torch.from_numpy(sparse_index(np.concatenate(pairs), k, n0, group)).to(dev)
+    return (torch.cat(blocks).view(nblk, 32, group // 8), torch.cat(scales), index)
 
 
 def rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
@@ -165,7 +186,8 @@ def deferred_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tenso
     down sums them itself."""
     s = layer.s
     n_q = layer.qkv.slices
-    defer_qkv = defer_qkv and s.head_dim == 128 and 2 <= n_q <= MAX_DEFERRED_SLICES and layer.qkv.bias is None
+    defer_qkv = (defer_qkv and s.head_dim == 128 and 2 <= n_q <= MAX_DEFERRED_SLICES and layer.qkv.bias is None
+                 and not layer.qkv.sparse_count)
     layer.qkv.gemv_fused(cur, b.qkv, b.ws, prologue=1, norm_weight=layer.ln1, eps=s.rms_eps,
                          slices_in=b.sd[:pending] if pending else None, x_out=other if pending else None,
                          slices_out=b.sq if defer_qkv else None)
@@ -187,7 +209,8 @@ def deferred_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tenso
     layer.gate_up.gemv_fused(other, b.gu, b.ws, prologue=1, norm_weight=layer.ln2, eps=s.rms_eps)
     cur, other = other, cur
     n_d = layer.down_proj.slices
-    if not last and defer_down and 2 <= n_d <= MAX_DEFERRED_SLICES and layer.down_proj.bias is None:
+    if (not last and defer_down and 2 <= n_d <= MAX_DEFERRED_SLICES and layer.down_proj.bias is None
+            and not layer.down_proj.sparse_count):
         layer.down_proj.gemv_fused(b.gu, other, b.ws, prologue=2, slices_out=b.sd)
         return cur, other, n_d
     layer.down_proj.gemv_fused(b.gu, other, b.ws, prologue=2, residual=cur)
@@ -325,10 +348,6 @@ class LlamaDecoder(nn.Module):
         self.defer_slices = True
         self.defer_qkv = False             # likewise q|k|v -> attention (set by the constructor, see qkv_to_attention)
         if impl == "hip":
-            if any(m.sparse_count for m in self.modules() if isinstance(m, HLQLinear)):
-                raise NotImplementedError("the fused decode step takes no sparse extra plane held as blocks: load the "
-                                          "layers with sparse_mode='dense', or build the decoder with fuse=False, "
-                                          "impl='torch'")
             ws = max(m.workspace_bytes for m in self.modules() if isinstance(m, HLQLinear))
             ws = max(ws, _lib.lib().elutq_decode_attn_workspace_bytes(s.n_heads, s.head_dim, 0))
             self._buf = FusedBuffers(s, ws, dev)
@@ -341,6 +360,8 @@ class LlamaDecoder(nn.Module):
             if self.defer_qkv:
                 for layer in self.layers:
                     q = layer.qkv
+                    if q.sparse_count:
+                        continue                         # its plane's launch reads the stored input: no slices
                     if q.bias is None and q.slices == 1 and 2 * ((q.out_features + 63) // 64) <= 256:
                         q.ksplit, q.waves = 2, 16
                     elif q.ksplit == 0:
@@ -349,6 +370,7 @@ class LlamaDecoder(nn.Module):
             # with more tiles than compute units, or tables that leave no room for the staged activations,
             # does not): decided here, once, so that a step never meets a refusing launch
             self._defer_down = [i + 1 < len(self.layers) and 2 <= layer.down_proj.slices <= MAX_DEFERRED_SLICES
+                                and not layer.down_proj.sparse_count and not self.layers[i + 1].qkv.sparse_count
                                 and self.layers[i + 1].qkv.accepts_slices(layer.down_proj.slices)
                                 for i, layer in enumerate(self.layers)]
             # a launch that leaves its K slices to the next one runs on the wide-tile kernel: a down that may do so

@@ -85,6 +85,28 @@ def make_sparse_plane(k: int, n: int, group: int = 128, density: float = 0.25, s
     return bits, scale, mask
 
 
+def with_device_sparse_plane(mod, density: float = 0.1, seed: int = 0):
+    """`mod` (an HLQLinear on the GPU) with a random block-sparse extra plane held as blocks, drawn on the device:
+    every (32-channel tile, group) pair is a block with probability `density`, in the list order the kernels expect
+    (ascending tile, then ascending k start).  The dense buffers are shared with `mod`."""
+    import torch
+
+    from .hlq_linear import HLQLinear, sparse_index
+
+    dev = mod.planes.device
+    g = torch.Generator(device=dev).manual_seed(seed)
+    k, n, group = mod.in_features, mod.out_features, mod.group_size
+    tiles = (n + 31) // 32
+    pick = torch.rand(tiles, k // group, generator=g, device=dev) < density
+    where = pick.nonzero()                                          # row-major: tile, then group
+    nblk = where.shape[0]
+    mask = torch.stack([where[:, 0] * 32, where[:, 1] * group], 1).cpu().numpy().astype(np.uint32)
+    index = torch.from_numpy(sparse_index(mask, k, n, group)).to(dev)
+    blocks = torch.randint(0, 256, (nblk, 32, group // 8), generator=g, device=dev, dtype=torch.uint8)
+    scales = (torch.rand(nblk, 32, generator=g, device=dev) * 0.004 + 0.001).to(torch.float16)
+    return HLQLinear(k, n, mod.bits, group, mod.planes, mod.scales, mod.zeros, mod.bias, (blocks, scales, index))
+
+
 # (K, N) of the LLaMA-3-8B projections and of the LLaMA-2-13B prefill shapes.
 LLAMA3_8B_SHAPES = {
     "q_proj": (4096, 4096), "k_proj": (4096, 1024), "v_proj": (4096, 1024), "o_proj": (4096, 4096),

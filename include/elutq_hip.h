@@ -373,6 +373,13 @@ int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void
  * workspace must hold elutq_hlq_sparse_workspace_bytes(K, N, bits, group, M) bytes, zero-filled
  * once like every workspace.  elutq_hlq_sparse_dequant_add_f16: the plane added to a dense fp16
  * W [N][K] (after elutq_hlq_dequant_f16; W is then rounded twice).
+ *
+ * elutq_hlq_sparse_gemv_fused_f16: elutq_hlq_sparse_gemv_f16 in a decode step, i.e. with the prologue
+ * and residual of elutq_hlq_gemv_fused_f16 (`fusion`, `ksplit`, `waves` as there; arm_gemm takes
+ * use_sparse on any call, arm_gemm.cpp:894-920, so a layer held as blocks can stand anywhere in
+ * llama.cpp:204-617).  The plane's launch forms the projection's input from the same stored vectors
+ * with the same operations as the dense launch's prologue.  K slices handed over by, or left to,
+ * another launch (d_slices_in / d_slices_out) are refused: ELUTQ_ERR_TUNING.
  */
 size_t elutq_hlq_sparse_index_bytes(int N, int nblk);
 int elutq_hlq_sparse_index_host(const uint32_t *h_mask, int mask_len, int K, int N, int group, void *h_index_out);
@@ -385,6 +392,11 @@ int elutq_hlq_sparse_gemm_f16(const void *d_planes, const void *d_scales, const 
                               const void *d_blocks, const void *d_blk_scales, const void *d_index, int nblk,
                               const void *d_x, void *d_y, int M, int K, int N, int bits, int group,
                               void *d_workspace, size_t workspace_bytes, void *stream);
+int elutq_hlq_sparse_gemv_fused_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                                    const void *d_blocks, const void *d_blk_scales, const void *d_index, int nblk,
+                                    const void *d_x, void *d_y, int K, int N, int bits, int group,
+                                    void *d_workspace, size_t workspace_bytes, void *stream,
+                                    const elutq_gemv_fusion *fusion, int ksplit, int waves);
 int elutq_hlq_sparse_dequant_add_f16(const void *d_blocks, const void *d_blk_scales, const void *d_index, int nblk,
                                      void *d_w, int K, int N, int group, void *stream);
 

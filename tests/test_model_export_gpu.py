@@ -64,16 +64,15 @@ def test_decoder_from_export_tree(cuda, tmp_path, kind, impl):
 def test_decoder_with_sparse_extra_planes(cuda, tmp_path):
     """Layers with a sparse extra plane: by default the plane is written out as one more dense plane at load, so the
     fused step runs them (q carries three planes, k and v two: the concatenation lifts k and v); held as blocks they
-    run through the plain HLQLinear calls of the PyTorch-glue step, and the fused step refuses them."""
+    run through the plain HLQLinear calls of the PyTorch-glue step, or through the fused step with a launch of the
+    plane in front of each such projection (q|k|v: the block lists concatenated like the dense buffers)."""
     src, dst, plain = str(tmp_path / "export"), str(tmp_path / "repacked"), str(tmp_path / "plain")
     write_tiny_export(src, sparse_on=("down_proj", "q_proj"))
     write_tiny_export(plain)
     repack_tree(src, dst)
-    with pytest.raises(NotImplementedError):
-        LlamaDecoder.from_export(src, TINY, device=cuda, impl="hip", sparse_mode="blocks")
     outs = []
     for root, kw in ((src, dict(impl="hip")), (dst, dict(impl="hip")), (src, dict(fuse=False, impl="torch", sparse_mode="blocks")),
-                     (plain, dict(impl="hip"))):
+                     (plain, dict(impl="hip")), (src, dict(impl="hip", sparse_mode="blocks"))):
         m = LlamaDecoder.from_export(root, TINY, device=cuda, **kw)
         m.fill_cache(9, seed=3)
         m.token.fill_(5)
@@ -86,6 +85,22 @@ def test_decoder_with_sparse_extra_planes(cuda, tmp_path):
     # fused step on dense planes against the glue step on blocks: the first step's logits
     a, b = outs[0][1][:1].float(), outs[2][1][:1].float()
     assert float((a - b).abs().max()) <= 2e-2 * float(b.abs().max())
+    # the fused step on blocks: against the glue step on the same blocks and against the fused step on dense planes
+    fb = outs[4][0]
+    assert fb.layers[0].down_proj.sparse_count > 0 and fb.layers[0].qkv.sparse_count > 0 and fb.layers[0].qkv.bits == 2
+    assert fb.layers[0].qkv.sparse_count == outs[2][0].layers[0].q_proj.sparse_count
+    c = outs[4][1][:1].float()
+    assert float((c - b).abs().max()) <= 2e-2 * float(b.abs().max())
+    assert float((c - a).abs().max()) <= 2e-2 * float(a.abs().max())
+    assert not torch.equal(outs[4][1], outs[3][1])
+    # ... and replayed from a graph: the same logits as its eager steps
+    fb.fill_cache(9, seed=3)
+    fb.token.fill_(5)
+    fb.capture()
+    for i in range(3):
+        fb.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(fb._logits, outs[4][1][i:i + 1])
     # every layer held as blocks equals its own dequantized weight applied densely
     x = torch.randn(3, TINY.ffn, device=cuda).to(torch.float16)
     mod = outs[2][0].layers[1].down_proj

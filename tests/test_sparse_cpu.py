@@ -47,14 +47,24 @@ def test_index_is_a_row_pointer_over_channel_tiles():
     k, n, g = 512, 160, 128
     _, _, mask = make_sparse_plane(k, n, g, 0.5, seed=3)
     idx = sparse_index(mask, k, n, g)
-    tiles = n // 32
-    assert idx.dtype == np.int32 and idx.size == tiles + 1 + mask.shape[0]
+    tiles, nblk, head = n // 32, mask.shape[0], 16
+    assert idx.dtype == np.int32 and idx.size == tiles + 1 + nblk + tiles * head
     counts = np.bincount(mask[:, 0] // 32, minlength=tiles)
-    assert np.array_equal(idx[:tiles + 1], np.concatenate([[0], np.cumsum(counts)]))
-    assert np.array_equal(idx[tiles + 1:], mask[:, 1].astype(np.int32))
+    ptr = np.concatenate([[0], np.cumsum(counts)])
+    assert np.array_equal(idx[:tiles + 1], ptr)
+    assert np.array_equal(idx[tiles + 1:tiles + 1 + nblk], mask[:, 1].astype(np.int32))
+    # behind it, per tile, the k starts of its first 16 blocks once more (-1: no such block)
+    h = idx[tiles + 1 + nblk:].reshape(tiles, head)
+    for t in range(tiles):
+        want = mask[ptr[t]:ptr[t + 1], 1].astype(np.int32)[:head]
+        assert np.array_equal(h[t, :want.size], want) and np.all(h[t, want.size:] == -1)
     # ragged N: the last tile is partial
-    assert sparse_index(np.array([[96, 0]], np.uint32), 128, 100, 128).tolist() == [0, 0, 0, 0, 1, 0]
-    assert sparse_index(np.zeros((0, 2), np.uint32), 128, 64, 64).tolist() == [0, 0, 0]
+    assert sparse_index(np.array([[96, 0]], np.uint32), 128, 100, 128).tolist() == [0, 0, 0, 0, 1, 0] + [-1] * 48 + [0] + [-1] * 15
+    assert sparse_index(np.zeros((0, 2), np.uint32), 128, 64, 64).tolist() == [0, 0, 0] + [-1] * 32
+    # more blocks on a tile than the head holds: the first 16 there, all of them in the list
+    many = np.array([[0, 4 * i] for i in range(20)], np.uint32)
+    idx = sparse_index(many, 256, 32, 128)
+    assert idx[:2].tolist() == [0, 20] and idx[2:22].tolist() == [4 * i for i in range(20)] and idx[22:].tolist() == [4 * i for i in range(16)]
 
 
 @pytest.mark.parametrize("mask", [

@@ -10,6 +10,7 @@ import numpy as np
 import pytest
 import torch
 
+from elutq_amd import _lib
 from elutq_amd.export_io import SparseBlocks, write_export_dir
 from elutq_amd.hlq_linear import GemvGroup, HLQLinear
 from elutq_amd.repack import repack_tree
@@ -208,11 +209,131 @@ def test_dense_form_matches_oracle(cuda, k, n, bits, group, density):
     assert np.max(np.abs(w - wref)) <= 2.0 ** -11 * np.max(np.abs(wref))
 
 
-def test_no_fused_or_grouped_launch_for_sparse_layers(cuda):
+def _fused_case(k, n, bits, group, density, seed, dev):
+    L, sp, mod = build(k, n, bits, group, density, seed, dev)
+    g = torch.Generator(device=dev).manual_seed(seed)
+    res = torch.randn(1, n, generator=g, device=dev).half()
+    out = torch.full((1, n), float("nan"), dtype=torch.float16, device=dev)
+    ws = torch.zeros(mod.workspace_bytes, dtype=torch.uint8, device=dev)
+    return L, sp, mod, g, res, out, ws
+
+
+FUSED_SHAPES = [(1024, 256, 2, 128, 0.3), (512, 96, 3, 64, 0.5), (4096, 1024, 2, 128, 0.1), (1088, 160, 2, 64, 0.4),
+                (4096, 4096, 2, 128, 0.05)]
+
+
+@pytest.mark.parametrize("k,n,bits,group,density", FUSED_SHAPES)
+@pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 4), (2, 16), (_lib.GEMV_NARROW16, 0), (_lib.GEMV_NARROW32, 0),
+                                          (_lib.GEMV_WIDE, 0)])
+def test_fused_rmsnorm_prologue_and_residual(cuda, k, n, bits, group, density, ksplit, waves):
+    """The layer inside a decode step: RMSNorm in front (formed by both launches, the plane's and the dense one's),
+    bias, the plane's fp32 term and the residual behind, one rounding."""
+    L, sp, mod, g, res, out, ws = _fused_case(k, n, bits, group, density, k + n + 3, cuda)
+    print(f"sparse fused gemv K={k} N={n} w{bits}g{group} ksplit={ksplit} waves={waves} blocks={mod.sparse_count}", flush=True)
+    mod.ksplit, mod.waves = ksplit, waves
+    x = (torch.randn(1, k, generator=g, device=cuda) * 3).half()
+    w = (1 + 0.1 * torch.randn(k, generator=g, device=cuda)).half()
+    eps = 1e-5
+    mod.gemv_fused(x, out, ws, prologue=1, norm_weight=w, eps=eps, residual=res)
+    xf = x.float()
+    h = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).half()
+    ref = (O.gemv_sparse_f64(h.cpu().numpy()[0], L.w_quant, L.w_scale, L.w_zero, sp, L.bias)
+           + res.cpu().numpy()[0].astype(np.float64))
+    y = out.cpu().numpy()[0]
+    assert O.rel_err(y, ref) <= TOL
+    # against the unfused calls on the normalised input (1 / rms is summed in another order there: h may differ
+    # in the last fp16 bit of a few elements)
+    unfused = mod(h).float() + res.float()
+    assert float((out.float() - unfused).abs().max()) <= 2e-2 * float(unfused.abs().max())
+    # no prologue, no residual: the same bits as the plain entry point (which launches the library's own shape)
+    mod.gemv_fused(h, out, ws)
+    if (ksplit, waves) == (0, 0):
+        assert torch.equal(out, mod(h))
+    else:
+        assert float((out.float() - mod(h).float()).abs().max()) <= 2.0 ** -9 * float(unfused.abs().max())
+    assert int(ws[:65536].count_nonzero()) == 0        # the head of the workspace is left zero-filled
+
+
+@pytest.mark.parametrize("k,n,bits,group,density", [(1024, 256, 2, 128, 0.3), (1536, 192, 4, 64, 0.2), (960, 96, 2, 64, 0.5),
+                                                     (14336, 4096, 2, 128, 0.02)])
+@pytest.mark.parametrize("ksplit", [0, _lib.GEMV_NARROW32, _lib.GEMV_WIDE])
+def test_fused_silu_mul_prologue(cuda, k, n, bits, group, density, ksplit):
+    import torch.nn.functional as F
+    if ksplit == _lib.GEMV_NARROW32 and k > 8192:
+        pytest.skip("the narrow-tile kernel holds the tables of at most 8192 activations")
+    L, sp, mod, g, res, out, ws = _fused_case(k, n, bits, group, density, k + n + 5, cuda)
+    print(f"sparse fused silu gemv K={k} N={n} w{bits}g{group} ksplit={ksplit} blocks={mod.sparse_count}", flush=True)
+    mod.ksplit = ksplit
+    gu = torch.randn(1, 2 * k, generator=g, device=cuda).half()
+    mod.gemv_fused(gu, out, ws, prologue=2, residual=res)
+    act = (F.silu(gu[:, :k].float()) * gu[:, k:].float()).half()
+    ref = (O.gemv_sparse_f64(act.cpu().numpy()[0], L.w_quant, L.w_scale, L.w_zero, sp, L.bias)
+           + res.cpu().numpy()[0].astype(np.float64))
+    assert O.rel_err(out.cpu().numpy()[0], ref) <= TOL
+
+
+def test_fused_wide_layer_runs_of_column_blocks(cuda):
+    """gate|up of LLaMA-3-8B with a sparse plane: more column blocks than compute units, so the dense launch
+    walks runs of them; the plane's term and the RMSNorm go through the same launch pair."""
+    k, n = 4096, 28672
+    L, sp, mod, g, res, out, ws = _fused_case(k, n, 2, 128, 0.05, 91, cuda)
+    x = (torch.randn(1, k, generator=g, device=cuda) * 2).half()
+    w = (1 + 0.1 * torch.randn(k, generator=g, device=cuda)).half()
+    mod.gemv_fused(x, out, ws, prologue=1, norm_weight=w, eps=1e-5)
+    xf = x.float()
+    h = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5) * w.float()).half()
+    # the oracle on 128 sampled channel tiles (4096 columns), the plane's blocks on those tiles renumbered
+    tiles = np.sort(np.random.default_rng(n).choice(n // 32, 128, replace=False))
+    tiles[0], tiles[-1] = 0, n // 32 - 1
+    idx = (tiles[:, None] * 32 + np.arange(32)[None, :]).reshape(-1)
+    pos = {int(t): i for i, t in enumerate(tiles)}
+    keep = [i for i, c in enumerate(sp.mask[:, 0]) if int(c) // 32 in pos]
+    sub_mask = np.array([[pos[int(sp.mask[i, 0]) // 32] * 32, sp.mask[i, 1]] for i in keep], np.uint32)
+    sub = O.SparsePlane(sp.bits[keep], sp.scale[keep], sub_mask, 128)
+    assert len(keep) > 100
+    ref = O.gemv_sparse_f64(h.cpu().numpy()[0], L.w_quant[:, idx], L.w_scale[:, idx], L.w_zero[idx], sub, L.bias[idx])
+    y = out.cpu().numpy()[0]
+    assert O.rel_err(y[idx], ref) <= TOL
+    # without the plane the result differs: the blocks do take part
+    dense = HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, 128, L.bias, cuda)
+    yd = torch.empty_like(out)
+    dense.gemv_fused(x, yd, ws, prologue=1, norm_weight=w, eps=1e-5)
+    assert not torch.equal(yd, out)
+
+
+def test_fused_integer_inputs_bit_exact(cuda):
+    """SiLU(gate) * up with gate = 0 is 0, and a unit norm weight on inputs whose mean square is 1 - eps leaves
+    integers: exact arithmetic in both launches, so the result is the float64 one."""
+    k, n, group = 512, 128, 128
+    r = np.random.default_rng(5)
+    wq = O.pack_planes(r.integers(0, 2, (2, n, k), dtype=np.uint8))
+    ws_ = np.stack([np.full((n, k // group), 0.5), np.full((n, k // group), 1.0)]).astype(np.float16)
+    wz = np.full((n, k // group), -0.5, np.float16)
+    b, _, mk = make_sparse_plane(k, n, group, 0.5, seed=6)
+    s = np.full((mk.shape[0], 32), 2.0, np.float16)
+    sp = O.SparsePlane(b, s, mk, group)
+    mod = HLQLinear.from_export_arrays(wq, ws_, wz, group, None, cuda, SparseBlocks(sp.packed, s, mk), sparse_mode="blocks")
+    x = r.choice(np.array([-1.0, 1.0], np.float16), (1, k))          # mean square exactly 1
+    xd = torch.from_numpy(x).to(cuda)
+    out = torch.empty(1, n, dtype=torch.float16, device=cuda)
+    ws = torch.zeros(mod.workspace_bytes, dtype=torch.uint8, device=cuda)
+    one = torch.ones(k, dtype=torch.float16, device=cuda)
+    mod.gemv_fused(xd, out, ws, prologue=1, norm_weight=one, eps=0.0)
+    want = x.astype(np.float64) @ O.dequantize_sparse(wq, ws_, wz, sp).T
+    assert np.array_equal(out.cpu().numpy().astype(np.float64), want)
+
+
+def test_fused_refuses_slices_and_group_refuses_sparse(cuda):
     L, sp, mod = build(256, 64, 2, 128, 0.5, 81, cuda)
     x = torch.from_numpy(L.x).to(cuda)
     out = torch.empty(1, 64, dtype=torch.float16, device=cuda)
-    with pytest.raises(NotImplementedError):
-        mod.gemv_fused(x, out, torch.zeros(1 << 20, dtype=torch.uint8, device=cuda))
+    ws = torch.zeros(mod.workspace_bytes, dtype=torch.uint8, device=cuda)
+    sl = torch.zeros(4, 256, dtype=torch.float32, device=cuda)
+    with pytest.raises(ValueError):
+        mod.gemv_fused(x, out, ws, prologue=1, norm_weight=torch.ones(256, dtype=torch.float16, device=cuda), slices_in=sl)
+    with pytest.raises(ValueError):
+        mod.gemv_fused(x, out, ws, slices_out=torch.zeros(4, 64, dtype=torch.float32, device=cuda))
+    with pytest.raises(_lib.ElutqError):                 # the dense part's workspace alone is too small
+        mod.gemv_fused(x, out, ws[:mod._ws_bytes])
     with pytest.raises(NotImplementedError):
         GemvGroup([mod], [x], [out])
