@@ -18,7 +18,7 @@
 // the same operations (prologue_value), from the same stored vectors.
 //
 // The block bits and scales stay exactly as the files hold them -- [block][32 channels][G/8
-// bytes] is already what a wave wants: 8 consecutive lanes own the 8 k-eighths of one channel, so a
+// bytes] is already what a wave wants: consecutive lanes own consecutive parts of one channel's k, so a
 // block is one contiguous 32*G/8-byte read -- and the pair list becomes an index by channel tile.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -325,6 +325,8 @@ int launch_sparse_plane(SparseArgs a, const void *d_x, float *d_extra, int M, in
     a.extra = d_extra;
     a.M = M;
     if (M == 1) {
+        // the kernel reads block bits as dwords and activations as fp16 pairs
+        if (((uintptr_t)a.blocks & 3) != 0 || ((uintptr_t)d_x & 3) != 0 || ((uintptr_t)a.norm_w & 3) != 0) return ELUTQ_ERR_SHAPE;
         // as many waves per tile as leave all tiles resident at once (32 waves per compute unit)
         const int tiles = sp_tiles(a.N);
         const int waves = tiles * 16 <= HLQ_NUM_CU * 32 ? 16 : (tiles * 8 <= HLQ_NUM_CU * 32 ? 8 : 4);

@@ -371,7 +371,7 @@ int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void
  * `stream`: the plane's term in fp32 into the tail of the workspace, then the dense kernel, which
  * adds it before its one rounding to fp16.  `bits` counts the dense planes (base_bit).  The
  * workspace must hold elutq_hlq_sparse_workspace_bytes(K, N, bits, group, M) bytes, zero-filled
- * once like every workspace.  elutq_hlq_sparse_dequant_add_f16: the plane added to a dense fp16
+ * once like every workspace; d_blocks and d_x (and a norm weight) must be 4-byte aligned (ELUTQ_ERR_SHAPE).  elutq_hlq_sparse_dequant_add_f16: the plane added to a dense fp16
  * W [N][K] (after elutq_hlq_dequant_f16; W is then rounded twice).
  *
  * elutq_hlq_sparse_gemv_fused_f16: elutq_hlq_sparse_gemv_f16 in a decode step, i.e. with the prologue
