@@ -61,6 +61,7 @@ constexpr int depth_of(int bits) { return bits == 3 ? 6 : (bits == 4 ? 8 : 4); }
 //   GEMV_FUSED  prologue, residual and the fp32 term `a.extra` as `a` says (the decode step's launches)
 //   GEMV_PLAIN  none of them (their fields of `a` are not read)
 //   GEMV_EXTRA  plain, plus `a.extra`, added before the output is rounded
+//   GEMV_INT8   plain, tables quantized to int8 per group as the reference's int8-LUT variant does
 template <int BITS, bool G64, int NSLOT, bool MULTI, int VAR, bool PAIRED>
 __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, int ncb_run, unsigned char *smem, int &red_sel)
 {
@@ -72,7 +73,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     constexpr bool PLAIN = VAR != GEMV_FUSED;
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
-    const HLQ_GLOBAL float *extra = VAR == GEMV_PLAIN ? nullptr : a.extra;
+    const HLQ_GLOBAL float *extra = (VAR == GEMV_FUSED || VAR == GEMV_EXTRA) ? a.extra : nullptr;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
@@ -141,8 +142,12 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
 
     // ... the tables are built as soon as the activations are in (a wave that first queued all
     // its weight loads would sit in the memory pipeline's back-pressure instead) ...
-    if (lane < nchunks)
-        build_chunk(prologue, raw, raw2, rstd, lut + (size_t)lane * TBL_BYTES, xs_inv + (lane >> 4), (lane & 15) == 0, lane);
+    if (lane < nchunks) {
+        if constexpr (VAR == GEMV_INT8)
+            build_chunk_int8<G64>(raw, lut + (size_t)lane * TBL_BYTES, xs_inv + (lane >> 4), (lane & 15) == 0);
+        else
+            build_chunk(prologue, raw, raw2, rstd, lut + (size_t)lane * TBL_BYTES, xs_inv + (lane >> 4), (lane & 15) == 0, lane);
+    }
     asm volatile("" ::: "memory");
 
     // ... and the rest of the run's loads follow.
@@ -155,7 +160,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         load_chunk<PLAIN>(a, prologue, K, hlq_x_load_k(kc, K), raw, raw2);
         if (sliced) raw = stage[hlq_stage_index(k0, ci, K)];
         if (kc >= (size_t)K) raw = make_uint2(0u, 0u);
-        build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0, lane);
+        if constexpr (VAR == GEMV_INT8)
+            build_chunk_int8<G64>(raw, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0);
+        else
+            build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0, lane);
     }
     HLQ_STAMP(1);
     // The tables were written by this wave and are read by this wave: LDS executes a wave's
@@ -357,7 +365,7 @@ int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
     if (!allow_big_lds((const void *)kern, lds, MAX_LDS, big_lds_done)) return ELUTQ_ERR_HIP;
     // more tiles than CUs and runs that fit the slots: runs of column blocks, one workgroup per CU
     const int run = (a.ncb * a.ksplit + NUM_CU_RUN - 1) / NUM_CU_RUN;
-    if (VAR != GEMV_EXTRA && run > 1 && a.spw <= NSLOT && waves == 16) {       // (plain plus extra term: no run instances)
+    if (VAR != GEMV_EXTRA && VAR != GEMV_INT8 && run > 1 && a.spw <= NSLOT && waves == 16) {       // (plain plus extra term, int8 tables: no run instances)
         auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT, PAIRED, PLAIN>;
         static bool big_lds_run_done[64] = {};
         if (!allow_big_lds((const void *)kern_run, lds, MAX_LDS, big_lds_run_done)) return ELUTQ_ERR_HIP;
@@ -382,6 +390,10 @@ int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 template <int BITS, bool G64, int NSLOT>
 int launch_gemv_n(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
+    if (a.lut_int8) {        // plain calls only, one load pattern
+        if (a.prologue != 0 || a.residual || a.extra || a.defer || a.n_slices_in != 0) return ELUTQ_ERR_TUNING;
+        return launch_gemv_pp<BITS, G64, NSLOT, false, GEMV_INT8>(a, waves, lds, stream);
+    }
     if constexpr (MetaGroup<BITS, G64>::fits(NSLOT)) {
         if (paired_ok<BITS, G64, NSLOT>(a.spw, a.ups, a.ksplit)) return launch_gemv_p<BITS, G64, NSLOT, true>(a, waves, lds, stream);
     }
@@ -541,7 +553,7 @@ struct LaunchShape {
 };
 
 // `allow_narrow`: the call has nothing the narrow-tile kernel lacks (extra term, handed-over slices).
-int plan_launch(const HlqGeo &g, int bits, int ksplit, int waves, bool allow_narrow, LaunchShape &sh)
+int plan_launch(const HlqGeo &g, int bits, int ksplit, int waves, bool allow_narrow, LaunchShape &sh, bool lut_only = false)
 {
     sh.mfma = false;
     sh.narrow = 0;
@@ -572,7 +584,7 @@ int plan_launch(const HlqGeo &g, int bits, int ksplit, int waves, bool allow_nar
     // measured on MI355X: the matrix-core kernel streams large layers as fast as the LUT kernel but a launch of one
     // tile per workgroup takes 0.5-1 us longer (its A operands cost more to build than the tables), so the
     // library's own choice is the LUT kernel throughout
-    sh.mfma = g_gemv_engine == ELUTQ_GEMV_ENGINE_MFMA;
+    sh.mfma = !lut_only && g_gemv_engine == ELUTQ_GEMV_ENGINE_MFMA;
     if (sh.mfma && g.K % HLQ_UNIT != 0) return ELUTQ_ERR_TUNING;      // the matrix-core kernel takes whole units only
     choose_shape(g, ksplit, waves);
     int ups = (g.U + ksplit - 1) / ksplit;
@@ -648,19 +660,21 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
 
 // The fused GEMV with an fp32 vector [N] added to every output before it is rounded to fp16
 // (the block-sparse extra plane of a use_sparse layer, computed by another kernel on the same stream).
-int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
-                        const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
-                        size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,
-                        int waves, const float *d_extra)
+// `lut_int8`: the wide-tile LUT kernel's instance with int8 tables (plain calls only).
+static int gemv_launch(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                       const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
+                       size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,
+                       int waves, const float *d_extra, bool lut_int8)
 {
     int rc = check_shape(K, N, bits, group);
     if (rc != ELUTQ_OK) return rc;
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     LaunchShape sh;
-    const bool allow_narrow = !(fusion && fusion->d_slices_out);
-    rc = plan_launch(g, bits, ksplit, waves, allow_narrow, sh);
+    const bool allow_narrow = !(fusion && fusion->d_slices_out) && !lut_int8;
+    rc = plan_launch(g, bits, ksplit, waves, allow_narrow, sh, lut_int8);
     if (rc != ELUTQ_OK) return rc;
+    if (lut_int8 && (sh.mfma || sh.narrow || fusion || d_extra)) return ELUTQ_ERR_TUNING;
     ksplit = sh.ksplit; waves = sh.waves;
     const int ups = sh.ups;
 
@@ -677,7 +691,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     a.spw = wp.spw; a.nuw_max = wp.nuw_max; a.wave_lds = wp.wave_lds;
     a.partial = nullptr; a.counters = nullptr; a.meet_slots = 0;
     a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
-    a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr;
+    a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr; a.lut_int8 = 0;
     if (fusion) {
         if (fusion->prologue < 0 || fusion->prologue > 2) return ELUTQ_ERR_TUNING;
         if (fusion->prologue == 1 && !fusion->d_norm_weight) return ELUTQ_ERR_NULL;
@@ -687,6 +701,7 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
         a.residual = (const HLQ_GLOBAL uint16_t *)fusion->d_residual;
     }
     a.extra = (const HLQ_GLOBAL float *)d_extra;
+    a.lut_int8 = lut_int8 ? 1 : 0;
     size_t stage_bytes = 0;
     if (fusion && fusion->n_slices_in != 0) {
         // x arrives as a base vector plus the unsummed K slices of the launch that produced it
@@ -725,6 +740,24 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
     if (sh.narrow) return hlq_gemv_narrow_launch(&a, sizeof(a), bits, group, sh.narrow, stage_bytes, stream);
     if (sh.mfma) return hlq_gemv_mfma_launch(&a, sizeof(a), bits, group, waves, stage_bytes, stream);
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves) + stage_bytes, (hipStream_t)stream);
+}
+
+int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                        const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
+                        size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,
+                        int waves, const float *d_extra)
+{
+    return gemv_launch(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace, workspace_bytes,
+                       stream, fusion, ksplit, waves, d_extra, false);
+}
+
+extern "C" int elutq_hlq_gemv_int8lut_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                                          const void *d_x, void *d_y, int K, int N, int bits, int group,
+                                          void *d_workspace, size_t workspace_bytes, void *stream)
+{
+    // the library's own launch shape on wide tiles, whatever engine is selected for the exact GEMV
+    return gemv_launch(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace, workspace_bytes,
+                       stream, nullptr, ELUTQ_GEMV_WIDE, 0, nullptr, true);
 }
 
 extern "C" int elutq_hlq_set_gemv_engine(int engine)
@@ -877,7 +910,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
             a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + poff[i]);
         }
         a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
-        a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr;
+        a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr; a.lut_int8 = 0;
         const int ns = a.spw < depth_of(bits) ? a.spw : depth_of(bits);
         if (ns > nslot) nslot = ns;
         const size_t l = gemv_lds_bytes(sh.ups, bits, 16);

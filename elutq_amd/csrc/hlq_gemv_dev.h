@@ -54,6 +54,7 @@ struct GemvArgs {
     int n_slices_in;                      // > 0: x = fp16(sum of slices_in in order + x), prologue 1 only
     const HLQ_GLOBAL float *slices_in;    // fp32 [n_slices_in][K]
     HLQ_GLOBAL uint16_t *x_out;           // fp16 [K] or null: the combined x, written by workgroup (0, 0)
+    int lut_int8;                         // host side only: launch the instance whose tables are quantized to int8 (GEMV_INT8)
 };
 
 #ifdef HLQ_TIMING
@@ -326,6 +327,47 @@ __device__ __forceinline__ void build_chunk(int prologue, uint2 raw, uint2 raw2,
     if (leader) *half = make_float2(s, inv);
 }
 
+// The same table with the entries quantized as the reference's int8-LUT variant quantizes them
+// (t_mac_g4_groupsize32_calculate_lut_impl, C++/ops/src/arm/arm_t_mac_kernal.cpp:15-93): every entry is the fp16
+// sum of its activations added in ascending order (:22-48), the quantization group's scale is
+// fp16(max|entry| / 127) (:50) and an entry becomes round-to-nearest-even(fp16(entry / scale)), saturated to int8
+// (:59-90).  The entries are stored as int32 like the exact ones, so the lookups and their integer sums are the
+// same code; *half gets the scale in place of the exact tables' power of two.  A group of zeros has scale 0 and
+// zero entries.  The 16 lanes of a DPP row cover 64 activations: one group at G = 64, half of one at G = 128,
+// where the rows of a unit's two halves exchange their maxima.
+template <bool G64>
+__device__ __forceinline__ void build_chunk_int8(uint2 raw, unsigned char *tbl, float2 *half, bool leader)
+{
+    const _Float16 a[4] = {__builtin_bit_cast(_Float16, (uint16_t)(raw.x & 0xffffu)), __builtin_bit_cast(_Float16, (uint16_t)(raw.x >> 16)),
+                           __builtin_bit_cast(_Float16, (uint16_t)(raw.y & 0xffffu)), __builtin_bit_cast(_Float16, (uint16_t)(raw.y >> 16))};
+    float s = ((float)a[0] + (float)a[1]) + ((float)a[2] + (float)a[3]);
+    HLQ_ROW_REDUCE(s, op_add);
+    _Float16 e[16];
+    e[0] = (_Float16)0.f;
+    float m = 0.f;
+#pragma unroll
+    for (int g = 1; g < 16; g++) {
+        const int top = g >= 8 ? 3 : (g >= 4 ? 2 : (g >= 2 ? 1 : 0));          // the activation added last
+        e[g] = (g & ~(1 << top)) ? (_Float16)(e[g & ~(1 << top)] + a[top]) : a[top];
+        m = fmaxf(m, fabsf((float)e[g]));
+    }
+    HLQ_ROW_REDUCE(m, op_max);
+    if (!G64) m = fmaxf(m, __shfl_xor(m, 16, 64));
+    const float scale = (float)(_Float16)(m / 127.0f);
+    int q[16];
+#pragma unroll
+    for (int g = 0; g < 16; g++) {
+        const float r = rintf((float)(_Float16)((float)e[g] / scale));
+        q[g] = scale != 0.f ? (int)fminf(fmaxf(r, -128.f), 127.f) : 0;
+    }
+    // (the quarters go out in table order: picking them by the lane's rotation, as build_chunk does to spread the
+    // stores over the banks, would cost a chain of selects per entry here)
+    int4 *dst = (int4 *)tbl;
+#pragma unroll
+    for (int i = 0; i < 4; i++) dst[i] = make_int4(q[4 * i], q[4 * i + 1], q[4 * i + 2], q[4 * i + 3]);
+    if (leader) *half = make_float2(s, scale);
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
 // outstanding global load of the wave (its fence covers all address spaces), which here would
 // be the weight loads that are meant to stay in flight across the barrier.
@@ -522,7 +564,8 @@ __device__ __forceinline__ void progress_prio(int done, int total)
 //   GEMV_FUSED  prologue, residual and the fp32 term `extra` as the argument block says (the decode step's launches)
 //   GEMV_PLAIN  none of them (their fields are not read)
 //   GEMV_EXTRA  plain, plus the fp32 term `extra` added before the output is rounded
-enum { GEMV_FUSED = 0, GEMV_PLAIN = 1, GEMV_EXTRA = 2 };
+//   GEMV_INT8   plain, with the tables quantized to int8 per group (build_chunk_int8)
+enum { GEMV_FUSED = 0, GEMV_PLAIN = 1, GEMV_EXTRA = 2, GEMV_INT8 = 3 };
 
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
 template <int B, int E, typename F>

@@ -272,6 +272,24 @@ class HLQLinear(nn.Module):
         y = y.reshape(*x.shape[:-1], self.out_features)
         return y if in_dtype == torch.float16 else y.to(in_dtype)
 
+    def gemv_int8lut(self, x: torch.Tensor) -> torch.Tensor:
+        """Batch-1 GEMV with the lookup tables quantized to int8 per group, as the reference's int8-LUT variant
+        quantizes them (elutq_hlq_gemv_int8lut_f16; arm_gemv.cpp:4-34, arm_t_mac_kernal.cpp:15-93): lossy."""
+        if self.sparse_count:
+            raise NotImplementedError("the int8-LUT GEMV takes dense layers only")
+        if x.dtype != torch.float16 or x.numel() != self.in_features or not x.is_cuda:
+            raise ValueError("x must be fp16 [in_features] on the GPU")
+        x = x.contiguous()
+        y = torch.empty((1, self.out_features), dtype=torch.float16, device=x.device)
+        ws = _workspace(x.device, self._ws_bytes)
+        rc = _lib.lib().elutq_hlq_gemv_int8lut_f16(
+            self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
+            self.bias.data_ptr() if self.bias is not None else None, x.data_ptr(), y.data_ptr(), self.in_features,
+            self.out_features, self.bits, self.group_size, ws.data_ptr(), ws.numel(),
+            torch.cuda.current_stream(x.device).cuda_stream)
+        _lib.check(rc, "elutq_hlq_gemv_int8lut_f16")
+        return y
+
     def gemv_fused(self, x: torch.Tensor, out: torch.Tensor, ws: torch.Tensor, prologue: int = 0,
                    norm_weight: torch.Tensor | None = None, eps: float = 0.0,
                    residual: torch.Tensor | None = None, slices_out: torch.Tensor | None = None,

@@ -160,6 +160,24 @@ int elutq_hlq_gemv_f16_tuned(const void *d_planes, const void *d_scales, const v
                              int ksplit, int waves);
 
 /*
+ * The batch-1 GEMV with its lookup tables quantized to int8, the reference's int8-LUT variant
+ * (arm_gemv, C++/ops/src/arm/arm_gemv.cpp:4-34, which nothing in the reference calls): per
+ * quantization group of `group` activations the table entries -- fp16 subset sums of four activations --
+ * share one scale = fp16(max|entry| / 127) and become saturate_int8(round-to-nearest-even(entry / scale))
+ * (t_mac_g4_groupsize32_calculate_lut_impl, C++/ops/src/arm/arm_t_mac_kernal.cpp:15-93); the looked-up
+ * entries of a group are summed as integers and the sum is multiplied by that scale and the weight's scale
+ * (t_mac_g4_int8_update_impl, :258-362).  Here the weights stay HLQ layers -- a scale per plane and
+ * a zero point, of which the reference's uniform format (one scale, planes weighted 2^order, no zero)
+ * is the special case scale[b] = 2^b scale[0], zero = 0 -- the zero term uses the exact activation sums
+ * and everything after the integer sums is fp32 with one rounding to fp16.  A lossy mode (the tables
+ * keep seven bits): offered for parity with the reference's inventory, not used by any path here.
+ * Arguments as elutq_hlq_gemv_f16; runs on the wide-tile LUT kernel.
+ */
+int elutq_hlq_gemv_int8lut_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                               const void *d_x, void *d_y, int K, int N, int bits, int group,
+                               void *d_workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Batch-1 GEMV fused with the ops that surround a projection in a decoder layer, so a
  * decode step needs one launch where the reference runs two or three operators:
  *   prologue 1  x <- fp16(rmsnorm(x) * norm_weight)     launch_pre_rms_norm + arm_gemm

@@ -16,6 +16,10 @@ Reference lines each function follows (paths relative to the reference root):
   gemv_fp16_chain               C++/ops/src/arm/arm_gemm.cpp:248-308 +
                                 C++/ops/src/arm/arm_t_mac_kernal.cpp:364-469
   gemm_rows                     C++/ops/src/arm/arm_gemm.cpp:362-387
+  lut_int8                      C++/ops/src/arm/arm_t_mac_kernal.cpp:15-93  (int8 LUT, absmax/127 per group)
+  gemv_int8lut_f64              the HLQ sum evaluated exactly on those int8 tables
+  gemv_int8lut_chain_uniform    C++/ops/src/arm/arm_gemv.cpp:4-34 +
+                                C++/ops/src/arm/arm_t_mac_kernal.cpp:258-362 (no caller in the reference)
   sparse_export_arrays          C++/ops/src/arm/parameters.cpp:19-64 (what the loader reads)
   rearrange_sparse_reference    C++/ops/src/arm/arm_t_mac_kernal.cpp:554-647
   dequantize_sparse             C++/ops/src/arm/arm_t_mac_kernal.cpp:678-788 (which weights a block adds to)
@@ -37,7 +41,13 @@ producer in the reference (its exporter always writes use_sparse = false), so it
 format is the one the C++ loader and kernel consume; it is pinned by the cases
 that reduce to the dense path (blocks on every tile and group == one more dense
 plane, bit for bit; no blocks == the base layer), by brute force over the
-loader's index expressions, and by the C restatement bit for bit.
+loader's index expressions, and by the C restatement bit for bit.  The int8-LUT
+variant has no caller either: lut_int8 and the two GEMVs on its tables are pinned
+(tests/test_oracle_int8lut_pins.py) by a scalar re-derivation with Python floats,
+by invariance under power-of-two scaling and negation, by the cases where int8
+tables lose nothing (the exact oracle must come out) and by closed forms; the
+byte interleave of its update kernel is not restated, so the variant's WEIGHT
+ARRANGEMENT is "parity unpinned" (no loader, exporter or fixture holds one).
 """
 from __future__ import annotations
 
@@ -267,6 +277,88 @@ def gemm_rows(x, w_quant, w_scale, w_zero, group, bias=None, fused=True) -> np.n
     """m > 1 in the reference is a row loop over the GEMV (arm_gemm.cpp:380-385)."""
     x = np.asarray(x, dtype=np.float16)
     return np.stack([gemv_fp16_chain(r, w_quant, w_scale, w_zero, group, bias, fused) for r in x])
+
+
+# --------------------------------------------------------------------------- #
+# a14: the int8-LUT variant (arm_gemv.cpp:4-34; arm_t_mac_kernal.cpp:15-93 and 258-362).
+# Nothing in the reference calls it and its exporter writes no weights for it (one scale per
+# (channel, group) shared by all planes, planes weighted 2^order, no zero point).  What it
+# defines on its own is the quantization of the tables, which is what lut_int8 restates; the
+# update kernel's byte interleave (low nibbles to channels 0..15 of a tile, high nibbles to
+# channels 16..31, :296-318) is not restated: no loader or exporter produces that arrangement.
+# --------------------------------------------------------------------------- #
+def lut_int8(x, actk: int):
+    """x fp16 [K] -> (q int8 [K/4, 16], scale fp16 [K/actk]).  Per group of `actk` activations
+    (arm_t_mac_kernal.cpp:22-48): the fp16 subset sums of lut_float, scale = fp16(max|entry| / 127)
+    (:50), q = saturate_int8(round-to-nearest-even(fp16(entry / scale))) (:59-90; a NaN quotient,
+    0 / 0 in a group of zeros, converts to 0, an infinite one saturates)."""
+    lut = lut_float(x)
+    per = actk // 4
+    ng = lut.shape[0] // per
+    assert actk % 4 == 0 and ng * per == lut.shape[0]
+    scale = np.zeros(ng, dtype=np.float16)
+    q = np.zeros(lut.shape, dtype=np.int8)
+    for g in range(ng):
+        t = lut[g * per:(g + 1) * per]
+        m = np.max(np.abs(t))
+        s = (np.float32(m) / np.float32(127.0)).astype(np.float16)
+        scale[g] = s
+        with np.errstate(divide="ignore", invalid="ignore"):
+            d = (t.astype(np.float32) / np.float32(s)).astype(np.float16)
+        r = np.rint(d.astype(np.float32))
+        r = np.where(np.isnan(r), np.float32(0), r)
+        q[g * per:(g + 1) * per] = np.clip(r, -128, 127).astype(np.int8)
+    return q, scale
+
+
+def _nibbles(w_quant) -> np.ndarray:
+    """uint8 [bits, N, K/8] -> table index per chunk of 4 activations, uint8 [bits, N, K/4]
+    (low nibble = the byte's first four k, arm_t_mac_kernal.cpp:302-305)."""
+    w = np.asarray(w_quant, dtype=np.uint8)
+    return np.stack([w & 15, w >> 4], axis=-1).reshape(w.shape[0], w.shape[1], -1)
+
+
+def gemv_int8lut_f64(x, w_quant, w_scale, w_zero, group, bias=None) -> np.ndarray:
+    """The HLQ sum with the tables quantized by lut_int8, everything else exact:
+    y[n] = sum_g ( z[n,g] * sum_{k in g} x[k] + sum_b s[b,n,g] * scale[g] * sum_{chunks c in g} q[c, nibble_b(n, c)] )."""
+    x = np.asarray(x, dtype=np.float16).reshape(-1)
+    q, sc = lut_int8(x, group)
+    idx = _nibbles(w_quant)
+    bits, n, k4 = idx.shape
+    ng = k4 * 4 // group
+    looked = np.take_along_axis(np.broadcast_to(q.astype(np.int64)[None, None], (bits, n, k4, 16)),
+                                idx[..., None].astype(np.int64), axis=-1)[..., 0]
+    isum = looked.reshape(bits, n, ng, group // 4).sum(-1)
+    xs = x.astype(np.float64).reshape(ng, group).sum(-1)
+    y = (np.asarray(w_zero, dtype=np.float64) * xs[None, :]).sum(-1)
+    y = y + (np.asarray(w_scale, dtype=np.float64) * sc.astype(np.float64)[None, None, :] * isum).sum((0, 2))
+    return y if bias is None else y + np.asarray(bias).astype(np.float64)
+
+
+def gemv_int8lut_chain_uniform(x, w_quant, w_scale, actk: int) -> np.ndarray:
+    """arm_gemv (arm_gemv.cpp:4-34) on uniformly quantized planes, op for op in fp16 as
+    t_mac_g4_int8_update_impl (:258-362) orders them, every channel reading every chunk:
+    per plane `order`, per group: int16 sum of the looked-up int8 entries, converted to fp16;
+    c = (v * lut_scale) * w_scale for the first group, c += (v * lut_scale) * w_scale after it (:341-352);
+    out = c for plane 0, out += c * 2^order after it (:356-367).  w_scale fp16 [N, K/actk]."""
+    x = np.asarray(x, dtype=np.float16).reshape(-1)
+    q, sc = lut_int8(x, actk)
+    idx = _nibbles(w_quant)
+    bits, n, k4 = idx.shape
+    ng = k4 * 4 // actk
+    w_scale = np.asarray(w_scale, dtype=np.float16)
+    out = np.zeros(n, dtype=np.float16)
+    for order in range(bits):
+        c = None
+        for g in range(ng):
+            cs = slice(g * actk // 4, (g + 1) * actk // 4)
+            acc = np.take_along_axis(np.broadcast_to(q[cs].astype(np.int16)[None], (n, actk // 4, 16)),
+                                     idx[order][:, cs, None].astype(np.int64), axis=-1)[..., 0].sum(-1, dtype=np.int16)
+            v = acc.astype(np.float16)
+            t = _h(_h(v.astype(np.float32) * np.float32(sc[g])).astype(np.float32) * w_scale[:, g].astype(np.float32))
+            c = t if g == 0 else _h(c.astype(np.float32) + t.astype(np.float32))
+        out = c if order == 0 else _h(out.astype(np.float32) + _h(c.astype(np.float32) * np.float32(1 << order)).astype(np.float32))
+    return out
 
 
 # --------------------------------------------------------------------------- #
