@@ -6,8 +6,8 @@
 //
 //   y[m][n] = sum_g ( z[n,g] * (sum_{k in g} x[m][k])  +  sum_b s[b,n,g] * (sum_{k in g} x[m][k] * B_b[n][k]) )
 //
-// The inner sum over one group and one plane is a chain of v_mfma_f32_32x32x16_f16 whose B operand is the
-// plane itself as fp16 zeros and ones.  That operand is not computed: every byte of a plane dword (8 k of
+// The inner sum over one group and one plane is a chain of v_mfma_f32_32x32x16_f16 (up to 16 rows:
+// v_mfma_f32_16x16x32_f16) whose B operand is the plane itself as fp16 zeros and ones.  That operand is not computed: every byte of a plane dword (8 k of
 // one column) indexes a 256-row table in LDS whose row v holds the eight fp16 values of v's bits, so one
 // address instruction and one ds_read_b128 deliver the operand of one MFMA.  Every product is x or 0, the
 // chain accumulates in fp32 from zero, and its result is scaled once by the fp32 value of the group's
@@ -30,13 +30,11 @@ namespace {
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
+typedef float float4v __attribute__((ext_vector_type(4)));
 typedef const half8 __attribute__((address_space(3))) *lds_half8_ptr;
 
 constexpr int GW = HLQ_GEMM_WAVES;             // waves per workgroup = K parts
 constexpr int WS_COUNTER_BYTES = HLQ_WS_COUNTER_BYTES;
-#ifndef HLQ_GEMM_LA
-#define HLQ_GEMM_LA 2                          // MFMA steps between an operand read and its use
-#endif
 #ifndef HLQ_GEMM_LA
 #define HLQ_GEMM_LA 2                          // MFMA steps between an operand read and its use
 #endif
@@ -178,6 +176,35 @@ __device__ __forceinline__ void split_tiles(uint32_t lo_src, uint32_t hi_src, ui
     t1 = r[1];
 }
 
+// The wave as four rows of 16 lanes.  transpose_rows: out[j] in lane row r = in[r] of lane row j, same position in
+// the row (a 4 x 4 transposition between register index and lane row in four swaps).  bcast_rows: out[j] in every
+// lane row = v of lane row j.
+__device__ __forceinline__ void transpose_rows(const uint32_t (&in)[4], uint32_t (&out)[4])
+{
+    const auto p02 = __builtin_amdgcn_permlane32_swap(in[0], in[2], false, false);     // [0] = in0.r0 in0.r1 in2.r0 in2.r1
+    const auto p13 = __builtin_amdgcn_permlane32_swap(in[1], in[3], false, false);     // [1] = the same of rows 2, 3
+    const auto lo = __builtin_amdgcn_permlane16_swap(p02[0], p13[0], false, false);
+    const auto hi = __builtin_amdgcn_permlane16_swap(p02[1], p13[1], false, false);
+    out[0] = lo[0]; out[1] = lo[1]; out[2] = hi[0]; out[3] = hi[1];
+}
+
+__device__ __forceinline__ void bcast_rows(uint32_t v, uint32_t (&out)[4])
+{
+    const auto q = __builtin_amdgcn_permlane32_swap(v, v, false, false);               // [0] = r0 r1 r0 r1, [1] = r2 r3 r2 r3
+    const auto lo = __builtin_amdgcn_permlane16_swap(q[0], q[0], false, false);
+    const auto hi = __builtin_amdgcn_permlane16_swap(q[1], q[1], false, false);
+    out[0] = lo[0]; out[1] = lo[1]; out[2] = hi[0]; out[3] = hi[1];
+}
+
+// out[j] in lane rows 0, 1 = a of lane row j, in lane rows 2, 3 = b of lane row j.
+__device__ __forceinline__ void bcast_row_pairs(uint32_t a, uint32_t b, uint32_t (&out)[4])
+{
+    const auto q = __builtin_amdgcn_permlane32_swap(a, b, false, false);               // [0] = a.r0 a.r1 b.r0 b.r1, [1] = a.r2 a.r3 b.r2 b.r3
+    const auto lo = __builtin_amdgcn_permlane16_swap(q[0], q[0], false, false);
+    const auto hi = __builtin_amdgcn_permlane16_swap(q[1], q[1], false, false);
+    out[0] = lo[0]; out[1] = lo[1]; out[2] = hi[0]; out[3] = hi[1];
+}
+
 __device__ __forceinline__ float h2f(uint32_t v, bool hi)
 {
     return (float)__builtin_bit_cast(_Float16, (uint16_t)(hi ? v >> 16 : v & 0xffffu));
@@ -233,9 +260,8 @@ struct GemmLds {
     static_assert(WAVE_BYTES % 16 == 0, "aligned regions");
 };
 
-// MR = activation rows of the launch rounded up to 16, 32 or 64.  The MFMA tile has 32 rows; with
-// MR = 16 only rows 0..15 are staged (lanes of rows 16..31 read rows 0..15 again) and only the
-// accumulator registers of those rows (0..7 of 16) are scaled, reduced and stored.  With MR = 64 every B
+// MR = activation rows of the launch rounded up to 16, 32 or 64.  With MR = 16 the MFMA tile is 16 rows x 16
+// columns x 32 k (four column tiles per wave, four result registers each); otherwise 32 x 32 x 16.  With MR = 64 every B
 // operand serves two MFMAs (rows 0..31 and 32..63) and the activations are staged half a unit at a time.
 // grid = column blocks * K slices.
 template <int BITS, bool G64, int MR>
@@ -251,6 +277,14 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
     const int cb = blockIdx.x / a.ksplit, slice = blockIdx.x - cb * a.ksplit;
     const int u_begin = slice * a.ups, u_end = min(u_begin + a.ups, a.U);
 
+    // Up to 16 rows: v_mfma_f32_16x16x32_f16 on four 16-column tiles (no idle rows in the matrix core, four result
+    // registers per tile).  The 32 k of a step must lie in one quantization group: at G = 128 lane row r takes k
+    // quarter r of the unit and step s byte s of it; at G = 64 lane row r takes 16 k of the step's group (k = 64 g +
+    // 16 r + 8 s).
+    constexpr bool T16 = MR == 16;
+    float4v acc4[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc4[j] = float4v{0.f, 0.f, 0.f, 0.f};
     float16v acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; mt++)
@@ -287,7 +321,8 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
     const uint32_t lanepart = (uint32_t)(lane % TREP) * 16u;
     unsigned char *xw = smem + L::TAB_BYTES + wave * L::WAVE_BYTES;
     float *xs = (float *)(xw + MR * ROW_BYTES);
-    const unsigned char *arow = xw + (MR == 16 ? (col & 15) : col) * ROW_BYTES + h * 64;
+    const unsigned char *arow = T16 ? xw + (lane & 15) * ROW_BYTES + (lane >> 4) * (G64 ? 32 : 64)
+                                    : xw + col * ROW_BYTES + h * 64;
 
     // One unit: stage its activations (LDS operations of one wave execute in order, so the wave reads
     // what it has just written without a barrier), refill `cur` with the unit two turns ahead, compute.
@@ -295,6 +330,87 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
         if constexpr (MT == 1) {
             stage_store<MR>(xr, xw, xs, 0, lane);
             if (u + NW < u_end) stage_load<MR>(xr, a, u + NW, 0, lane);
+        }
+        if constexpr (T16) {
+            // Lane (c, r) of tile j works on column 16 j + c of the block: the scale / zero dwords of that column in
+            // every lane row, and the plane bits of its k (rotation undone).  G = 128: plane dword r, bit i = k 32 r + i,
+            // step s = byte s.  G = 64: per group g plane dword 2 g + r / 2 (bit i = k 64 g + 32 (r / 2) + i), step s =
+            // byte 2 (r % 2) + s -- the byte's place in the dword differs between lanes, so the v_perm selector is a
+            // register.
+            constexpr int NG = G64 ? 2 : 1, NQ = G64 ? 2 : 4;          // groups per unit, steps per chain
+            uint32_t sc4[BITS][4], zz4[4], tq[BITS][NG][4];
+#pragma unroll
+            for (int b = 0; b < BITS; b++) {
+                bcast_rows(cur.sc[b], sc4[b]);
+                if constexpr (G64) {
+                    bcast_row_pairs(cur.w[b].x, cur.w[b].y, tq[b][0]);
+                    bcast_row_pairs(cur.w[b].z, cur.w[b].w, tq[b][1]);
+                } else {
+                    const uint32_t dw[4] = {cur.w[b].x, cur.w[b].y, cur.w[b].z, cur.w[b].w};
+                    transpose_rows(dw, tq[b][0]);
+                }
+#pragma unroll
+                for (int g = 0; g < NG; g++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) tq[b][g][j] = __builtin_amdgcn_alignbit(tq[b][g][j], tq[b][g][j], HLQ_ROT);
+            }
+            bcast_rows(cur.zz, zz4);
+            if (u + 2 * NW < u_end) load_unit<BITS, G64>(cur, a, cb, u + 2 * NW, lane);
+            // the A operands of the unit's four (group, step) pairs serve every plane
+            half8 aop[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) aop[q] = *(const half8 *)(arow + (G64 ? (q >> 1) * 128 + (q & 1) * 16 : q * 16));
+            const uint32_t sel0 = 0x0c0c0000u | ((4u + 2u * ((uint32_t)(lane >> 4) & 1u)) << 8);      // G = 64: byte 2 (r % 2) + s
+            constexpr int LA = HLQ_GEMM_LA, RING = LA + 1, NSTEP = 4 * BITS;
+            half8 bop[RING][4];
+            float4v tmp[4];
+            auto issue = [&](int t) __attribute__((always_inline)) {
+                const int g = t / (BITS * NQ), b = (t / NQ) % BITS, sq = t % NQ;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if constexpr (G64) bop[t % RING][j] = table_row(__builtin_amdgcn_perm(tq[b][g][j], lanepart, sel0 + ((uint32_t)sq << 8)));
+                    else bop[t % RING][j] = table_row(row_addr<TREP>(tq[b][0][j], sq, lanepart));
+                }
+            };
+#pragma unroll
+            for (int t = 0; t < LA && t < NSTEP; t++) issue(t);
+#pragma unroll
+            for (int t = 0; t < NSTEP; t++) {
+                const int g = t / (BITS * NQ), b = (t / NQ) % BITS, sq = t % NQ;
+                if (t + LA < NSTEP) issue(t + LA);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    tmp[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[G64 ? 2 * g + sq : sq], bop[t % RING][j],
+                                                                    sq == 0 ? float4v{0.f, 0.f, 0.f, 0.f} : tmp[j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (sq == NQ - 1) {
+                    const bool hi = G64 ? g == 1 : (u & 1) != 0;      // fp16 of the meta dwords this group belongs to
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const float sf = h2f(sc4[b][j], hi);
+#pragma unroll
+                        for (int i = 0; i < 4; i++) acc4[j][i] = fmaf(sf, tmp[j][i], acc4[j][i]);
+                    }
+                    if (b == BITS - 1) {
+                        // zero term of the group: z[n, g] * sum_{k in g} x[m, k]; C rows of register i: 4 * (lane / 16) + i
+                        float4 sx = *(const float4 *)(xs + (G64 ? g : 1) * MR + 4 * (lane >> 4));
+                        if (!G64) {
+                            const float4 s0 = *(const float4 *)(xs + 4 * (lane >> 4));
+                            sx.x += s0.x; sx.y += s0.y; sx.z += s0.z; sx.w += s0.w;
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const float zf = h2f(zz4[j], hi);
+                            acc4[j][0] = fmaf(zf, sx.x, acc4[j][0]);
+                            acc4[j][1] = fmaf(zf, sx.y, acc4[j][1]);
+                            acc4[j][2] = fmaf(zf, sx.z, acc4[j][2]);
+                            acc4[j][3] = fmaf(zf, sx.w, acc4[j][3]);
+                        }
+                    }
+                }
+            }
+            return;
         }
         // Lane (col, h) of tile j works on column 32j + col of the block: bring that column's
         // scale / zero dwords and its plane dwords (k half h of each 64-k pair, rotation undone:
@@ -450,19 +566,34 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
     GEMM_STAMP(13);
     // Sum of the K parts through LDS: red[wave][tile = mt*2+j][reg][lane].
     __syncthreads();
+    if constexpr (T16) {
+        static_assert(VALS == 4 * 4 * 64, "four tiles of four registers");
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++)
+        for (int j = 0; j < 4; j++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+            for (int i = 0; i < 4; i++) red[((wave * 4 + j) * 4 + i) * 64 + lane] = acc4[j][i];
+    } else {
 #pragma unroll
-            for (int i = 0; i < REGS; i++) red[((wave * MT * 2 + mt * 2 + j) * REGS + i) * 64 + lane] = acc[mt][j][i];
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int i = 0; i < REGS; i++) red[((wave * MT * 2 + mt * 2 + j) * REGS + i) * 64 + lane] = acc[mt][j][i];
+    }
     __syncthreads();
 
     constexpr int NV = VALS / THREADS;               // results per thread
     const size_t npad = (size_t)a.ncb * HLQ_CB;
     // value v = (tile, reg, lane); C layout of the 32x32 MFMA: column = lane % 32,
     // row = 8 * (reg / 4) + 4 * (lane / 32) + reg % 4.
+    // (16x16 tiles: column = lane % 16, row = 4 * (lane / 16) + reg.)
     auto decode = [&](int v, int &m, int &n) {
+        if constexpr (T16) {
+            const int ln = v & 63, reg = (v >> 6) & 3, tile = v >> 8;
+            m = 4 * (ln >> 4) + reg;
+            n = cb * HLQ_CB + tile * 16 + (ln & 15);
+            return;
+        }
         const int ln = v & 63, reg = (v >> 6) % REGS, tile = v / (64 * REGS);
         m = (tile >> 1) * 32 + 8 * (reg >> 2) + 4 * (ln >> 5) + (reg & 3);
         n = cb * HLQ_CB + (tile & 1) * 32 + (ln & 31);
