@@ -56,6 +56,14 @@ struct SparseArgs {
 __device__ __forceinline__ float hf(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
 __device__ __forceinline__ uint16_t fh(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
 
+// v where bit `pos` of `bits` is set, else +0: the sums below add every activation, masked, rather than branch on
+// the bits (the compiler turns `if (bit) sum += v` into a branch around each load).
+__device__ __forceinline__ float bit_select(float v, uint32_t bits, int pos)
+{
+    const uint32_t mask = (uint32_t)__builtin_amdgcn_sbfe((int)bits, pos, 1);      // the bit, sign-extended
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) & mask);
+}
+
 // Thread (channel, part) of a block: its G/8 bits, LSB = lowest k.
 template <int G>
 __device__ __forceinline__ uint32_t block_bits(const uint8_t *blocks, int blk, int ch, int part)
@@ -116,8 +124,7 @@ __global__ __launch_bounds__(SP_THREADS) void hlq_sparse_plane_kernel(const Spar
                     const uint16_t h[4] = {(uint16_t)(v.x & 0xffffu), (uint16_t)(v.x >> 16), (uint16_t)(v.y & 0xffffu),
                                            (uint16_t)(v.y >> 16)};
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        if (bits[i] >> (4 * q + j) & 1u) sum += hf(h[j]);
+                    for (int j = 0; j < 4; j++) sum += bit_select(hf(h[j]), bits[i], 4 * q + j);
                 }
                 // the 8 parts of a channel sit in 8 consecutive lanes
                 sum += __shfl_xor(sum, 1);
@@ -134,20 +141,14 @@ __global__ __launch_bounds__(SP_THREADS) void hlq_sparse_plane_kernel(const Spar
     }
 }
 
-// Batch 1: one workgroup of sixteen waves per channel tile; wave w takes the tile's blocks w, w + 16, ... and works
-// on a block alone (a tile's blocks cost a chain of dependent memory round trips -- block range, k starts,
-// activations -- whatever their number, so as many as possible go through it side by side).  The G activations of a block are the same for its 32 channels, so the wave forms them once
-// (two per lane, through the prologue if there is one), parks them in LDS as fp32 and every lane (channel, half of
-// the block's k) adds up the ones its bits select: LDS reads of one address per half, no bank conflicts.  NB
-// blocks of a wave are in flight at a time (their k starts, bits, scales and activations depend on each other only
-// through addresses).  The waves' sums meet in LDS in wave order: the result does not depend on timing.
-// v where bit `pos` of `bits` is set, else +0.
-__device__ __forceinline__ float bit_select(float v, uint32_t bits, int pos)
-{
-    const uint32_t mask = (uint32_t)__builtin_amdgcn_sbfe((int)bits, pos, 1);      // the bit, sign-extended
-    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) & mask);
-}
-
+// Batch 1: one workgroup of up to sixteen waves per channel tile; wave w takes the tile's blocks w, w + 16, ... and
+// works on a block alone (a tile's blocks cost a chain of dependent memory round trips -- block range, k starts,
+// activations -- whatever their number, so as many as possible go through it side by side).  The G activations of a
+// block are the same for its 32 channels, so the wave forms them once (two per lane, through the prologue if there
+// is one), parks them in LDS as fp32 and every lane (channel, half of the block's k) adds up the ones its bits
+// select: LDS reads of one address per half, no bank conflicts.  NB blocks of a wave are in flight at a time (their
+// k starts, bits, scales and activations depend on each other only through addresses).  The waves' sums meet in LDS
+// in wave order: the result does not depend on timing.
 constexpr int SPV_WAVES = 16;                    // at most; the launch decides (blockDim.x / 64)
 
 template <int G, bool PRO, int NB>
