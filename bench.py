@@ -50,7 +50,7 @@ def parse():
     p.add_argument("--sweep-only", action="store_true",
                    help="only the sweep and the per-shape rings of the per-GEMV entry point (no grouped / multi-stream / "
                         "copy / other-format / large-shape legs): the run a kernel trace of the dominant kernel is taken from")
-    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "decode-eager", "gemm", "group", "sparse", "shape-sweep"],
+    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "decode-eager", "gemm", "group", "sparse", "shape-sweep", "lds-rate"],
                    default="full",
                    help="kernel: only the dominant GEMV (4096x14336) over its weight ring, for counter runs; "
                         "copy: a plain 64 MiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE; "
@@ -188,6 +188,35 @@ def gemm_leg(torch, lib, dev, steps):
         del mods
         torch.cuda.empty_cache()
     return out
+
+
+def lds_rate_leg(torch, lib, dev, passes=4000):
+    """Rate at which one compute unit retires wavefront-wide 16-entry table lookups: bare ds_read_b32 instructions, and
+    the LUT GEMV's own sub-task sequence on plane words held in registers (tables already in LDS, nothing loaded from
+    memory).  A lookup covers 4 k of one column and one plane, i.e. 4 weight bits per lane; the rates are restated as
+    the HBM stream a w2g128 GEMV would sustain at them (planes are 2048 of the 2432 bytes of a unit)."""
+    out = torch.zeros(256 * 2048, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {}
+    for sequence, name in ((0, "bare_ds_read_b32"), (1, "gemv_subtask_sequence")):
+        res[name] = {}
+        for waves in (4, 8, 16, 32):
+            best = None
+            for _ in range(4):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                rc = lib.elutq_diag_lds_lookup_rate(sequence, waves, passes, out.data_ptr(), stream)
+                e1.record()
+                if rc:
+                    raise RuntimeError(f"elutq_diag_lds_lookup_rate failed: {rc}")
+                torch.cuda.synchronize()
+                ms = e0.elapsed_time(e1)
+                best = ms if best is None else min(best, ms)
+            ns = best * 1e6 / (passes * 16 * waves)
+            plane_tbps = 256 * 64 * 4 / 8 / ns / 1e3
+            res[name][f"{waves}_waves_per_cu"] = {"ns_per_wave_lookup_per_cu": ns, "cycles_at_2p4_GHz": ns * 2.4,
+                                                  "w2g128_algorithmic_TBps_at_that_rate": plane_tbps * 2432 / 2048}
+    return res
 
 
 def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
@@ -488,6 +517,9 @@ def main():
         print(json.dumps({"mode": "group", "gemvs_per_launch": len(mods), "bytes_per_launch": nbytes, "us_per_launch": sec * 1e6,
                           "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}))
         grp.close()
+        return
+    if a.mode == "lds-rate":
+        print(json.dumps({"mode": "lds-rate", "lds_lookup_rate": lds_rate_leg(torch, lib, dev)}))
         return
     if a.mode == "sparse":
         print(json.dumps({"mode": "sparse", "sparse_gemv_w2g128": sparse_leg(torch, lib, dev, a.steps, a.warmup)}))
