@@ -109,7 +109,13 @@ __global__ __launch_bounds__(ATTN_WAVES * 64) void rope_attn_kernel(const AttnAr
     const int j = lane < half ? lane : 0;
     const bool active = lane < half;
     const int pos = (int)*a.pos;
-    if (pos < 0 || pos >= a.max_seq) return;      // outside the cache: nothing is read or written
+    if (pos < 0 || pos >= a.max_seq) {            // outside the cache: nothing is read, the output says so (NaN)
+        if (wave == 0 && active) {
+            a.out[(size_t)h * d + j] = 0x7e00u;
+            a.out[(size_t)h * d + j + half] = 0x7e00u;
+        }
+        return;
+    }
 
     const float inv_freq = exp2f(-(float)(2 * j) / (float)d * a.log2_base);
     float sn, cs;
@@ -265,7 +271,10 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     const uint16_t qa16 = el[0], qb16 = el[1], ka16 = el[2], kb16 = el[3], va16 = el[4], vb16 = el[5];
     asm volatile("" ::: "memory");
     const int pos = (int)pos64;
-    if (pos64 < 0 || pos64 >= a.max_seq) return;
+    if (pos64 < 0 || pos64 >= a.max_seq) {          // outside the cache: nothing is read, the output says so (NaN)
+        if (sp == 0 && tid < D) a.out[(size_t)h * D + tid] = 0x7e00u;
+        return;
+    }
     // How many of the launched workgroups take part follows the context: meeting in device memory
     // costs about 2 us plus 0.1-0.2 us per partial result, a further 64-row block about 0.6 us.  So a
     // context of at most SHORT_BLOCKS blocks is one workgroup's work, up to 12 blocks are shared by

@@ -478,7 +478,7 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
     ((generate_num - 1) / elapsed, main.cpp:110).  `hlq_lm_head`: see random_parts."""
     s = shape or LlamaShape()
     if n_ctx + n_gen > s.max_seq:
-        # the attention launch of a position beyond the cache returns at once: such tokens must not be timed
+        # the attention launch of a position beyond the cache returns at once (NaN output): such tokens must not be timed
         raise ValueError(f"n_ctx + n_gen = {n_ctx + n_gen} exceeds the cache of {s.max_seq} positions")
     dev = torch.device(device)
     model = LlamaDecoder(s, device=dev, seed=0, impl=impl, parts=random_parts(s, dev, 0, hlq_lm_head))

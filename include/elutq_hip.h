@@ -290,7 +290,8 @@ int elutq_hlq_gemm_f16_tuned(const void *d_planes, const void *d_scales, const v
  * (C++/ops/src/arm/arm_rotary.cpp:4-89, arm_cache.cpp:17-22, arm_attention.cpp:162-316).
  * d_qkv fp16 [n_heads*d | n_kv_heads*d | n_kv_heads*d]; caches fp16 [max_seq][n_kv_heads][d];
  * d_pos a DEVICE int64 (so a captured graph can advance it); head_dim even, <= 128.
- * If *d_pos is outside [0, max_seq) the kernel does nothing.
+ * If *d_pos is outside [0, max_seq) the kernel reads and caches nothing and fills d_out with fp16 NaN, so that
+ * a step beyond the cache shows in the logits instead of passing with the previous step's attention output.
  */
 int elutq_decode_rope_attn_f16(const void *d_qkv, void *d_k_cache, void *d_v_cache, const void *d_pos,
                                void *d_out, int n_heads, int n_kv_heads, int head_dim, int max_seq,

@@ -178,12 +178,22 @@ def test_rope_attn_rejects_bad_arguments(cuda):
     assert L.elutq_decode_rope_attn_f16(*args(8, 3, 64)) == -2       # heads not a multiple of kv heads
     assert L.elutq_decode_rope_attn_f16(*args(8, 2, 256)) == -2      # head_dim > 128
     assert L.elutq_decode_rope_attn_f16(None, t.data_ptr(), t.data_ptr(), p.data_ptr(), t.data_ptr(), 8, 2, 64, 8, 1e4, s) == -1
-    # a position outside the cache leaves the output untouched
-    out = torch.full((1, 256), 7.0, dtype=torch.float16, device=cuda)
-    p.fill_(8)
-    assert L.elutq_decode_rope_attn_f16(t.data_ptr(), t.data_ptr(), t.data_ptr(), p.data_ptr(), out.data_ptr(), 4, 1, 64, 8, 1e4, s) == 0
-    torch.cuda.synchronize()
-    assert bool((out == 7).all())
+    # a position outside the cache: the caches stay as they are and the output is NaN throughout, so that a step
+    # beyond the cache shows in the logits (general kernel, and the head_dim 128 kernel with and without splits)
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device=cuda)
+    for d, pos in ((64, 8), (128, 8), (128, -1)):
+        out = torch.full((1, 4 * d), 7.0, dtype=torch.float16, device=cuda)
+        kc = torch.full((8, 1, d), 3.0, dtype=torch.float16, device=cuda)
+        vc = kc.clone()
+        p.fill_(pos)
+        assert L.elutq_decode_rope_attn_f16(t.data_ptr(), kc.data_ptr(), vc.data_ptr(), p.data_ptr(), out.data_ptr(), 4, 1, d, 8, 1e4, s) == 0
+        torch.cuda.synchronize()
+        assert bool(out.isnan().all()) and bool((kc == 3).all()) and bool((vc == 3).all())
+        out.fill_(7.0)
+        assert L.elutq_decode_rope_attn_split_f16(t.data_ptr(), kc.data_ptr(), vc.data_ptr(), p.data_ptr(), out.data_ptr(), 4, 1, d, 8,
+                                                  1e4, 0, ws.data_ptr(), ws.numel(), s) == 0
+        torch.cuda.synchronize()
+        assert bool(out.isnan().all()) and bool((kc == 3).all()) and int(ws.count_nonzero()) == 0
 
 
 @pytest.mark.parametrize("split", [False, True])
