@@ -40,6 +40,7 @@ def run(mod, x, dev):
 @pytest.mark.parametrize("k,n,bits,group,density", [
     (256, 64, 2, 128, 0.5), (512, 128, 2, 128, 0.3), (1024, 256, 3, 64, 0.2), (1024, 192, 1, 64, 1.0),
     (2048, 512, 2, 128, 0.05), (384, 96, 4, 128, 0.5), (704, 128, 2, 64, 0.3),
+    (4096, 64, 2, 64, 1.0), (8192, 32, 2, 128, 0.9),          # 64 / ~58 blocks on a tile: more than one round of the plane kernel's waves
 ])
 def test_gemv_matches_oracle(cuda, lutref, k, n, bits, group, density):
     L, sp, mod = build(k, n, bits, group, density, k + n, cuda)
@@ -218,7 +219,7 @@ def _fused_case(k, n, bits, group, density, seed, dev):
     return L, sp, mod, g, res, out, ws
 
 
-FUSED_SHAPES = [(1024, 256, 2, 128, 0.3), (512, 96, 3, 64, 0.5), (4096, 1024, 2, 128, 0.1), (1088, 160, 2, 64, 0.4),
+FUSED_SHAPES = [(4096, 64, 2, 64, 1.0), (1024, 256, 2, 128, 0.3), (512, 96, 3, 64, 0.5), (4096, 1024, 2, 128, 0.1), (1088, 160, 2, 64, 0.4),
                 (4096, 4096, 2, 128, 0.05)]
 
 
