@@ -306,11 +306,6 @@ __global__ __launch_bounds__(1024) void hlq_gemv_run_kernel(const GemvArgs a, in
 // the first memory round trips and the tail of a GEMV are paid once per list instead of once
 // per GEMV, and with two workgroups per CU the sum-and-store of one tile hides under the
 // lookups of another.
-struct GroupItem {
-    int problem, cb, slice;  // first column block and K slice
-    int ncb_run;             // consecutive column blocks of that slice
-};
-
 template <int BITS, bool G64, int NSLOT, bool PAIRED>
 __global__ __launch_bounds__(1024) void hlq_gemv_group_kernel(const GemvArgs *__restrict__ problems,
                                                               const GroupItem *__restrict__ items, int n_items)
@@ -672,12 +667,22 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
     const HlqGeo g = hlq_geo(K, N, bits, group);
     LaunchShape sh;
     const bool allow_narrow = !(fusion && fusion->d_slices_out) && !lut_int8;
+    const bool own_shape = ksplit == 0 && waves == 0;              // the library chooses the launch shape
     rc = plan_launch(g, bits, ksplit, waves, allow_narrow, sh, lut_int8);
     if (rc != ELUTQ_OK) return rc;
     if (lut_int8 && (sh.mfma || sh.narrow || fusion || d_extra)) return ELUTQ_ERR_TUNING;
     ksplit = sh.ksplit; waves = sh.waves;
     const int ups = sh.ups;
 
+    // A plain call on a layer with more column blocks than the chip has compute units and K > 4096: the streaming
+    // matrix-core kernel, every workgroup an equal share of the column blocks over all of K (no slices, no workspace).
+    // Measured on MI355X against the LUT kernel's runs of column blocks with K slices: 8192 x 28672 17.7 against
+    // 21.2 us, 14336 x 32768 29.2 against 51.8 us; at K = 4096, where the LUT kernel needs no slices, the two are level
+    // (4096 x 128256: 31.0 against 30.6 us) and the LUT kernel stays.
+    const bool wide = g_gemv_engine != ELUTQ_GEMV_ENGINE_LUT && !lut_int8 && !fusion && !d_extra && own_shape &&
+                      g.K % HLQ_UNIT == 0 && g.ncb > NUM_CU && (g.U > 32 || g_gemv_engine == ELUTQ_GEMV_ENGINE_MFMA);
+    if (wide) sh.ksplit = 1;
+    ksplit = sh.ksplit;
     GemvArgs a;
     a.planes = (const HLQ_GLOBAL uint4 *)d_planes;
     a.scales = (const HLQ_GLOBAL uint32_t *)d_scales;
@@ -737,6 +742,7 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
             a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
         }
     }
+    if (wide) return hlq_gemv_mfma_wide_launch(&a, sizeof(a), bits, group, stream);
     if (sh.narrow) return hlq_gemv_narrow_launch(&a, sizeof(a), bits, group, sh.narrow, stage_bytes, stream);
     if (sh.mfma) return hlq_gemv_mfma_launch(&a, sizeof(a), bits, group, waves, stage_bytes, stream);
     return dispatch_gemv(a, bits, group, waves, gemv_lds_bytes(ups, bits, waves) + stage_bytes, (hipStream_t)stream);
@@ -802,12 +808,19 @@ struct GroupShape {                      // tile shape of one problem inside a g
     WavePlan wp;
 };
 
-static int group_shape(const elutq_gemv_problem &p, int bits, int group, GroupShape &sh)
+static int group_shape(const elutq_gemv_problem &p, int bits, int group, bool mfma, GroupShape &sh)
 {
     int rc = check_shape(p.K, p.N, bits, group);
     if (rc != ELUTQ_OK) return rc;
     if (!p.d_planes || !p.d_scales || !p.d_zeros || !p.d_x || !p.d_y) return ELUTQ_ERR_NULL;
     sh.g = hlq_geo(p.K, p.N, bits, group);
+    if (mfma) {
+        // a tile of the matrix-core kernel covers all of K: no slices, nothing to meet in the workspace
+        sh.ups = sh.g.U;
+        sh.ksplit = 1;
+        sh.wp = wave_plan(1, bits, 16);              // (the wave-run fields are not read by the matrix-core kernel)
+        return ELUTQ_OK;
+    }
     // the list supplies the parallelism: slice K only as far as LDS and the run length ask for
     // (a wave's run must fit its slots: at most 16 * depth_of(bits) sub-tasks per slice)
     const int DEPTH = depth_of(bits);
@@ -824,11 +837,20 @@ static int group_shape(const elutq_gemv_problem &p, int bits, int group, GroupSh
 
 struct GemvGroupPlan {
     int bits, group, nslot, n_items, grid;
-    bool paired;
+    bool paired, mfma;
     size_t lds;
     GemvArgs *d_problems;
-    GroupItem *d_items;
+    void *d_items;           // GroupItem array, or the tile blob of the matrix-core kernel
 };
+
+// The grouped launch runs on the matrix cores where that engine is selected and every layer has whole units.
+static bool group_on_mfma(const elutq_gemv_problem *problems, int count)
+{
+    if (g_gemv_engine == ELUTQ_GEMV_ENGINE_LUT) return false;          // (the library's own choice: measured 6.3 against 5.6 TB/s)
+    for (int i = 0; i < count; i++)
+        if (problems[i].K % HLQ_UNIT != 0) return false;
+    return true;
+}
 
 static size_t group_layout(const elutq_gemv_problem *problems, int count, int bits, int group,
                            std::vector<GroupShape> *shapes, std::vector<size_t> *counter_off, std::vector<size_t> *partial_off,
@@ -836,9 +858,10 @@ static size_t group_layout(const elutq_gemv_problem *problems, int count, int bi
 {
     size_t counters = 0, partials = 0;
     *rc_out = ELUTQ_OK;
+    const bool mfma = group_on_mfma(problems, count);
     for (int i = 0; i < count; i++) {
         GroupShape sh;
-        const int rc = group_shape(problems[i], bits, group, sh);
+        const int rc = group_shape(problems[i], bits, group, mfma, sh);
         if (rc != ELUTQ_OK) { *rc_out = rc; return 0; }
         if (shapes) shapes->push_back(sh);
         if (counter_off) counter_off->push_back(counters);
@@ -889,6 +912,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
     if (cbs_per_item < 1) cbs_per_item = 1;
     int nslot = 1;
     size_t lds = 0;
+    const bool mfma = group_on_mfma(problems, count);
     for (int i = 0; i < count; i++) {
         const GroupShape &sh = shapes[i];
         GemvArgs &a = args[i];
@@ -913,6 +937,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
         a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr; a.lut_int8 = 0;
         const int ns = a.spw < depth_of(bits) ? a.spw : depth_of(bits);
         if (ns > nslot) nslot = ns;
+        if (mfma) continue;                          // its tile list is made below, over all layers at once
         const size_t l = gemv_lds_bytes(sh.ups, bits, 16);
         if (l > lds) lds = l;
         // runs of column blocks share one table build
@@ -925,18 +950,33 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
     GemvGroupPlan *pl = new GemvGroupPlan();
     pl->bits = bits; pl->group = group; pl->nslot = nslot; pl->n_items = (int)items.size(); pl->lds = lds;
     pl->paired = true;
+    pl->mfma = mfma;
     for (auto &sh : shapes) pl->paired = pl->paired && paired_ok_rt(bits, group == 64, nslot, sh.wp.spw, sh.ups, sh.ksplit);
-    // as many workgroups as the chip holds at once: each walks the list with that stride
-    int per_cu = dispatch_group(bits, group == 64, nslot, pl->paired, nullptr, nullptr, 0, -1, 16, lds, nullptr);
-    if (per_cu < 1) per_cu = 1;
-    if (per_cu > 2) per_cu = 2;
-    const int slots = NUM_CU * per_cu;
-    pl->grid = pl->n_items < slots ? pl->n_items : slots;
+    std::vector<unsigned char> blob;
+    const void *h_items = items.data();
+    size_t items_bytes = items.size() * sizeof(GroupItem);
+    if (mfma) {
+        // one workgroup per compute unit, each with its own contiguous share of the layers' column blocks
+        std::vector<int> units(count), ncbs(count);
+        for (int i = 0; i < count; i++) { units[i] = shapes[i].g.U; ncbs[i] = shapes[i].g.ncb; }
+        pl->grid = total_cbs < NUM_CU ? (int)total_cbs : NUM_CU;
+        blob.resize(hlq_gemv_mfma_group_plan(units.data(), ncbs.data(), count, pl->grid, nullptr));
+        hlq_gemv_mfma_group_plan(units.data(), ncbs.data(), count, pl->grid, blob.data());
+        h_items = blob.data();
+        items_bytes = blob.size();
+    } else {
+        // as many workgroups as the chip holds at once: each walks the list with that stride
+        int per_cu = dispatch_group(bits, group == 64, nslot, pl->paired, nullptr, nullptr, 0, -1, 16, lds, nullptr);
+        if (per_cu < 1) per_cu = 1;
+        if (per_cu > 2) per_cu = 2;
+        const int slots = NUM_CU * per_cu;
+        pl->grid = pl->n_items < slots ? pl->n_items : slots;
+    }
     pl->d_problems = nullptr; pl->d_items = nullptr;
     if (hipMalloc((void **)&pl->d_problems, args.size() * sizeof(GemvArgs)) != hipSuccess ||
-        hipMalloc((void **)&pl->d_items, items.size() * sizeof(GroupItem)) != hipSuccess ||
+        hipMalloc((void **)&pl->d_items, items_bytes) != hipSuccess ||
         hipMemcpy(pl->d_problems, args.data(), args.size() * sizeof(GemvArgs), hipMemcpyHostToDevice) != hipSuccess ||
-        hipMemcpy(pl->d_items, items.data(), items.size() * sizeof(GroupItem), hipMemcpyHostToDevice) != hipSuccess) {
+        hipMemcpy(pl->d_items, h_items, items_bytes, hipMemcpyHostToDevice) != hipSuccess) {
         if (pl->d_problems) (void)hipFree(pl->d_problems);
         if (pl->d_items) (void)hipFree(pl->d_items);
         delete pl;
@@ -950,7 +990,8 @@ int elutq_hlq_gemv_group_run(void *plan, void *stream)
 {
     if (!plan) return ELUTQ_ERR_NULL;
     const GemvGroupPlan *pl = (const GemvGroupPlan *)plan;
-    return dispatch_group(pl->bits, pl->group == 64, pl->nslot, pl->paired, pl->d_problems, pl->d_items, pl->n_items, pl->grid, 16,
+    if (pl->mfma) return hlq_gemv_mfma_group_launch(pl->bits, pl->group, pl->d_problems, pl->d_items, pl->grid, stream);
+    return dispatch_group(pl->bits, pl->group == 64, pl->nslot, pl->paired, pl->d_problems, (const GroupItem *)pl->d_items, pl->n_items, pl->grid, 16,
                           pl->lds, (hipStream_t)stream);
 }
 

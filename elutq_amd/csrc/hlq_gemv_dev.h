@@ -75,6 +75,13 @@ __device__ unsigned long long *g_hlq_stamps = nullptr;
 #define HLQ_STAMP_FLUSH do { } while (0)
 #endif
 
+// One tile of a grouped launch (many independent GEMVs in one launch): a run of consecutive column blocks of one
+// K slice of one problem of the list.
+struct GroupItem {
+    int problem, cb, slice;  // first column block and K slice
+    int ncb_run;             // consecutive column blocks of that slice
+};
+
 typedef __attribute__((address_space(3))) const int lds_cint;
 
 __device__ __forceinline__ int lds_ld(uint32_t addr, int imm)

@@ -136,3 +136,88 @@ HLQ_HD int hlq_narrow_half_index(int ci) { return ci >> 4; }
 HLQ_HD int hlq_narrow_x_chunk(int ub, int ci, int K) { const int c = ub * 32 + ci; return c < K / 4 - 1 ? c : K / 4 - 1; }
 // Unit whose weights a lane loads in round r (clamped to the last unit; past it the lane's sum is masked).
 HLQ_HD int hlq_narrow_unit(int ub, int r, int ul_count, int ul, int U) { const int u = ub + r * ul_count + ul; return u < U - 1 ? u : U - 1; }
+
+// ---- grouped launch of the matrix-core GEMV (hlq_gemv_mfma.hip) ---------------------------------------------------
+// A tile is up to HLQ_MFMA_ITEM_CBS consecutive column blocks of one layer over all of K.  Its work units (unit pair,
+// column block), pair-major, are dealt to the sixteen waves of the workgroup in equal contiguous shares.
+#define HLQ_MFMA_ITEM_CBS 8
+
+struct HlqMfmaItem {
+    int problem, cb0;      // layer and first column block
+    int ncb, magic;        // column blocks (1..HLQ_MFMA_ITEM_CBS), ceil(2^20 / ncb)
+};
+
+// What one wave does of a tile.
+struct HlqMfmaShare {
+    int npairs, u_last;    // unit pairs and last unit of the layer
+    int cb0, ncb, magic;
+    int m_lo, nt, nt_pad;  // first work unit of the wave's share, positions (unit, plane) in it, the same rounded up to `unroll`
+};
+
+HLQ_HD HlqMfmaShare hlq_mfma_share(int U, const HlqMfmaItem &it, int wave, int bits, int unroll)
+{
+    HlqMfmaShare v;
+    v.npairs = (U + 1) >> 1;
+    v.u_last = U - 1;
+    v.cb0 = it.cb0; v.ncb = it.ncb; v.magic = it.magic;
+    const int n_units = v.npairs * it.ncb;
+    v.m_lo = wave * n_units / 16;
+    v.nt = ((wave + 1) * n_units / 16 - v.m_lo) * bits;
+    v.nt_pad = (v.nt + unroll - 1) / unroll * unroll;
+    return v;
+}
+
+// work unit m of a tile -> unit pair and column block inside the tile (exact for m < 2^17, ncb <= 8)
+HLQ_HD void hlq_mfma_unit_of(const HlqMfmaShare &v, int m, int &p, int &c)
+{
+    p = (int)(((unsigned)m * (unsigned)v.magic) >> 20);
+    c = m - p * v.ncb;
+}
+
+// The unit pair and column block whose plane data a wave loads for position `pos` of its share (positions past the
+// share re-read its last one; a wave without a share reads a valid block of the tile).
+HLQ_HD void hlq_mfma_load_target(const HlqMfmaShare &v, int pos, int bits, int &p, int &c)
+{
+    const int last = v.nt - 1 > 0 ? v.nt - 1 : 0;
+    hlq_mfma_unit_of(v, v.m_lo + (pos < last ? pos : last) / bits, p, c);
+    if (p > v.npairs - 1) p = v.npairs - 1;
+    if (c > v.ncb - 1) c = v.ncb - 1;
+}
+
+// The tile list: the column blocks of all layers, in order, are cut into `grid` contiguous shares of equal weight (a
+// column block weighs its layer's unit count, i.e. its bytes), one per workgroup, and every share into tiles of at most
+// HLQ_MFMA_ITEM_CBS column blocks of one layer.  Blob layout: int wg_begin[grid + 1] (padded to 16 bytes), then the
+// tiles.  h_blob null: only the size is returned.
+static inline size_t hlq_mfma_group_plan(const int *units, const int *ncbs, int count, int grid, void *h_blob)
+{
+    long long total = 0;
+    for (int i = 0; i < count; i++) total += (long long)units[i] * ncbs[i];
+    const size_t head = ((size_t)(grid + 1) * sizeof(int) + 15) & ~(size_t)15;
+    int *wg_begin = (int *)h_blob;
+    HlqMfmaItem *items = h_blob ? (HlqMfmaItem *)((unsigned char *)h_blob + head) : nullptr;
+    size_t n_items = 0;
+    int layer = 0, cb = 0;
+    long long done = 0;
+    for (int g = 0; g < grid; g++) {
+        if (wg_begin) wg_begin[g] = (int)n_items;
+        const long long goal = total * (g + 1) / grid;       // cumulative weight at the end of this share
+        while (layer < count) {
+            if (cb >= ncbs[layer]) { layer++; cb = 0; continue; }
+            // column blocks of this layer that still belong to the share (at least half of a block's weight inside it)
+            long long room = (goal - done + units[layer] / 2) / units[layer];
+            if (g == grid - 1) room = ncbs[layer] - cb;
+            if (room <= 0) break;
+            int take = (int)(room < ncbs[layer] - cb ? room : ncbs[layer] - cb);
+            done += (long long)take * units[layer];
+            while (take > 0) {
+                const int len = take < HLQ_MFMA_ITEM_CBS ? take : HLQ_MFMA_ITEM_CBS;
+                if (items) items[n_items] = HlqMfmaItem{layer, cb, len, (int)(((1u << 20) + len - 1) / len)};
+                n_items++;
+                cb += len;
+                take -= len;
+            }
+        }
+    }
+    if (wg_begin) wg_begin[grid] = (int)n_items;
+    return head + n_items * sizeof(HlqMfmaItem);
+}

@@ -29,6 +29,19 @@ HLQ_INTERNAL int hlq_gemm_chunk_with_extra(const void *d_planes, const void *d_s
 HLQ_INTERNAL int hlq_gemv_mfma_launch(const void *gemv_args, size_t args_bytes, int bits, int group, int waves,
                                       size_t stage_bytes, void *stream);
 HLQ_INTERNAL size_t hlq_gemv_mfma_lds_bytes(int ups, int waves);
+// Grouped launch of the matrix-core kernel.  hlq_gemv_mfma_group_plan cuts the column blocks of `count` layers
+// (units[i] = K / 128, ncbs[i] = ceil(N / 64)) into `grid` contiguous shares of equal bytes and writes the tile list
+// into h_blob (null: only the size is returned); the launch takes that blob on the device and a device array of the
+// launcher's argument blocks (pointers, N, U, K, NT, ncb are read).  A tile covers all of K, so no workspace is used.
+HLQ_INTERNAL size_t hlq_gemv_mfma_group_plan(const int *units, const int *ncbs, int count, int grid, void *h_blob);
+HLQ_INTERNAL size_t hlq_gemv_mfma_group_lds_bytes(void);
+HLQ_INTERNAL int hlq_gemv_mfma_group_launch(int bits, int group, const void *d_problems, const void *d_blob, int grid,
+                                            void *stream);
+
+// The same streaming kernel for one plain GEMV of a layer with many column blocks (no prologue, residual, extra term,
+// handed-over slices; K a multiple of 128): every workgroup takes an equal share of the column blocks over all of K,
+// so the launch uses no workspace.
+HLQ_INTERNAL int hlq_gemv_mfma_wide_launch(const void *gemv_args, size_t args_bytes, int bits, int group, void *stream);
 
 // The narrow-tile LUT GEMV kernel (hlq_gemv_narrow.hip): a workgroup owns `cw` = 16 or 32 columns over all of K,
 // no K slices.  hlq_gemv_narrow_rounds: units per unit lane of a wave for a layer of U = K / 128 units, 0 where the

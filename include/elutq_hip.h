@@ -88,9 +88,13 @@ int elutq_hlq_unpack_host(const void *h_planes, const void *h_scales, const void
  * Which kernel the batch-1 GEMV entry points launch (process-wide; for tests, benchmarks and debugging):
  *   ELUTQ_GEMV_ENGINE_LUT   activation tables in LDS, 4-bit lookups (the T-MAC scheme of the reference's
  *                           t_mac_g4_float_update_impl, C++/ops/src/arm/arm_t_mac_kernal.cpp:364-469)
- *   ELUTQ_GEMV_ENGINE_MFMA  the plane bits go to the matrix cores as fp4 operands against fixed-point
- *                           digits of the activations; no lookups
- *   ELUTQ_GEMV_ENGINE_AUTO  the library's choice per shape (the default)
+ *   ELUTQ_GEMV_ENGINE_MFMA  the plane bits go to the matrix cores as fp4 operands against balanced base-7 digits
+ *                           of the activations (fp4 x fp4 MFMA); no lookups
+ *   ELUTQ_GEMV_ENGINE_AUTO  the library's choice per launch (the default): the LUT kernels for a single GEMV of up to
+ *                           256 column blocks of 64 (its launch is latency bound and the tables are built sooner than
+ *                           the digits); the matrix-core kernel where a launch streams many column blocks per
+ *                           workgroup -- grouped launches, and plain calls on layers with more than 256 column blocks
+ *                           and K > 4096
  * Both compute the same sums (fp32 fold per group and plane); results agree to the final fp16 rounding and
  * are bit-identical where the arithmetic is exact.  Returns ELUTQ_ERR_TUNING for another value.
  */
@@ -243,8 +247,13 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
  * A plan holds the device-side problem list: create it once (allocates and copies; not
  * capturable), run it any number of times (one kernel launch, capturable), destroy it.
  * The workspace (elutq_hlq_gemv_group_workspace_bytes, zero-filled once) is bound at creation
- * and must not be shared with calls that may run concurrently.  Results equal those of
- * elutq_hlq_gemv_f16_tuned with the same K slicing, which the group chooses itself.
+ * and must not be shared with calls that may run concurrently.  On the LUT engine the results equal those of
+ * elutq_hlq_gemv_f16_tuned with the same K slicing, which the group chooses itself.  On the matrix-core engine
+ * (the default for a group whose layers all have K % 128 == 0) every workgroup streams one contiguous share of
+ * all the layers' bytes and a tile covers all of K, so nothing meets in device memory and the workspace is not
+ * used; a layer's sums are the same numbers added in an order that depends on where its tiles fall in the plan:
+ * bit-identical from run to run of a plan, within the final fp16 rounding of any other launch of the layer,
+ * exact where the arithmetic is exact.
  */
 typedef struct elutq_gemv_problem {
     const void *d_planes, *d_scales, *d_zeros, *d_bias;  /* as for elutq_hlq_gemv_f16; bias may be NULL */

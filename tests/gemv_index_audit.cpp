@@ -14,6 +14,7 @@
 #include <cstring>
 #include <map>
 #include <string>
+#include <vector>
 
 #include "hlq_gemv_index.h"
 
@@ -163,6 +164,85 @@ void audit_narrow(int bits, bool g64, int cw, int rounds, int U, int ncb, bool r
 #undef CHECK
 }
 
+// The grouped launch of the matrix-core kernel (hlq_gemv_mfma.hip: hlq_gemv_mfma_group_kernel): the plan's shares and
+// tiles must cover every column block of every layer exactly once, every work unit (unit pair, column block) of a tile
+// must fall to exactly one wave, and every plane / scale / zero / activation load -- the positions past a wave's share
+// and the ring refills that reach into the next tile included -- must stay inside the layer's buffers.
+void audit_mfma_group(const std::vector<int> &units, const std::vector<int> &ncbs, int grid, int bits, bool g64)
+{
+    const int count = (int)units.size();
+    std::vector<unsigned char> blob(hlq_mfma_group_plan(units.data(), ncbs.data(), count, grid, nullptr));
+    hlq_mfma_group_plan(units.data(), ncbs.data(), count, grid, blob.data());
+    const int *wg_begin = (const int *)blob.data();
+    const HlqMfmaItem *items = (const HlqMfmaItem *)(blob.data() + (((size_t)(grid + 1) * sizeof(int) + 15) & ~(size_t)15));
+    const int slice = 0, n_slices_in = 0, multi = 2, waves = 16;
+    const int unroll = bits % 2 ? 2 * bits : bits;
+    std::vector<std::vector<int>> seen(count);
+    for (int i = 0; i < count; i++) seen[i].assign(ncbs[i], 0);
+    long long total = 0, heaviest = 0;
+    for (int i = 0; i < count; i++) total += (long long)units[i] * ncbs[i];
+    int wave = 0, U = 0, ups = 0;
+#define CHECK(ok, what) check((ok), what, bits, g64, waves, U, ups, slice, wave, n_slices_in, multi)
+    CHECK(wg_begin[0] == 0, "g-plan");
+    for (int g = 0; g < grid; g++) {
+        long long weight = 0;
+        CHECK(wg_begin[g] <= wg_begin[g + 1], "g-plan");
+        for (int i = wg_begin[g]; i < wg_begin[g + 1]; i++) {
+            const HlqMfmaItem &it = items[i];
+            CHECK(it.problem >= 0 && it.problem < count && it.ncb >= 1 && it.ncb <= HLQ_MFMA_ITEM_CBS && it.cb0 >= 0 &&
+                  it.cb0 + it.ncb <= ncbs[it.problem] && it.magic == (int)(((1u << 20) + it.ncb - 1) / it.ncb), "g-item");
+            U = units[it.problem]; ups = it.ncb;
+            for (int c = 0; c < it.ncb; c++) seen[it.problem][it.cb0 + c]++;
+            weight += (long long)U * it.ncb;
+            const int npairs = (U + 1) / 2;
+            std::vector<int> unit_seen(npairs * it.ncb, 0);
+            const int K = U * UNIT, NT = ((g64 ? K / 64 : U) + 1) / 2, ncb_layer = ncbs[it.problem];
+            const size_t planes_bytes = (size_t)ncb_layer * U * bits * CB * 16;
+            const size_t scale_bytes = (size_t)ncb_layer * NT * bits * CB * 4, zero_bytes = (size_t)ncb_layer * NT * CB * 4;
+            for (wave = 0; wave < 16; wave++) {
+                const HlqMfmaShare v = hlq_mfma_share(U, it, wave, bits, unroll);
+                CHECK(v.nt >= 0 && v.nt % bits == 0 && v.nt_pad >= v.nt && v.nt_pad % unroll == 0, "g-share");
+                for (int pos = 0; pos < v.nt; pos += bits) {
+                    int p, c;
+                    hlq_mfma_unit_of(v, v.m_lo + pos / bits, p, c);
+                    CHECK(p >= 0 && p < npairs && c >= 0 && c < it.ncb, "g-unit");
+                    if (p >= 0 && p < npairs && c >= 0 && c < it.ncb) unit_seen[p * it.ncb + c]++;
+                }
+                // loads: every position of the share, the refills past it, and what a wave without a share reads
+                for (int pos = -2; pos < v.nt_pad + 4; pos++) {
+                    int p, c;
+                    hlq_mfma_load_target(v, pos < 0 ? 0 : pos, bits, p, c);
+                    CHECK(p >= 0 && p < npairs && c >= 0 && c < it.ncb, "g-load");
+                    const int cb = it.cb0 + c, u = 2 * p, u1 = u + 1 < U - 1 ? u + 1 : U - 1;
+                    for (int b = 0; b < bits; b++)
+                        for (int uu : {u, u1}) {
+                            CHECK(uu >= 0 && uu < U && (((size_t)cb * U + uu) * bits + b) * (CB * 16) + 63 * 16 + 16 <= planes_bytes, "g-planes");
+                            const int row = g64 ? uu : (uu >> 1);
+                            CHECK(row < NT && ((size_t)cb * NT * bits + (size_t)row * bits + b) * (CB * 4) + 63 * 4 + 4 <= scale_bytes, "g-scales");
+                            CHECK(((size_t)cb * NT + row) * (CB * 4) + 63 * 4 + 4 <= zero_bytes, "g-zeros");
+                        }
+                    // the activations of the pair (and of the one requested ahead): unit min(2 p + 1, U - 1), 128 k each
+                    for (int pp : {p, p + 1 < npairs ? p + 1 : npairs - 1}) {
+                        const int ku = 2 * pp + 1 < U - 1 ? 2 * pp + 1 : U - 1;
+                        CHECK((size_t)ku * UNIT + 31 * 4 + 4 <= (size_t)K, "g-x");
+                    }
+                }
+            }
+            wave = -1;
+            for (int x : unit_seen) CHECK(x == 1, "g-cover");
+        }
+        if (weight > heaviest) heaviest = weight;
+    }
+    wave = -1; U = 0; ups = 0;
+    for (int i = 0; i < count; i++)
+        for (int x : seen[i]) CHECK(x == 1, "g-blocks");
+    // balance: no share exceeds the mean by more than one column block of the heaviest layer
+    int umax = 0;
+    for (int u : units) umax = u > umax ? u : umax;
+    CHECK(heaviest <= total / grid + umax + 1, "g-balance");
+#undef CHECK
+}
+
 }  // namespace
 
 int main(int argc, char **argv)
@@ -194,6 +274,24 @@ int main(int argc, char **argv)
                             audit_narrow(bits, g64 != 0, cr[0], cr[1], U, 3, ragged != 0, staged != 0);
                             shapes++;
                         }
+    // grouped launch of the matrix-core kernel: the LLaMA-3-8B sweep, one wide layer, mixed odd shapes, fewer blocks than shares
+    {
+        std::vector<int> su, sn;
+        for (int layer = 0; layer < 32; layer++) {
+            const int kn[7][2] = {{32, 64}, {32, 16}, {32, 16}, {32, 64}, {32, 224}, {32, 224}, {112, 64}};
+            for (auto &x : kn) { su.push_back(x[0]); sn.push_back(x[1]); }
+        }
+        for (int bits = 1; bits <= 4; bits++)
+            for (int g64 = 0; g64 < 2; g64++) {
+                audit_mfma_group(su, sn, 256, bits, g64 != 0);
+                audit_mfma_group({32}, {2004}, 256, bits, g64 != 0);
+                audit_mfma_group({4, 8, 32, 64, 1, 72, 5}, {2, 2, 4, 1, 1, 3, 3}, 16, bits, g64 != 0);
+                audit_mfma_group({1, 3, 224, 7}, {1, 300, 5, 9}, 256, bits, g64 != 0);
+                audit_mfma_group({40, 108}, {80, 216}, 256, bits, g64 != 0);
+                audit_mfma_group({2}, {1}, 1, bits, g64 != 0);
+                shapes += 6;
+            }
+    }
     long total = 0;
     for (auto &kv : g_viol) {
         std::printf("category %s %ld\n", kv.first.c_str(), kv.second);

@@ -1,5 +1,8 @@
-"""Grouped launch of independent GEMVs (elutq_hlq_gemv_group_*) against the single-GEMV entry
-point: same tiles, same K slicing, so the same bits."""
+"""Grouped launch of independent GEMVs (elutq_hlq_gemv_group_*).  On the LUT engine against the single-GEMV entry
+point: same tiles, same K slicing, so the same bits.  On the matrix-core engine (the library's own choice for a group
+whose layers have whole units of 128 k) a tile covers all of K, so the sums differ from the single-GEMV launch in
+order only: the float64 oracle to the dense path's bars, bit-identical repeats, bit-exact where the arithmetic is
+exact, and within an fp16 rounding of the LUT engine."""
 import ctypes
 
 import numpy as np
@@ -25,8 +28,15 @@ def single(mod, x, ksplit):
     return y
 
 
+@pytest.fixture
+def lut_engine():
+    _lib.set_gemv_engine("lut")
+    yield
+    _lib.set_gemv_engine("auto")
+
+
 @pytest.mark.parametrize("bits,group", [(2, 128), (3, 128), (2, 64), (4, 64), (1, 128)])
-def test_group_equals_single_calls(cuda, bits, group):
+def test_group_equals_single_calls(cuda, lut_engine, bits, group):
     shapes = [(512, 128), (1024, 70), (4096, 256), (8192, 64), (128, 1), (9216, 130), (640, 192)]
     if group == 64:
         shapes += [(704, 100), (4160, 64)]                        # K ends half way through the last unit of 128
@@ -47,7 +57,7 @@ def test_group_equals_single_calls(cuda, bits, group):
     grp.close()
 
 
-def test_group_of_a_whole_layer_at_full_size(cuda):
+def test_group_of_a_whole_layer_at_full_size(cuda, lut_engine):
     names = list(LLAMA3_8B_SHAPES)
     mods = [make_device_layer(*LLAMA3_8B_SHAPES[n], 2, 128, seed=i, device=cuda) for i, n in enumerate(names)]
     xs = [torch.randn(1, m.in_features, device=cuda).half() for m in mods]
@@ -79,7 +89,110 @@ def test_group_of_a_whole_layer_at_full_size(cuda):
     grp.close()
 
 
-def test_group_rejects_bad_arguments(cuda):
+@pytest.mark.parametrize("engine", ["auto", "mfma"])
+@pytest.mark.parametrize("bits,group", [(2, 128), (3, 128), (2, 64), (4, 64), (1, 128), (4, 128), (3, 64), (1, 64)])
+def test_group_on_the_matrix_cores_matches_oracle(cuda, engine, bits, group):
+    """Layers of every kind in one group -- one unit, an odd unit count, more pairs than waves, ragged N, a single
+    column, more column blocks than a tile holds, bias -- against the float64 oracle; repeats give the same bits
+    (the second run also finds the ring and the LDS tables as the first left them)."""
+    _lib.set_gemv_engine(engine)
+    try:
+        shapes = [(512, 128), (1024, 70), (4096, 256), (8192, 64), (128, 1), (9216, 130), (640, 192), (384, 1100),
+                  (14336, 192), (256, 64)]
+        layers = [make_layer(k, n, bits=bits, group=group, seed=10 * i + bits, bias=(i % 2 == 0)) for i, (k, n) in enumerate(shapes)]
+        mods = [HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, L.group, L.bias, cuda) for L in layers]
+        xs = [torch.from_numpy(L.x).to(cuda) for L in layers]
+        ys = [torch.full((1, L.n), float("nan"), dtype=torch.float16, device=cuda) for L in layers]
+        grp = GemvGroup(mods, xs, ys)
+        prev = None
+        for rep in range(3):
+            for y in ys:
+                y.fill_(float("nan"))
+            grp.run()
+            torch.cuda.synchronize()
+            outs = [y[0].cpu().numpy().copy() for y in ys]
+            for L, o in zip(layers, outs):
+                ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, L.group, L.bias)
+                assert O.rel_err(o, ref) <= 1e-2, (L.k, L.n, rep)
+                assert np.max(np.abs(o.astype(np.float64) - ref)) <= 2.0 ** -10 * max(1.0, np.max(np.abs(ref)))
+            assert prev is None or all(np.array_equal(a, b) for a, b in zip(prev, outs))
+            prev = outs
+        grp.close()
+    finally:
+        _lib.set_gemv_engine("auto")
+
+
+@pytest.mark.parametrize("bits,group", [(2, 128), (3, 64), (4, 128), (1, 64)])
+def test_group_on_the_matrix_cores_is_exact_on_integer_inputs(cuda, bits, group):
+    """x in {-2..2}, power-of-two scales, quarter-integer zeros: every digit, product and partial sum is exactly
+    representable in fp32, so the grouped launch == the float64 result rounded once to fp16, bit for bit, whatever the
+    order of its sums."""
+    r = np.random.default_rng(7)
+    layers = []
+    for (k, n) in [(768, 128), (4096, 200), (9216, 64), (384, 520)]:
+        L = make_layer(k, n, bits=bits, group=group, seed=k + n)
+        L.x[:] = r.integers(-2, 3, (1, k)).astype(np.float16)
+        L.w_scale[:] = (2.0 ** r.integers(-3, 1, L.w_scale.shape)).astype(np.float16)
+        L.w_zero[:] = (r.integers(-8, 9, L.w_zero.shape) / 4.0).astype(np.float16)
+        layers.append(L)
+    mods = [HLQLinear.from_export_arrays(L.w_quant, L.w_scale, L.w_zero, L.group, None, cuda) for L in layers]
+    xs = [torch.from_numpy(L.x).to(cuda) for L in layers]
+    ys = [torch.zeros(1, L.n, dtype=torch.float16, device=cuda) for L in layers]
+    grp = GemvGroup(mods, xs, ys)
+    grp.run()
+    torch.cuda.synchronize()
+    for L, y in zip(layers, ys):
+        ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, L.group)
+        assert np.array_equal(y[0].cpu().numpy(), ref.astype(np.float16))
+    grp.close()
+
+
+def test_group_of_whole_layers_on_both_engines(cuda):
+    """Three LLaMA-3-8B layers' projections as one group on the library's choice of engine (the matrix cores)
+    against the dense fp32 product and against the LUT engine's group: within an fp16 rounding; replayed from a
+    captured graph with eager work in between, every replay the same bits."""
+    names = list(LLAMA3_8B_SHAPES)
+    mods = [make_device_layer(*LLAMA3_8B_SHAPES[n], 2, 128, seed=i, device=cuda) for i, n in enumerate(names)]
+    xs = [torch.randn(1, m.in_features, device=cuda).half() for m in mods]
+    out = {}
+    for engine in ("auto", "lut"):
+        _lib.set_gemv_engine(engine)
+        try:
+            ys = [torch.zeros(1, m.out_features, dtype=torch.float16, device=cuda) for m in mods * 3]
+            grp = GemvGroup(mods * 3, xs * 3, ys)
+            grp.run()
+            torch.cuda.synchronize()
+            for m, x, y in zip(mods, xs, ys):
+                ref = x.float() @ m.dequantize().float().t()
+                assert (y.float() - ref).abs().max() <= 1e-2 * ref.pow(2).mean().sqrt()
+            for i in range(len(mods)):          # the copies of a layer: same sums, in an order that depends on where its tiles fall
+                for j in (1, 2):
+                    assert (ys[i].float() - ys[i + j * len(mods)].float()).abs().max() <= 2.0 ** -9 * max(1.0, ys[i].float().abs().max().item())
+                    assert engine != "lut" or torch.equal(ys[i], ys[i + j * len(mods)])
+            g = torch.cuda.CUDAGraph()
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                grp.run()
+            s.synchronize()
+            with torch.cuda.graph(g, stream=s):
+                grp.run()
+            want = [y.clone() for y in ys]
+            for _ in range(3):
+                for y in ys:
+                    y.zero_()
+                g.replay()
+                torch.cuda.synchronize()
+                _ = torch.randn(32, 32, device=cuda) @ torch.randn(32, 32, device=cuda)
+                assert all(torch.equal(a, b) for a, b in zip(ys, want))
+            out[engine] = want[:len(mods)]
+            grp.close()
+        finally:
+            _lib.set_gemv_engine("auto")
+    for a, b in zip(out["auto"], out["lut"]):
+        assert (a.float() - b.float()).abs().max() <= 2.0 ** -9 * max(1.0, b.float().abs().max().item())
+
+
+def test_group_rejects_bad_arguments(cuda, lut_engine):
     L = _lib.lib()
     m = make_device_layer(512, 64, 2, 128, seed=0, device=cuda)
     x = torch.zeros(1, 512, dtype=torch.float16, device=cuda)

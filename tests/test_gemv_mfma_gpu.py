@@ -1,5 +1,5 @@
 """The matrix-core GEMV kernel (ELUTQ_GEMV_ENGINE_MFMA: plane bits as fp4 operands of v_mfma_f32_32x32x64_f8f6f4
-against fp8 terms of the activations) behind the same C-ABI entry points as the LUT kernel, to the same bars:
+against fp4 base-7 digits of the activations) behind the same C-ABI entry points as the LUT kernel, to the same bars:
 float64 oracle within rel_err <= 1e-2 (observed: the final fp16 rounding), bit-exact where the arithmetic is exact,
 the fused prologues / epilogue and the hand-over of K slices bit for bit what the unfused calls give, and within an
 fp16 rounding of the LUT kernel on the same inputs.  Reference path: arm_gemm (m = 1),
@@ -56,6 +56,32 @@ def test_mfma_gemv_matches_oracle(cuda, k, n, bits, group, ksplit, waves):
     assert np.array_equal(y, run(m, L.x, cuda)[0])
 
 
+@pytest.mark.parametrize("k,n,bits,group,bias", [(4224, 16640, 2, 128, False), (8192, 16500, 3, 64, True), (4096, 16400, 1, 128, False)])
+def test_mfma_wide_layers_stream_over_all_of_k(cuda, k, n, bits, group, bias):
+    """A plain call on a layer with more column blocks than compute units runs on the streaming kernel (every workgroup an
+    equal share of the column blocks over all of K; with the engine on its default only where K > 4096): an odd unit
+    count, ragged N, bias, more pairs than waves; 4096 sampled columns against the float64 oracle evaluated on those
+    columns, bit-identical repeats, y(-x) = -y(x) exactly, and a column slice of the layer gives the same columns."""
+    L = make_layer(k, n, bits=bits, group=group, seed=k + n, bias=bias)
+    for engine in ("mfma", "auto"):
+        _lib.set_gemv_engine(engine)
+        m = to_mod(L, cuda)
+        print(f"wide layer K={k} N={n} engine {engine}", flush=True)
+        y = run(m, L.x, cuda)[0]
+        idx = np.sort(np.random.default_rng(n).choice(n, 4096, replace=False))
+        idx[:3], idx[-3:] = (0, 1, 63), (n - 64, n - 2, n - 1)
+        ref = O.gemv_f64(L.x[0], L.w_quant[:, idx], L.w_scale[:, idx], L.w_zero[idx], group, None if L.bias is None else L.bias[idx])
+        assert O.rel_err(y[idx], ref) <= TOL
+        assert np.max(np.abs(y[idx].astype(np.float64) - ref)) <= 2.0 ** -10 * max(1.0, np.max(np.abs(ref)))
+        assert np.array_equal(y, run(m, L.x, cuda)[0])
+        if not bias:
+            assert np.array_equal(-run(m, (-L.x).astype(np.float16), cuda)[0], y)
+        sub = HLQLinear.from_export_arrays(L.w_quant[:, 4096:8192], L.w_scale[:, 4096:8192], L.w_zero[4096:8192], group,
+                                           None if L.bias is None else L.bias[4096:8192], cuda)
+        ys = run(sub, L.x, cuda)[0]
+        assert np.max(np.abs(ys.astype(np.float64) - y[4096:8192].astype(np.float64))) <= 2.0 ** -9 * max(1.0, np.max(np.abs(ref)))
+
+
 def test_mfma_refuses_more_than_two_pairs_per_wave(cuda):
     L = make_layer(4096, 64, bits=2, group=128, seed=1)
     m = to_mod(L, cuda, 1, 2)                          # 16 pairs on 2 waves
@@ -73,7 +99,7 @@ def test_mfma_takes_whole_units_only(cuda):
 
 @pytest.mark.parametrize("bits,group,ksplit", [(2, 128, 1), (2, 128, 2), (3, 64, 0), (4, 128, 3), (1, 64, 0)])
 def test_mfma_bit_exact_on_integer_inputs(cuda, lutref, bits, group, ksplit):
-    """x in {-2..2}, power-of-two scales, quarter-integer zeros: every fp8 term, product and partial sum is exactly
+    """x in {-2..2}, power-of-two scales, quarter-integer zeros: every digit, product and partial sum is exactly
     representable, so GPU == float64 == the reference's fp16 chain, bit for bit."""
     r = np.random.default_rng(5)
     k, n = 768, 128
@@ -107,8 +133,9 @@ def test_mfma_closed_forms_unit_vectors_and_range(cuda):
         e[0, kk] = 1
         y = run(m, e, cuda)[0]
         assert np.array_equal(y, w[:, kk].astype(np.float32).astype(np.float16)), kk
-    # every fp16 value is the sum of its three fp8 terms: against a one-plane layer with scale 0.5 and zero 0 a single
-    # activation of any magnitude and mantissa must come back as 0.5 * x where the plane bit is set, bit for bit
+    # the largest activation of a half unit is held exactly by its base-7 digits: against a one-plane layer with scale 0.5
+    # and zero 0 a single activation of any magnitude and mantissa must come back as 0.5 * x where the plane bit is set,
+    # bit for bit
     r = np.random.default_rng(3)
     one = r.integers(0, 2, (1, 128, 512), dtype=np.uint8)
     half = HLQLinear.from_export_arrays(O.pack_planes(one), np.full((1, 128, 4), 0.5, np.float16), np.zeros((128, 4), np.float16),
@@ -120,7 +147,7 @@ def test_mfma_closed_forms_unit_vectors_and_range(cuda):
         e[0, kk] = val
         y = run(half, e, cuda)[0]
         assert np.array_equal(y, (one[0, :, kk].astype(np.float32) * np.float32(val) * np.float32(0.5)).astype(np.float16)), (kk, val)
-        # beside a much larger activation in the same half unit the small one keeps the bits above 2^-15 of the large one
+        # beside a much larger activation in the same half unit the small one keeps the bits above 2^-18 of the large one
         if abs(float(val)) >= 512:
             continue
         e[0, kk ^ 1] = np.float16(float(val) * 64)
