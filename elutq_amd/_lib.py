@@ -30,6 +30,7 @@ SIGNATURES = {
     "elutq_hlq_gemv_int8lut_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp]),
     "elutq_hlq_gemv_fused_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
     "elutq_hlq_gemv_slices": (_ci, [_ci] * 6),
+    "elutq_hlq_gemv_fault_count": (_ci, [_ci]),
     "elutq_hlq_set_gemv_engine": (_ci, [_ci]),
     "elutq_hlq_get_gemv_engine": (_ci, []),
     "elutq_hlq_static_scratch_bytes": (_sz, []),
@@ -68,7 +69,8 @@ class GemvFusion(ctypes.Structure):
     _fields_ = [("prologue", ctypes.c_int), ("eps", ctypes.c_float),
                 ("d_norm_weight", ctypes.c_void_p), ("d_residual", ctypes.c_void_p),
                 ("d_slices_out", ctypes.c_void_p), ("d_slices_in", ctypes.c_void_p),
-                ("n_slices_in", ctypes.c_int), ("d_x_out", ctypes.c_void_p)]
+                ("n_slices_in", ctypes.c_int), ("d_x_out", ctypes.c_void_p),
+                ("slices_out_bytes", ctypes.c_size_t), ("slices_in_bytes", ctypes.c_size_t)]
 
 
 class GemvProblem(ctypes.Structure):

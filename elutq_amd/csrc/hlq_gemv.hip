@@ -25,6 +25,7 @@
 //  * slices are combined through a workspace by the last workgroup to arrive (fixed
 //    summation order, so results are deterministic).
 #include <hip/hip_runtime.h>
+#include <mutex>
 #include <type_traits>
 #include <vector>
 #include <stdint.h>
@@ -532,12 +533,40 @@ void choose_shape(const HlqGeo &g, int &ksplit, int &waves)
         const int max_ups = g.ncb >= 128 ? 48 : 32;
         const int by_len = (g.U + max_ups - 1) / max_ups;
         if (ksplit < by_len) ksplit = by_len;
+        // 3 -> 4 and 5..7 -> 8 slices where the slots of the meeting then fit the head of a workspace: slots are used
+        // for 2, 4 or 8 slices only (slices_meet_slots), and they cost one trip through memory where counters cost three
+        const int up = ksplit == 3 ? 4 : (ksplit > 4 && ksplit < 8 ? 8 : ksplit);
+        if (up != ksplit && up <= g.U && (size_t)(up - 1) * g.ncb * HLQ_CB * sizeof(float) <= (size_t)HLQ_WS_COUNTER_BYTES &&
+            g.ncb * up <= NUM_CU) ksplit = up;
         if (ksplit > g.U) ksplit = g.U;
     }
     if (waves <= 0) waves = 16;
 }
 
 int g_gemv_engine = ELUTQ_GEMV_ENGINE_AUTO;
+
+// Count of slot meetings whose bounded wait ran out (slices_meet_slots), one word per GPU, held until the process ends.
+// The name is a host-side stand-in: the device address is looked up once per device.
+static __device__ unsigned g_gemv_fault_word[4];
+std::mutex g_fault_lock;
+unsigned *g_fault_ptr[64] = {};
+
+int fault_address(unsigned **out)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return ELUTQ_ERR_HIP;
+    std::lock_guard<std::mutex> hold(g_fault_lock);
+    if (!g_fault_ptr[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_gemv_fault_word)) != hipSuccess || !p) return ELUTQ_ERR_HIP;
+        g_fault_ptr[dev] = (unsigned *)p;
+    }
+    *out = g_fault_ptr[dev];
+    return ELUTQ_OK;
+}
+
+// Test hook (elutq_test_gemv_meeting): a slice that leaves without storing, and the poll limit of the waiting wave.
+int g_test_drop_slice = -1, g_test_spin_limit = SLICE_SPIN_LIMIT;
 
 // The launch shape of a batch-1 GEMV: which kernel, K slices, units per slice, waves per workgroup.  One
 // function for the launch itself and for the queries about it (elutq_hlq_gemv_slices, _accepts_slices).
@@ -697,6 +726,7 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
     a.partial = nullptr; a.counters = nullptr; a.meet_slots = 0;
     a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
     a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr; a.lut_int8 = 0;
+    a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1;
     if (fusion) {
         if (fusion->prologue < 0 || fusion->prologue > 2) return ELUTQ_ERR_TUNING;
         if (fusion->prologue == 1 && !fusion->d_norm_weight) return ELUTQ_ERR_NULL;
@@ -721,10 +751,14 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
         a.x_out = (HLQ_GLOBAL uint16_t *)fusion->d_x_out;
         stage_bytes = (size_t)K * sizeof(uint16_t);
         if (shape_lds_bytes(sh, bits) + stage_bytes > (size_t)MAX_LDS) return ELUTQ_ERR_SHAPE;
+        if (fusion->slices_in_bytes < (size_t)fusion->n_slices_in * K * sizeof(float)) return ELUTQ_ERR_WORKSPACE;
     }
     if (fusion && fusion->d_slices_out) {
         // the K slices stay unsummed for the next launch: nothing else may be due in the output stage
         if (ksplit < 2 || d_bias || a.residual || d_extra || N % HLQ_CB != 0) return ELUTQ_ERR_TUNING;
+        // every slice writes a row of N floats: the buffer's size is the caller's word, checked here because a row
+        // too many would land on whatever lies behind the buffer
+        if (fusion->slices_out_bytes < (size_t)ksplit * N * sizeof(float)) return ELUTQ_ERR_WORKSPACE;
         a.defer = 1;
         a.partial = (HLQ_GLOBAL float *)fusion->d_slices_out;
     } else if (ksplit > 1) {
@@ -734,9 +768,17 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
             return ELUTQ_ERR_WORKSPACE;
         // slots that fit the head of the workspace, which every kernel leaves zero-filled, are filled and emptied
         // instead of counted (slices_meet_slots); else arrival counters there and the partial sums behind it
-        if ((size_t)(ksplit - 1) * g.ncb * HLQ_CB * sizeof(float) <= (size_t)WS_COUNTER_BYTES) {
+        // -- with 2, 4 or 8 slices only: the fixed waiter must not share an XCD with a slice it waits for (slices_meet_slots)
+        if ((size_t)(ksplit - 1) * g.ncb * HLQ_CB * sizeof(float) <= (size_t)WS_COUNTER_BYTES &&
+            (ksplit == 2 || ksplit == 4 || ksplit == 8)) {
             a.meet_slots = 1;
             a.partial = (HLQ_GLOBAL float *)d_workspace;
+            unsigned *fault = nullptr;
+            rc = fault_address(&fault);
+            if (rc != ELUTQ_OK) return rc;
+            a.fault = (HLQ_GLOBAL unsigned *)fault;
+            a.spin_limit = g_test_spin_limit;
+            a.drop_slice = g_test_drop_slice;
         } else {
             a.counters = (HLQ_GLOBAL unsigned *)d_workspace;
             a.partial = (HLQ_GLOBAL float *)((unsigned char *)d_workspace + WS_COUNTER_BYTES);
@@ -775,6 +817,28 @@ extern "C" int elutq_hlq_set_gemv_engine(int engine)
 }
 
 extern "C" int elutq_hlq_get_gemv_engine(void) { return g_gemv_engine; }
+
+extern "C" int elutq_hlq_gemv_fault_count(int clear)
+{
+    unsigned *p = nullptr;
+    const int rc = fault_address(&p);
+    if (rc != ELUTQ_OK) return rc;
+    unsigned h = 0;
+    if (hipDeviceSynchronize() != hipSuccess || hipMemcpy(&h, p, sizeof(h), hipMemcpyDeviceToHost) != hipSuccess) return ELUTQ_ERR_HIP;
+    if (clear && h && hipMemset(p, 0, sizeof(h)) != hipSuccess) return ELUTQ_ERR_HIP;
+    return h > 0x7fffffffu ? 0x7fffffff : (int)h;
+}
+
+// Not part of the C ABI (no declaration in include/elutq_hip.h): lets a test force the give-up path of the slot meeting
+// from the host with every kernel still ending normally.  drop_slice >= 0: that K slice of the following slot-meeting
+// launches leaves without storing its sums; spin_limit: polls before the waiting wave gives up (<= 0: the default).
+// elutq_test_gemv_meeting(-1, 0) restores normal operation.
+extern "C" int elutq_test_gemv_meeting(int drop_slice, int spin_limit)
+{
+    g_test_drop_slice = drop_slice < 0 ? -1 : drop_slice;
+    g_test_spin_limit = spin_limit > 0 ? spin_limit : SLICE_SPIN_LIMIT;
+    return ELUTQ_OK;
+}
 
 // Whether a launch of this shape (ksplit / waves as the call would pass them) takes `n_slices` handed-over
 // K slices in its RMSNorm prologue: the same steps and limits as the launch itself.
@@ -935,6 +999,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
         }
         a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
         a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr; a.lut_int8 = 0;
+        a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1;
         const int ns = a.spw < depth_of(bits) ? a.spw : depth_of(bits);
         if (ns > nslot) nslot = ns;
         if (mfma) continue;                          // its tile list is made below, over all layers at once

@@ -55,6 +55,10 @@ struct GemvArgs {
     const HLQ_GLOBAL float *slices_in;    // fp32 [n_slices_in][K]
     HLQ_GLOBAL uint16_t *x_out;           // fp16 [K] or null: the combined x, written by workgroup (0, 0)
     int lut_int8;                         // host side only: launch the instance whose tables are quantized to int8 (GEMV_INT8)
+    // the slot meeting's bounded wait (meet_slots == 1)
+    HLQ_GLOBAL unsigned *fault;           // the library's count of meetings that gave up (never null when meet_slots)
+    int spin_limit;                       // polls before a waiting wave gives up
+    int drop_slice;                       // -1; tests only: this slice leaves without storing its sums, so that the wait runs out
 };
 
 #ifdef HLQ_TIMING
@@ -390,14 +394,19 @@ __device__ __forceinline__ void lds_barrier()
 // agent-scope store (+0.0 goes in as -0.0, which adds the same) and leaves.  The workgroup of the last slice
 // keeps its own sum in registers, reads the other slots until none is empty, adds them in slice order and puts
 // the zeros back.  One trip through memory lies between the last store and the result (the counter needed
-// three dependent ones: store acknowledged, ticket drawn, slots read).  Who waits is fixed, so it must be
-// certain that the others run: the last slice has the highest workgroup index of its column block (slices
-// are the fastest grid dimension), and a dispatcher places workgroups in index order.  Take the lowest-indexed
-// workgroup still waiting for a place: every workgroup that holds a place ahead of it waits, if at all, for
-// ones with lower indices still -- which therefore hold their places or are done -- so places keep coming
-// free, whatever else shares the GPU.  (A launch whose workgroups walk a list of tiles cannot promise that
-// and keeps the counters.)  The wait is bounded all the same (SLICE_SPIN_LIMIT reads, about a second): a
-// wave that gives up returns what it has, and the kernel ends.
+// three dependent ones: store acknowledged, ticket drawn, slots read).
+//
+// Who waits is fixed, so the others must be certain to run.  The last slice has the highest workgroup index of its
+// column block (slices are the fastest grid dimension).  Workgroups go to the eight XCDs of the chip round robin by
+// index and every XCD places its own in index order, so with 2, 4 or 8 slices -- the only counts the launcher uses
+// slots for -- waiting workgroups sit on XCDs 1, 3, 5, 7 only and each waits for XCDs with lower numbers: XCD 0
+// never holds a waiter and drains whatever else shares the GPU, then XCD 1's waiters have what they wait for, and so
+// on up (tests/test_slot_meeting_model.py replays that placement for several launches sharing the chip, and shows
+// the cycle that three slices allow).  The argument rests on how the dispatcher places workgroups, which no document
+// promises, so the wait is bounded all the same (GemvArgs.spin_limit polls, about a second by default).  A wave that
+// gives up does not pass a partial result off as a sum: it counts the event in the library's fault word
+// (elutq_hlq_gemv_fault_count), makes its 64 outputs NaN, and empties the slots it can see; a slice that arrives
+// later still dirties its slot, so after a fault the workspace must be zero-filled again before it is reused.
 constexpr int SLICE_SPIN_LIMIT = 1 << 20;
 
 // Called by one whole wave (lane = column n of the block); true in the wave that holds the complete sum.
@@ -405,6 +414,7 @@ __device__ __forceinline__ bool slices_meet_slots(const GemvArgs &a, int slice, 
 {
     HLQ_GLOBAL float *mine = a.partial + (size_t)slice * npad + n;
     if (slice != a.ksplit - 1) {
+        if (slice == a.drop_slice) return false;        // (tests of the give-up path)
         const float v = __float_as_uint(total) == 0u ? -0.0f : total;
         __hip_atomic_store(mine, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return false;
@@ -412,6 +422,7 @@ __device__ __forceinline__ bool slices_meet_slots(const GemvArgs &a, int slice, 
     sum = 0.f;
     const int others = a.ksplit - 1;
     int spins = 0;
+    bool gave_up = false;
     for (int s0 = 0; s0 < others; s0 += 8) {            // eight independent loads in flight at a time
         float v[8];
         for (;;) {
@@ -422,7 +433,8 @@ __device__ __forceinline__ bool slices_meet_slots(const GemvArgs &a, int slice, 
                 v[j] = __hip_atomic_load(&a.partial[(size_t)sl * npad + n], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 here = here && __float_as_uint(v[j]) != 0u;
             }
-            if (__all(here) || ++spins > SLICE_SPIN_LIMIT) break;
+            if (__all(here)) break;
+            if (++spins > a.spin_limit) { gave_up = true; break; }
             __builtin_amdgcn_s_sleep(1);
         }
 #pragma unroll
@@ -433,6 +445,10 @@ __device__ __forceinline__ bool slices_meet_slots(const GemvArgs &a, int slice, 
             }
     }
     sum += total;
+    if (gave_up) {                                      // wave-uniform
+        sum = __builtin_nanf("");
+        if ((n & (HLQ_CB - 1)) == 0) __hip_atomic_fetch_add(a.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     return true;
 }
 

@@ -64,21 +64,28 @@ int elutq_hlq_gemv_f16_static(const void *d_planes, const void *d_scales, const 
     void *ws = nullptr;
     size_t ws_bytes = 0;
     const bool bad_args = slices == 0 || !d_planes || !d_scales || !d_zeros || !d_x || !d_y;    // the launch reports which
-    if (slices > 1 && !bad_args) {
+    if (!bad_args) {
         const HlqGeo g = hlq_geo(K, N, bits, group);
         const size_t need = (size_t)HLQ_WS_COUNTER_BYTES + (size_t)slices * g.ncb * HLQ_CB * sizeof(float);
-        if ((size_t)g.ncb * sizeof(unsigned) > (size_t)HLQ_WS_COUNTER_BYTES || need > STATIC_SCRATCH_BYTES)
+        if (slices > 1 && ((size_t)g.ncb * sizeof(unsigned) > (size_t)HLQ_WS_COUNTER_BYTES || need > STATIC_SCRATCH_BYTES))
             return ELUTQ_ERR_STATIC_LIMIT;
+        // the launch always gets the array (an engine other than the one the figure above is for may slice where that
+        // one does not; its counters are at zero then, as every kernel leaves them)
         const int rc = scratch_address(&ws);
         if (rc != ELUTQ_OK) return rc;
         ws_bytes = STATIC_SCRATCH_BYTES;
-        hipLaunchKernelGGL(clear_counters_kernel, dim3((g.ncb + 255) / 256), dim3(256), 0, (hipStream_t)stream,
-                           (unsigned *)ws, g.ncb);
-        if (hipGetLastError() != hipSuccess) return ELUTQ_ERR_HIP;
+        if (slices > 1 && (size_t)g.ncb * sizeof(unsigned) <= (size_t)HLQ_WS_COUNTER_BYTES) {
+            hipLaunchKernelGGL(clear_counters_kernel, dim3((g.ncb + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                               (unsigned *)ws, g.ncb);
+            if (hipGetLastError() != hipSuccess) return ELUTQ_ERR_HIP;
+        }
     }
-    // shape, pointer and plane-count errors are reported by the launch itself, as for elutq_hlq_gemv_f16
-    return hlq_gemv_with_extra(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, ws, ws_bytes, stream,
-                               nullptr, 0, 0, nullptr);
+    // shape, pointer and plane-count errors are reported by the launch itself, as for elutq_hlq_gemv_f16.  The launch
+    // checks the array's size against the slices it actually makes (the figure above is the wide-tile kernel's, an
+    // upper bound for the LUT kernels; another engine may slice differently): too small reads as the static limit.
+    const int rc = hlq_gemv_with_extra(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, ws, ws_bytes, stream,
+                                       nullptr, 0, 0, nullptr);
+    return rc == ELUTQ_ERR_WORKSPACE && ws ? ELUTQ_ERR_STATIC_LIMIT : rc;
 }
 
 }  // extern "C"

@@ -312,7 +312,9 @@ class HLQLinear(nn.Module):
                             slices_out.data_ptr() if slices_out is not None else None,
                             slices_in.data_ptr() if slices_in is not None else None,
                             slices_in.shape[0] if slices_in is not None else 0,
-                            x_out.data_ptr() if x_out is not None else None)
+                            x_out.data_ptr() if x_out is not None else None,
+                            slices_out.numel() * slices_out.element_size() if slices_out is not None else 0,
+                            slices_in.numel() * slices_in.element_size() if slices_in is not None else 0)
         if slices_out is not None and (slices_out.dtype != torch.float32 or slices_out.numel() < self.slices * self.out_features):
             raise ValueError("slices_out must be fp32 [slices, out_features]")
         if slices_in is not None and (slices_in.dtype != torch.float32 or slices_in.dim() != 2

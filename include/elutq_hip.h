@@ -217,7 +217,21 @@ typedef struct elutq_gemv_fusion {
     const void *d_slices_in;    /* consumer of deferred K slices (n_slices_in > 0) */
     int n_slices_in;            /* 0 = none */
     void *d_x_out;              /* fp16 [K] or NULL (consumer only) */
+    size_t slices_out_bytes;    /* size of d_slices_out: at least S * N * 4 or the call returns ELUTQ_ERR_WORKSPACE */
+    size_t slices_in_bytes;     /* size of d_slices_in: at least n_slices_in * K * 4 or ELUTQ_ERR_WORKSPACE */
 } elutq_gemv_fusion;
+
+/*
+ * The K slices of a GEMV launch that meet through the zero-kept head of the workspace have one workgroup per column
+ * block wait for the others' partial sums.  That wait is bounded (about a second); should it ever run out -- the
+ * launch could not get its workgroups placed, say because many launches oversubscribe the GPU -- the block's 64
+ * outputs are written as NaN and the event is counted in a word the library keeps on each GPU.  This call returns
+ * that count for the current device (>= 0; it synchronizes with the device) and sets it back to zero if `clear`
+ * is non-zero; negative: an elutq_status.  After a non-zero count the workspaces of the affected calls must be
+ * zero-filled again (elutq_hlq_workspace_init) before they are reused.  No counterpart in the reference, whose
+ * thread pool waits without a bound (C++/common/include/threadpool.h:107-113).
+ */
+int elutq_hlq_gemv_fault_count(int clear);
 
 /* K slices the GEMV launch of this shape is divided into (ksplit / waves as in
  * elutq_hlq_gemv_f16_tuned, 0 = default); 0 for an unsupported shape or tuning.  With ksplit = 0 the

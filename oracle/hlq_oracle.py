@@ -291,7 +291,12 @@ def lut_int8(x, actk: int):
     """x fp16 [K] -> (q int8 [K/4, 16], scale fp16 [K/actk]).  Per group of `actk` activations
     (arm_t_mac_kernal.cpp:22-48): the fp16 subset sums of lut_float, scale = fp16(max|entry| / 127)
     (:50), q = saturate_int8(round-to-nearest-even(fp16(entry / scale))) (:59-90; a NaN quotient,
-    0 / 0 in a group of zeros, converts to 0, an infinite one saturates)."""
+    0 / 0 in a group of zeros, converts to 0, an infinite one saturates).
+    One deliberate difference: the reference's quantizing loop runs `for k < Actk; k += 16` over a group's
+    4 * Actk table entries (:52-58), i.e. it converts only the first Actk of them and leaves the rest of
+    its output unwritten; here every entry of the group is converted with the group's scale.  The reference
+    definition with that loop bound corrected, in other words: parity with the reference is unpinned beyond
+    the first Actk entries of a group (nothing in the reference calls, loads or tests the variant)."""
     lut = lut_float(x)
     per = actk // 4
     ng = lut.shape[0] // per

@@ -289,6 +289,65 @@ def test_k_slices_whose_sums_are_zero(cuda, ksplit):
     assert O.rel_err(_tuned(m, xr, ws, ksplit, 4).cpu().numpy()[0], ref) <= TOL
 
 
+@pytest.mark.parametrize("ksplit,drop", [(2, 0), (4, 0), (4, 2), (8, 5)])
+def test_a_slot_meeting_that_gives_up_says_so(cuda, ksplit, drop):
+    """The bounded wait of the slot meeting, forced from the host: one slice of every column block leaves without storing
+    its sums (a test hook of the library, outside the C ABI) and the waiting wave polls 32 times instead of a million.
+    Every kernel ends normally; the outputs are NaN, not a partial sum passed off as the result; the fault count of the
+    GPU says how many column blocks gave up; and -- no slice arrives late in this forced case -- the slots are empty
+    again, so the next, undisturbed call on the same workspace gives the right result and counts nothing."""
+    import ctypes
+    L = make_layer(1024, 200, bits=2, group=128, seed=5 + ksplit)
+    m = to_mod(L, cuda)
+    x = torch.from_numpy(L.x).to(cuda)
+    ws = torch.zeros(max(m.workspace_bytes, 1 << 20), dtype=torch.uint8, device=cuda)
+    lib = _lib.lib()
+    hook = lib.elutq_test_gemv_meeting
+    hook.restype, hook.argtypes = ctypes.c_int, [ctypes.c_int, ctypes.c_int]
+    assert lib.elutq_hlq_gemv_fault_count(1) >= 0
+    ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, 128)
+    good = _tuned(m, x, ws, ksplit, 4).clone()
+    assert O.rel_err(good.cpu().numpy()[0], ref) <= TOL and lib.elutq_hlq_gemv_fault_count(0) == 0
+    try:
+        assert hook(drop, 32) == 0
+        print(f"slot meeting forced to give up: ksplit {ksplit}, slice {drop} dropped", flush=True)
+        y = _tuned(m, x, ws, ksplit, 4)
+        torch.cuda.synchronize()
+    finally:
+        assert hook(-1, 0) == 0
+    assert torch.isnan(y).all()
+    assert lib.elutq_hlq_gemv_fault_count(0) == 4                  # ceil(200 / 64) column blocks
+    assert lib.elutq_hlq_gemv_fault_count(1) == 4 and lib.elutq_hlq_gemv_fault_count(0) == 0
+    assert not ws[:65536].any()
+    assert torch.equal(_tuned(m, x, ws, ksplit, 4), good) and lib.elutq_hlq_gemv_fault_count(0) == 0
+
+
+def test_slots_are_for_two_four_or_eight_slices(cuda):
+    """With 3, 5, 6 or 7 slices a waiting workgroup could share an XCD with a slice it waits for, so those launches meet
+    through arrival counters (nothing waits); the library's own choice of slices avoids them where slots fit: the result
+    is the oracle's either way, and a dropped slice (the test hook acts on slot meetings only) disturbs nothing."""
+    import ctypes
+    lib = _lib.lib()
+    hook = lib.elutq_test_gemv_meeting
+    hook.restype, hook.argtypes = ctypes.c_int, [ctypes.c_int, ctypes.c_int]
+    L = make_layer(13440, 128, bits=2, group=128, seed=9)              # 105 units: 3, 5, 6 and 7 slices come out as asked
+    m = to_mod(L, cuda)
+    x = torch.from_numpy(L.x).to(cuda)
+    ws = torch.zeros(max(m.workspace_bytes, 1 << 20), dtype=torch.uint8, device=cuda)
+    ref = O.gemv_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, 128)
+    try:
+        assert hook(0, 32) == 0
+        for ks in (3, 5, 6, 7):
+            assert lib.elutq_hlq_gemv_slices(13440, 128, 2, 128, ks, 16) == ks
+            assert O.rel_err(_tuned(m, x, ws, ks, 16).cpu().numpy()[0], ref) <= TOL
+    finally:
+        assert hook(-1, 0) == 0
+    assert lib.elutq_hlq_gemv_fault_count(1) == 0
+    # K = 11008 (LLaMA-2-7B's down projection) x 4096: three slices by length become four, K = 28672 x 1024: seven become eight
+    assert lib.elutq_hlq_gemv_slices(11008, 4096, 2, 128, _lib.GEMV_WIDE, 0) == 4
+    assert lib.elutq_hlq_gemv_slices(28672, 1024, 2, 128, _lib.GEMV_WIDE, 0) == 8
+
+
 def test_k_sliced_launches_in_a_replayed_graph(cuda):
     """Three K-sliced GEMVs of different shapes share one workspace inside one HIP graph (the slots of one launch are
     the slots of the next): every replay, with eager work of the same kind in between, gives the eager result."""

@@ -90,6 +90,12 @@ def test_size_queries_and_argument_errors():
     assert wide == -7                                                   # a consumer has one tile per compute unit at most
     assert fused(_lib.GemvFusion(0, 0.0, None, one, one, None, 0, None), 4) == -7    # the consumer adds the residual
     assert fused(_lib.GemvFusion(0, 0.0, None, None, one, None, 0, None), 1) == -7   # one slice: nothing to hand over
+    # the buffers of handed-over slices come with their sizes: a producer's S x N floats, a consumer's n_slices_in x K
+    GF = _lib.GemvFusion
+    assert fused(GF(1, 1e-5, one, None, None, one, 2, None, 0, 2 * 4096 * 4 - 1)) == -5
+    assert fused(GF(1, 1e-5, one, None, None, one, 2, None, 0, 0)) == -5
+    assert fused(GF(0, 0.0, None, None, one, None, 0, None, 4 * 64 * 4 - 1, 0), 4) == -5
+    assert fused(GF(0, 0.0, None, None, one, None, 0, None, 0, 0), 2) == -5
     # the query a caller decides with before it lets a producer leave its slices unsummed: the launch's own limits
     acc = L.elutq_hlq_gemv_accepts_slices
     assert acc(4096, 6144, 2, 128, 2, 16, 4) == 1                       # LLaMA-3-8B q|k|v in two K slices: 192 tiles

@@ -32,7 +32,10 @@ def test_static_gemv_equals_the_workspace_entry_point_on_two_calls_in_a_row(cuda
     assert L.elutq_hlq_static_scratch_bytes() == (64 << 10) + (2 << 20)
     # first a K-sliced launch (14336 x 4096: four slices meet in the array), then a smaller one (4096 x 1024,
     # also sliced), then one without slices; every one against the entry point that takes a workspace
-    shapes = [(14336, 4096, 2, 128, False), (4096, 1024, 3, 64, True), (1024, 200, 2, 128, True), (4096, 6144, 2, 128, False)]
+    # ... and 14336 x 8192, whose four slices of 128 column blocks do not fit the slots of the array's head: arrival
+    # counters at its start (cleared by the call's fill kernel), partial sums behind the first 64 KiB
+    shapes = [(14336, 4096, 2, 128, False), (4096, 1024, 3, 64, True), (1024, 200, 2, 128, True), (4096, 6144, 2, 128, False),
+              (14336, 8192, 2, 128, False)]
     for rep in range(2):
         for k, n, bits, group, bias in shapes:
             print(f"static gemv K={k} N={n} w{bits}g{group} pass {rep}", flush=True)
@@ -74,6 +77,18 @@ def test_static_gemv_in_a_graph_and_its_limits(cuda):
         torch.cuda.synchronize()
         assert torch.equal(y, want)
         _ = mod(x)                       # eager work with a workspace of its own between the replays
+    # the matrix-core engine chooses its own K slices (whole unit pairs): the call sizes its check from the launch it makes
+    _lib.set_gemv_engine("mfma")
+    try:
+        for k, n in ((14336, 4096), (4096, 1024), (6144, 256)):
+            lay2 = make_layer(k, n, bits=2, group=128, seed=k + n)
+            mod2 = HLQLinear.from_export_arrays(lay2.w_quant, lay2.w_scale, lay2.w_zero, 128, None, cuda)
+            x2 = torch.from_numpy(lay2.x).to(cuda)
+            want2 = mod2(x2)
+            for _ in range(2):
+                assert torch.equal(static_gemv(mod2, x2), want2), (k, n)
+    finally:
+        _lib.set_gemv_engine("auto")
     # argument errors are those of the workspace entry point; a shape beyond the array's size is refused
     one = ctypes.c_void_p(1)
     assert L.elutq_hlq_gemv_f16_static(None, one, one, None, one, one, 4096, 64, 2, 128, None) == -1
