@@ -92,7 +92,7 @@ def quantize_groups(w: torch.Tensor, bits: int, group: int, iters: int = 10):
 
 @torch.no_grad()
 def gptq_hlq(weight: torch.Tensor, hessian: torch.Tensor, bits: int, group: int, percdamp: float = 0.01,
-             actorder: bool = False, iters: int = 10):
+             actorder: bool = False, iters: int = 10, quantizer=None):
     """GPTQ error compensation around the group-wise HLQ fit for one linear layer.
 
     weight [N, K]; hessian [K, K] = 2/n * sum x x^T over the calibration inputs (HLQ.add_batch,
@@ -101,7 +101,9 @@ def gptq_hlq(weight: torch.Tensor, hessian: torch.Tensor, bits: int, group: int,
     factor of H^-1, are propagated to the later columns of the group and then to all later
     groups.  Returns (w_q fp32 [N, K], codes uint8 [N, K, bits], scales fp32 [N, K/group, bits],
     zeros fp32 [N, K/group, 1]); with actorder the codes / scales / zeros refer to the permuted
-    column order, as in the reference."""
+    column order, as in the reference.  `quantizer(w1, bits, group_size, iters)` stands in for
+    quantize_groups (same arguments and results) where a test wants the loop alone."""
+    quantizer = quantizer or quantize_groups
     w = weight.detach().clone().float()
     h = hessian.detach().clone().float()
     n, k = w.shape
@@ -122,7 +124,7 @@ def gptq_hlq(weight: torch.Tensor, hessian: torch.Tensor, bits: int, group: int,
     for c0 in range(0, k, group):
         c1 = min(c0 + group, k)
         w1 = w[:, c0:c1].clone()
-        q1, cd, sc, zp = quantize_groups(w1, bits, c1 - c0, iters)
+        q1, cd, sc, zp = quantizer(w1, bits, c1 - c0, iters)
         codes.append(cd); scales.append(sc); zeros.append(zp)
         u1 = u[c0:c1, c0:c1]
         err = torch.zeros_like(w1)

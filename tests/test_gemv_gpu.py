@@ -173,6 +173,39 @@ def test_llama3_8b_shapes_full_size(cuda, name, bits, group, ksplit):
     assert np.array_equal(yn.view(np.uint16) ^ 0x8000, y.view(np.uint16)) or np.array_equal(-yn, y)
 
 
+@pytest.mark.parametrize("name", ["q_proj", "k_proj", "gate_proj", "down_proj"])
+@pytest.mark.parametrize("bits,group", [(2, 128), (3, 128), (2, 64)])
+def test_llama3_8b_shapes_against_the_reference_fp16_chain(cuda, lutref, name, bits, group):
+    """The GPU GEMV beside the reference's own CPU arithmetic at the benchmark's shapes: the C restatement of
+    MultiThreadGemvW_lowbit_Activation_FP::Run (C++/ops/src/arm/arm_gemm.cpp:248-308) and t_mac_g4_float_update_impl
+    (arm_t_mac_kernal.cpp:364-469), every operation rounded to fp16 as the NEON kernel rounds it, four threads as in
+    C++/examples/main.cpp:41.  That chain adds 32 (K = 4096) to 112 (K = 14336) group sums one after the other in
+    fp16, and its distance from the exact result grows with K -- measured on these inputs (max over the outputs, in
+    units of rms(y)): 0.9-1.4e-2 at K = 4096, 1.9-2.9e-2 at K = 14336; rms error 2.2-4.0e-3 and 5.4-6.9e-3.  The GPU
+    result (fp32 accumulation, one rounding) sits about 5e-4 from exact, so its distance from the chain is the
+    chain's own error.  Bars: max |gpu - chain| <= 2e-2 rms at K = 4096 and 4e-2 rms at K = 14336 (1.4 x the largest
+    measured chain error), rms |gpu - chain| <= 6e-3 / 1e-2 rms, and the GPU result at least five times closer to
+    exact than the chain is."""
+    k, n = LLAMA3_8B_SHAPES[name]
+    L = make_layer(k, n, bits=bits, group=group, seed=7)
+    y = run(to_mod(L, cuda), L.x, cuda)[0].astype(np.float64)
+    w = O.dequantize(L.w_quant, L.w_scale, L.w_zero, group, np.float32)
+    ref = w.astype(np.float64) @ L.x[0].astype(np.float64)
+    rms = np.sqrt(np.mean(ref ** 2))
+    chain = lutref.RefWeight(L.w_quant, L.w_scale, L.w_zero, group, 4).gemv(L.x[0]).astype(np.float64)
+    d_chain_exact = np.max(np.abs(chain - ref)) / rms
+    d_gpu_chain = np.max(np.abs(y - chain)) / rms
+    d_gpu_exact = np.max(np.abs(y - ref)) / rms
+    r_gpu_chain = np.sqrt(np.mean((y - chain) ** 2)) / rms
+    msg = (f"{name} {k}x{n} w{bits}g{group}: chain-exact {d_chain_exact:.3e}, gpu-chain {d_gpu_chain:.3e} (rms {r_gpu_chain:.3e}), "
+           f"gpu-exact {d_gpu_exact:.3e} [max over outputs / rms(y)]")
+    print(msg, flush=True)
+    big = k > 4096
+    assert d_gpu_chain <= (4e-2 if big else 2e-2), msg
+    assert r_gpu_chain <= (1e-2 if big else 6e-3), msg
+    assert d_gpu_exact <= 0.2 * d_chain_exact, msg
+
+
 @pytest.mark.parametrize("n", [28672, 128256])
 def test_widest_layers_sampled_columns(cuda, n):
     """The widest layers of the decode step -- gate|up concatenated (4096 x 28672) and an lm_head-sized layer

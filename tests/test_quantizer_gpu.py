@@ -75,3 +75,19 @@ def test_quantize_export_load_run(cuda, tmp_path, bits, group):
     y = mod(xv).float()
     ref = xv.float() @ deq.t()
     assert (y - ref).abs().max() <= 1e-2 * ref.pow(2).mean().sqrt()
+
+
+@pytest.mark.parametrize("k,group,bits,actorder", [(32, 8, 2, False), (32, 16, 3, True), (24, 8, 2, True), (32, 32, 2, False)])
+def test_gptq_loop_against_textbook_obq_on_the_device(cuda, k, group, bits, actorder):
+    """gptq_hlq on device tensors against the textbook restatement of the error-feedback loop (tests/obq_reference.py:
+    explicit float64 inverse Hessian, one column eliminated at a time), the same simple group quantizer injected into
+    both; the reference's loop is GPTQ/HLQ.py:108-153."""
+    import numpy as np
+    from obq_reference import correlated_problem, obq_reference, uniform_group_quantizer
+    for seed in range(3):
+        w, h = correlated_problem(100 * k + seed, 12, k)
+        want = obq_reference(w, h, bits, group, actorder=actorder)
+        got = HQ.gptq_hlq(torch.from_numpy(w).float().to(cuda), torch.from_numpy(h).float().to(cuda), bits, group,
+                          actorder=actorder, quantizer=uniform_group_quantizer)[0]
+        assert got.is_cuda
+        np.testing.assert_allclose(got.double().cpu().numpy(), want, atol=1e-5, rtol=0)
