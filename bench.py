@@ -32,7 +32,32 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-KERNEL_TRACE_AVG_US = 6.41     # hlq_gemv_kernel<2, false, 4, true, 1> at 4096 x 14336 in the committed kernel trace
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hlq_gemv_w2g128_4096x14336_hbm_traffic.md")
+TRACE_PROFILE = os.path.join(ROOT, "profiles", "hlq_gemv_w2g128_sweep_kernel_trace.md")
+KERNEL_SOURCES = ["hlq_gemv.hip", "hlq_gemv_dev.h", "hlq_gemv_index.h", "hlq_layout.h"]     # what the dominant kernel is compiled from
+
+
+def kernel_source_hash():
+    """First 16 hex digits of the SHA-256 of the dominant kernel's sources: the committed counter summaries carry the
+    hash of the sources they were measured on, so a figure taken from them can be told from a stale one."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "elutq_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def profile_figure(path, key):
+    """`key: value` and `kernel source hash: ...` lines of a committed profile summary -> (value or None, hash matches)."""
+    import re
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, False
+    m = re.search(r"^" + re.escape(key) + r":\s*([0-9.]+)", text, re.M)
+    h = re.search(r"^kernel source hash:\s*([0-9a-f]+)", text, re.M)
+    return (float(m.group(1)) if m else None), bool(h and h.group(1) == kernel_source_hash())
 BITS, GROUP = 2, 128
 N_LAYERS = 32
 
@@ -50,13 +75,12 @@ def parse():
     p.add_argument("--sweep-only", action="store_true",
                    help="only the sweep and the per-shape rings of the per-GEMV entry point (no grouped / multi-stream / "
                         "copy / other-format / large-shape legs): the run a kernel trace of the dominant kernel is taken from")
-    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "decode-eager", "gemm", "group", "sparse", "shape-sweep", "lds-rate"],
+    p.add_argument("--mode", choices=["full", "kernel", "copy", "decode", "decode-eager", "gemm", "group", "sparse"],
                    default="full",
                    help="kernel: only the dominant GEMV (4096x14336) over its weight ring, for counter runs; "
                         "copy: a plain 64 MiB device copy, the calibration kernel for FETCH_SIZE / WRITE_SIZE; "
                         "decode / gemm: only that leg (for kernel traces); "
                         "decode-eager: three eager decode steps of a two-layer model of the same widths (for counter runs); "
-                        "shape-sweep: the small LLaMA-3-8B shapes at every kernel, K split and wave count of the tuned entry point; "
                         "sparse: GEMVs of layers with a block-sparse extra plane beside the same layers without it")
     p.add_argument("--launches", type=int, default=256, help="launches in --mode kernel / copy")
     return p.parse_args()
@@ -77,9 +101,12 @@ class Gemv:
             raise RuntimeError(f"elutq_hlq_gemv_f16 failed: {rc}")
 
 
-def time_graph(torch, launch_all, replays, warmup):
+def time_graph(torch, launch_all, replays, warmup, sustain_s=0.0, cold=None):
     """Captures launch_all(stream) once, replays it; returns seconds per replay (HIP events on
-    the replay stream)."""
+    the replay stream).  sustain_s > 0: after the `warmup` replays the graph is replayed untimed for that long, and
+    the timed region is at least as long again, so that a leg whose rate follows the GPU's clocks is measured in the
+    state a long run reaches (the clocks follow the load with a delay of tens of milliseconds) whatever `replays` is;
+    the figure of the first `replays` replays after `warmup`, taken before that, goes into cold["s"]."""
     s = torch.cuda.Stream()
     with torch.cuda.stream(s):
         launch_all(s.cuda_stream)            # eager warm-up on the capture stream
@@ -90,13 +117,24 @@ def time_graph(torch, launch_all, replays, warmup):
     for _ in range(warmup):
         g.replay()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(replays):
-        g.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / replays
+
+    def timed(n):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / n
+
+    sec = timed(replays)
+    if sustain_s <= 0:
+        return sec
+    if cold is not None:
+        cold["s"] = sec
+    n = max(replays, int(sustain_s / max(sec, 1e-7)) + 1)
+    timed(n)                                 # untimed as far as the result goes
+    return timed(n)
 
 
 def cpu_baseline(budget_s):
@@ -190,35 +228,6 @@ def gemm_leg(torch, lib, dev, steps):
     return out
 
 
-def lds_rate_leg(torch, lib, dev, passes=4000):
-    """Rate at which one compute unit retires wavefront-wide 16-entry table lookups: bare ds_read_b32 instructions, and
-    the LUT GEMV's own sub-task sequence on plane words held in registers (tables already in LDS, nothing loaded from
-    memory).  A lookup covers 4 k of one column and one plane, i.e. 4 weight bits per lane; the rates are restated as
-    the HBM stream a w2g128 GEMV would sustain at them (planes are 2048 of the 2432 bytes of a unit)."""
-    out = torch.zeros(256 * 2048, dtype=torch.int32, device=dev)
-    stream = torch.cuda.current_stream().cuda_stream
-    res = {}
-    for sequence, name in ((0, "bare_ds_read_b32"), (1, "gemv_subtask_sequence")):
-        res[name] = {}
-        for waves in (4, 8, 16, 32):
-            best = None
-            for _ in range(4):
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                rc = lib.elutq_diag_lds_lookup_rate(sequence, waves, passes, out.data_ptr(), stream)
-                e1.record()
-                if rc:
-                    raise RuntimeError(f"elutq_diag_lds_lookup_rate failed: {rc}")
-                torch.cuda.synchronize()
-                ms = e0.elapsed_time(e1)
-                best = ms if best is None else min(best, ms)
-            ns = best * 1e6 / (passes * 16 * waves)
-            plane_tbps = 256 * 64 * 4 / 8 / ns / 1e3
-            res[name][f"{waves}_waves_per_cu"] = {"ns_per_wave_lookup_per_cu": ns, "cycles_at_2p4_GHz": ns * 2.4,
-                                                  "w2g128_algorithmic_TBps_at_that_rate": plane_tbps * 2432 / 2048}
-    return res
-
-
 def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
     """Batch-1 GEMV of w2g128 layers that carry a block-sparse extra plane on `density` of their
     (32 channels x 128 inputs) blocks, held as blocks -- two launches: the plane's fp32 term, then the
@@ -309,7 +318,7 @@ def sparse_decode_leg(torch, dev, density, n_ctx=512, n_gen=50):
             lin[name] = with_device_sparse_plane(lin[name], density, seed)
             nblk += lin[name].sparse_count
             seed += 1
-    model = LlamaDecoder(s, device=dev, seed=0, impl="hip", parts=parts)
+    model = LlamaDecoder(s, device=dev, seed=0, parts=parts)
     model.fill_cache(n_ctx)
     model.token.fill_(1)
     model.capture()
@@ -358,27 +367,45 @@ def counter_mode(a, torch, lib, dev):
                       "ring_sets": len(ring)}))
 
 
+SUSTAIN_S = 0.08       # untimed lead of the legs whose rate follows the GPU's clocks (and the least length of their timed region)
+
+
 def side_legs(a, torch, lib, dev, calls, xs, ws_bytes, step_bytes):
-    """The same 224 GEMVs through the grouped entry point (one launch, one launch per layer), the per-GEMV launches
-    dealt onto four streams of one graph, and a plain device copy as a yardstick."""
+    """The same 224 GEMVs through the grouped entry point (one launch on the engine the library picks -- the streaming
+    matrix-core kernel -- and on the LUT engine; one launch per layer), the per-GEMV launches dealt onto four streams
+    of one graph, and a plain device copy as a yardstick."""
+    from elutq_amd import _lib
     from elutq_amd.hlq_linear import GemvGroup
     from elutq_amd.synth import LLAMA3_8B_SHAPES
     g_mods = [c.mod for c in calls]
     g_xs = [xs[m.in_features] for m in g_mods]
     g_ys = [torch.empty(1, m.out_features, dtype=torch.float16, device=dev) for m in g_mods]
     grouped = {}
-    for label, per in (("one_launch", len(g_mods)), ("launch_per_layer", len(LLAMA3_8B_SHAPES))):
+    engine_before = lib.elutq_hlq_get_gemv_engine()
+    for label, per, engine in (("one_launch", len(g_mods), None), ("one_launch_lut_engine", len(g_mods), "lut"),
+                               ("launch_per_layer", len(LLAMA3_8B_SHAPES), None)):
+        if engine:
+            _lib.set_gemv_engine(engine)
         groups = [GemvGroup(g_mods[i:i + per], g_xs[i:i + per], g_ys[i:i + per]) for i in range(0, len(g_mods), per)]
+        lib.elutq_hlq_set_gemv_engine(engine_before)
 
         def launch_groups(stream, groups=groups):
             for g in groups:
                 g.run()
 
-        sec = time_graph(torch, launch_groups, a.steps, a.warmup)
+        cold = {}
+        sec = time_graph(torch, launch_groups, a.steps, a.warmup, SUSTAIN_S, cold)
         grouped[label] = {"launches": len(groups), "ms_per_step": sec * 1e3, "GBps": step_bytes / sec / 1e9,
-                          "frac_hbm_peak": step_bytes / sec / 1e9 / HBM_PEAK_GBPS}
+                          "frac_hbm_peak": step_bytes / sec / 1e9 / HBM_PEAK_GBPS,
+                          # the first `steps` replays after `warmup`, before the clocks have followed the load
+                          "cold_GBps": step_bytes / cold["s"] / 1e9, "sustained_lead_s": SUSTAIN_S}
         for g in groups:
             g.close()
+    grouped["one_launch"]["kernel"] = ("hlq_gemv_mfma_group_kernel<2,false>: fp4 x fp4 MFMA on the plane bits, 256 workgroups, "
+                                       "each streaming one contiguous share of the 2.08 GB")
+    grouped["one_launch"]["roofline"] = {"bound": "hbm", "achieved": grouped["one_launch"]["GBps"], "peak": HBM_PEAK_GBPS,
+                                         "unit": "GB/s", "frac": grouped["one_launch"]["frac_hbm_peak"],
+                                         "bytes_per_launch": step_bytes}
     # ---- the same 224 launches of the per-GEMV entry point, dealt round-robin onto four HIP streams
     # inside one graph (a workspace per stream): independent GEMVs overlap each other's start-up and tail
     n_streams = 4
@@ -443,7 +470,7 @@ def main():
         from elutq_amd.hlq_linear import HLQLinear
         from elutq_amd.llama_decode import LlamaDecoder, LlamaShape
         shape = LlamaShape(n_layers=2)
-        model = LlamaDecoder(shape, device=dev, seed=0, impl="hip")
+        model = LlamaDecoder(shape, device=dev, seed=0)
         model.fill_cache(512)
         model.token.fill_(1)
         steps = 3
@@ -455,49 +482,6 @@ def main():
         print(json.dumps({"mode": "decode-eager", "layers": shape.n_layers, "steps": steps,
                           "algorithmic_bytes_per_step": {"hlq_layers": hlq_bytes, "fp16_lm_head": model.lm_head.numel() * 2,
                                                          "kv_cache_read": kv_bytes, "embedding_row": shape.hidden * 2}}))
-        return
-    if a.mode == "shape-sweep":
-        # what a launch of the two small shapes costs however its work is arranged: every K split x wave count of the
-        # tuned entry point (and both kernels), each over a ring of distinct weight sets, one graph replay per ring
-        from elutq_amd.synth import make_device_layer as mk
-        table = {}
-        for (k, n) in ((4096, 1024), (4096, 4096)):
-            nbytes = algorithmic_bytes(k, n, BITS, GROUP)
-            ring = [mk(k, n, BITS, GROUP, seed=i, device=dev) for i in range(max(8, -(-400 * 2 ** 20 // nbytes)))]
-            x = torch.randn(1, k, device=dev).to(torch.float16)
-            y = torch.empty(1, n, dtype=torch.float16, device=dev)
-            ws = torch.zeros(max(lib.elutq_hlq_workspace_bytes(k, n, BITS, GROUP, 1), 1 << 22), dtype=torch.uint8, device=dev)
-            rows = []
-            named = {_lib.GEMV_NARROW16: "narrow tiles, 16 columns", _lib.GEMV_NARROW32: "narrow tiles, 32 columns",
-                     _lib.GEMV_WIDE: "wide tiles, the library's K split"}
-            for eng in ("lut", "mfma"):
-                _lib.set_gemv_engine(eng)
-                for ks in (0, _lib.GEMV_NARROW16, _lib.GEMV_NARROW32, _lib.GEMV_WIDE, 1, 2, 4, 8, 16):
-                    for wv in (0, 4, 8, 16):
-                        if ks < 0 and (wv or (eng == "mfma" and ks != _lib.GEMV_WIDE)):
-                            continue
-                        slices = lib.elutq_hlq_gemv_slices(k, n, BITS, GROUP, ks, wv)
-                        if slices == 0:
-                            continue
-
-                        def launch(stream, ks=ks, wv=wv):
-                            for m in ring:
-                                rc = lib.elutq_hlq_gemv_f16_tuned(m.planes.data_ptr(), m.scales.data_ptr(), m.zeros.data_ptr(), None,
-                                                                  x.data_ptr(), y.data_ptr(), k, n, BITS, GROUP, ws.data_ptr(),
-                                                                  ws.numel(), stream, ks, wv)
-                                if rc:
-                                    raise RuntimeError(f"elutq_hlq_gemv_f16_tuned: {rc}")
-
-                        us = time_graph(torch, launch, 10, 2) / len(ring) * 1e6
-                        ncb = (n + 63) // 64
-                        wgs = ncb * 4 if ks == _lib.GEMV_NARROW16 else ncb * 2 if ks == _lib.GEMV_NARROW32 else slices * ncb
-                        rows.append({"engine": eng, "ksplit": named.get(ks, ks), "waves": wv, "slices": slices,
-                                     "workgroups": wgs, "us": round(us, 3)})
-            _lib.set_gemv_engine("auto")
-            table[f"{k}x{n}"] = {"bytes": nbytes, "byte_floor_us_at_8TBps": nbytes / 8e6, "rows": rows}
-            del ring
-            torch.cuda.empty_cache()
-        print(json.dumps({"mode": "shape-sweep", "shapes": table}))
         return
     if a.mode == "gemm":
         print(json.dumps({"mode": "gemm", "gemm_w2g128_llama2_13b": gemm_leg(torch, lib, dev, a.steps)}))
@@ -513,13 +497,12 @@ def main():
         xk = {k: torch.randn(1, k, device=dev).to(torch.float16) for k in {m.in_features for m in mods}}
         grp = GemvGroup(mods, [xk[m.in_features] for m in mods],
                         [torch.empty(1, m.out_features, dtype=torch.float16, device=dev) for m in mods])
-        sec = time_graph(torch, lambda s: grp.run(), a.steps, a.warmup)
+        cold = {}
+        sec = time_graph(torch, lambda s: grp.run(), a.steps, a.warmup, SUSTAIN_S, cold)
         print(json.dumps({"mode": "group", "gemvs_per_launch": len(mods), "bytes_per_launch": nbytes, "us_per_launch": sec * 1e6,
-                          "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS}))
+                          "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
+                          "cold_GBps": nbytes / cold["s"] / 1e9, "engine": lib.elutq_hlq_get_gemv_engine()}))
         grp.close()
-        return
-    if a.mode == "lds-rate":
-        print(json.dumps({"mode": "lds-rate", "lds_lookup_rate": lds_rate_leg(torch, lib, dev)}))
         return
     if a.mode == "sparse":
         print(json.dumps({"mode": "sparse", "sparse_gemv_w2g128": sparse_leg(torch, lib, dev, a.steps, a.warmup)}))
@@ -626,10 +609,31 @@ def main():
             for c in ring:
                 c(stream)
 
-        sec = time_graph(torch, launch_big, max(3, min(a.steps, 2000)), 5) / len(ring)
+        cold = {}
+        sec = time_graph(torch, launch_big, max(3, min(a.steps, 2000)), 5, SUSTAIN_S, cold) / len(ring)
         large_shape = {f"{k}x{n}": {"us": sec * 1e6, "GBps": nbytes / sec / 1e9, "frac_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBPS,
-                                    "bytes": nbytes, "ring_sets": len(ring)}}
-        del ring
+                                    "bytes": nbytes, "ring_sets": len(ring), "cold_us": cold["s"] / len(ring) * 1e6}}
+        # ---- a wide layer with K > 4096 (a 14336 x 32768 projection, 143 MB): here the library's choice is the streaming
+        # matrix-core kernel (no K slices), beside the LUT kernel's runs of column blocks with K slices
+        from elutq_amd import _lib as _l
+        k2, n2 = 14336, 32768
+        nbytes2 = algorithmic_bytes(k2, n2, BITS, GROUP)
+        ws2 = torch.zeros(lib.elutq_hlq_workspace_bytes(k2, n2, BITS, GROUP, 1), dtype=torch.uint8, device=dev)
+        ring2 = [Gemv(lib, make_device_layer(k2, n2, BITS, GROUP, seed=31_000 + i, device=dev), xs[k2],
+                      torch.empty(1, n2, dtype=torch.float16, device=dev), ws2) for i in range(4)]
+
+        def launch_big2(stream):
+            for c in ring2:
+                c(stream)
+
+        sec = time_graph(torch, launch_big2, max(3, min(a.steps, 2000)), 5, SUSTAIN_S) / len(ring2)
+        engine_before = lib.elutq_hlq_get_gemv_engine()
+        _l.set_gemv_engine("lut")
+        sec_lut = time_graph(torch, launch_big2, max(3, min(a.steps, 2000)), 5, SUSTAIN_S) / len(ring2)
+        lib.elutq_hlq_set_gemv_engine(engine_before)
+        large_shape[f"{k2}x{n2}"] = {"us": sec * 1e6, "GBps": nbytes2 / sec / 1e9, "frac_hbm_peak": nbytes2 / sec / 1e9 / HBM_PEAK_GBPS,
+                                     "bytes": nbytes2, "ring_sets": len(ring2), "lut_engine_us": sec_lut * 1e6}
+        del ring2, ws2
         torch.cuda.empty_cache()
         # ---- the same lm_head unquantized: the dense fp16 GEMV of the decode step (two weight sets of 1.05 GB),
         # beside the hipBLASLt call it replaced
@@ -655,22 +659,26 @@ def main():
         torch.cuda.empty_cache()
 
     dom = per_shape["4096x14336"]
+    # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --mode kernel`,
+    # each scaled by what the same counter reads for `--mode copy`: read from the committed summary, a property of the
+    # kernel's access pattern, not of this run -- and null when the kernel's sources are no longer the ones measured
+    traffic, traffic_fresh = profile_figure(TRAFFIC_PROFILE, "traffic bytes per launch")
+    trace_us, trace_fresh = profile_figure(TRACE_PROFILE, "average duration us")
     roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": dom["GBps"] / HBM_PEAK_GBPS,
-                # HBM bytes per launch of this kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-                # `bench.py --mode kernel`, each scaled by what the same counter reads for `--mode copy`
-                # (summary under profiles/); a property of the kernel's access pattern, not of this run.
-                "traffic": 17_644_000,
-                "traffic_source": "constant from profiles/hlq_gemv_w2g128_4096x14336_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE and "
-                                  "WRITE_SIZE of `bench.py --mode kernel`, scaled by the same counters of `--mode copy`), not measured in this run",
+                "traffic": int(traffic) if traffic and traffic_fresh else None,
+                "traffic_source": "profiles/hlq_gemv_w2g128_4096x14336_hbm_traffic.md (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of "
+                                  "`bench.py --mode kernel`, scaled by the same counters of `--mode copy`), not measured in this run"
+                                  + ("" if traffic_fresh else "; the kernel's sources have changed since that measurement, so no figure is quoted"),
                 "kernel": "hlq_gemv_kernel<2,false> K=4096 N=14336", "us_per_launch": dom["us"],
-                "bytes_per_launch": dom["bytes"],
-                # the same kernel's average start-to-end duration in the rocprofv3 kernel trace of `bench.py --sweep-only`
-                # (profiles/hlq_gemv_w2g128_sweep_kernel_trace.md) and the fraction that follows from it: a replayed launch
-                # starts while its predecessor's completion is still being signalled, so the live per-launch period above
-                # is shorter than the traced duration
-                "kernel_trace_avg_us": KERNEL_TRACE_AVG_US,
-                "frac_kernel_trace": dom["bytes"] / (KERNEL_TRACE_AVG_US * 1e-6) / 1e9 / HBM_PEAK_GBPS}
+                "bytes_per_launch": dom["bytes"], "kernel_source_hash": kernel_source_hash()}
+    if trace_us and trace_fresh:
+        # the same kernel's average start-to-end duration in the rocprofv3 kernel trace of `bench.py --sweep-only`
+        # (profiles/hlq_gemv_w2g128_sweep_kernel_trace.md) and the fraction that follows from it: a replayed launch
+        # starts while its predecessor's completion is still being signalled, so the live per-launch period above
+        # is shorter than the traced duration
+        roofline["kernel_trace_avg_us"] = trace_us
+        roofline["frac_kernel_trace"] = dom["bytes"] / (trace_us * 1e-6) / 1e9 / HBM_PEAK_GBPS
     if grouped.get("device_copy_1GiB_GBps"):
         roofline["frac_of_device_copy_rate"] = dom["GBps"] / grouped["device_copy_1GiB_GBps"]
 

@@ -26,7 +26,6 @@ SIGNATURES = {
     "elutq_hlq_workspace_init": (_ci, [_vp, _sz, _vp]),
     "elutq_hlq_gemv_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp]),
     "elutq_hlq_gemv_f16_tuned": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _ci, _ci]),
-    "elutq_diag_lds_lookup_rate": (_ci, [_ci, _ci, _ci, _vp, _vp]),
     "elutq_hlq_gemv_int8lut_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp]),
     "elutq_hlq_gemv_fused_f16": (_ci, [_vp] * 6 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
     "elutq_hlq_gemv_slices": (_ci, [_ci] * 6),

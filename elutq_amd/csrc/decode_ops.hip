@@ -83,17 +83,6 @@ __device__ __forceinline__ float wave_sum(float v)
     return v;
 }
 
-#ifdef HLQ_TIMING
-// Profiling builds only: wall-clock stamps (100 MHz) of thread 0 of every workgroup.
-__device__ unsigned long long *g_attn_stamps = nullptr;
-#define ATTN_STAMP(i)                                                                                  \
-    do {                                                                                               \
-        if (g_attn_stamps && threadIdx.x == 0 && (i) < 16) g_attn_stamps[(size_t)blockIdx.x * 16 + (i)] = wall_clock64(); \
-    } while (0)
-#else
-#define ATTN_STAMP(i) do { } while (0)
-#endif
-
 constexpr int ATTN_WAVES = 4;
 constexpr int ATTN_UNROLL = 4;
 
@@ -252,7 +241,6 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     // the first block of cache rows (row numbers clamped by the cache size, not by the position,
     // so the addresses do not depend on *pos; rows at or beyond it are masked later), q and the
     // new k / v, and the position itself.  One memory round trip instead of three dependent ones.
-    ATTN_STAMP(0);
     const long long pos64 = *a.pos;
     uint4 kk[BATCH], vv[BATCH];
 #pragma unroll
@@ -284,7 +272,6 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     const int nblocks = (pos + BLOCK_ROWS - 1) / BLOCK_ROWS;
     const int S = nblocks <= SHORT_BLOCKS ? 1 : min(SL, nblocks <= 12 ? min(nblocks, 4) : ATTN_MAX_SPLITS);
     if (sp >= S) return;
-    ATTN_STAMP(1);
 
     if (tid < HALF) {                                    // rotary pair (tid, tid + 64) of q and of the new k
         const int j = tid;
@@ -303,11 +290,8 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
         ((uint4 *)(a.vc + row))[tid] = ((const uint4 *)sv)[tid];
     }
 
-    ATTN_STAMP(2);
     const uint4 qv = ((const uint4 *)sq)[seg];
     const float scale = rsqrtf((float)D);
-    int stamp_i = 3;
-    (void)stamp_i;
     float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.f;
@@ -359,7 +343,6 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
         }
 #pragma unroll
         for (int b = 0; b < BATCH; b++) { kk[b] = kn[b]; vv[b] = vn[b]; }
-        ATTN_STAMP(stamp_i); stamp_i++;
     }
     if (wave == 0 && sp == 0) {                          // the token being decoded, from LDS (row 0 only)
         const float s = dot8(qv, ((const uint4 *)sk)[seg]) * scale;
@@ -381,9 +364,7 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
 #pragma unroll
         for (int i = 0; i < 8; i++) sm_o[wave][seg * 8 + i] = acc[i];
     }
-    ATTN_STAMP(12);
     __syncthreads();
-    ATTN_STAMP(13);
     float M = -INFINITY, L = 0.f, o = 0.f;               // this split's result for dimension tid
     if (tid < D) {
 #pragma unroll
@@ -397,7 +378,6 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
     }
     if (S == 1) {
         if (tid < D) a.out[(size_t)h * D + tid] = f2h(o / L);
-        ATTN_STAMP(14);
         return;
     }
     float *po = a.partial + ((size_t)h * SL + sp) * (D + 2);
@@ -436,7 +416,6 @@ __global__ __launch_bounds__(WAVES * 64) void rope_attn_d128_kernel(const AttnAr
         a.out[(size_t)h * D + tid] = f2h(oo / LL);
     }
     if (tid == 0) __hip_atomic_store(&a.counters[h], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    ATTN_STAMP(14);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -592,13 +571,6 @@ extern "C" size_t elutq_decode_attn_workspace_bytes(int n_heads, int head_dim, i
     const int s = splits == 0 ? ATTN_MAX_SPLITS : splits;
     return (size_t)HLQ_WS_COUNTER_BYTES + (size_t)n_heads * s * (head_dim + 2) * sizeof(float);
 }
-
-#ifdef HLQ_TIMING
-extern "C" int elutq_debug_set_attn_stamps(void *d_buf)
-{
-    return hipMemcpyToSymbol(HIP_SYMBOL(g_attn_stamps), &d_buf, sizeof(d_buf)) == hipSuccess ? 0 : -1;
-}
-#endif
 
 // d_qkv_slices non-null: q|k|v arrives as n_qkv_slices unsummed K slices (fp32 rows of qkv_stride floats)
 static int launch_rope_attn(const void *d_qkv, const void *d_qkv_slices, int n_qkv_slices, int qkv_stride,

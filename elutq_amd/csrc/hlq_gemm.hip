@@ -54,20 +54,6 @@ struct GemmArgs {
     int mpad;               // rows of `partial`: 32 or 64
 };
 
-#ifdef HLQ_TIMING
-// Profiling builds only: wall-clock stamps (100 MHz) of thread 0 of every workgroup.
-__device__ unsigned long long *g_gemm_stamps = nullptr;
-#define GEMM_STAMP(i)                                                                                  \
-    do {                                                                                               \
-        if (g_gemm_stamps && threadIdx.x == 0 && (i) < 16) {                                           \
-            g_gemm_stamps[(size_t)blockIdx.x * 16 + (i)] = wall_clock64();                             \
-            g_gemm_stamps[(size_t)(2048 + blockIdx.x) * 16 + (i)] = clock64();                         \
-        }                                                                                              \
-    } while (0)
-#else
-#define GEMM_STAMP(i) do { } while (0)
-#endif
-
 template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v)
 {
@@ -293,7 +279,6 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[mt][j][i] = 0.f;
 
-    GEMM_STAMP(0);
     // The plane data of two of the wave's units is in registers at any time (two alternating sets, so no
     // set is ever copied); the activations of the next unit wait in registers while the wave computes on
     // the staged ones.
@@ -317,7 +302,6 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
         *(uint4 *)(smem + e * 16) = row;
     }
     __syncthreads();
-    GEMM_STAMP(1);
     const uint32_t lanepart = (uint32_t)(lane % TREP) * 16u;
     unsigned char *xw = smem + L::TAB_BYTES + wave * L::WAVE_BYTES;
     float *xs = (float *)(xw + MR * ROW_BYTES);
@@ -563,7 +547,6 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
         if (u + NW < u_end) unit(ub, u + NW);
     }
 
-    GEMM_STAMP(13);
     // Sum of the K parts through LDS: red[wave][tile = mt*2+j][reg][lane].
     __syncthreads();
     if constexpr (T16) {
@@ -619,7 +602,6 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
                 a.y[(size_t)m * a.N + n] = __builtin_bit_cast(uint16_t, (_Float16)s);
             }
         }
-        GEMM_STAMP(15);
         return;
     }
     // Slices meet through device memory, as in the GEMV: agent-scope stores, wait for their
@@ -632,7 +614,6 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
                            __HIP_MEMORY_SCOPE_AGENT);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    GEMM_STAMP(14);
     __syncthreads();
     unsigned *s_ticket = (unsigned *)(smem + L::TICKET_OFF);
     unsigned *counter = a.counters + cb;
@@ -679,7 +660,6 @@ __global__ __launch_bounds__(GemmLds<MR>::NW * 64) void hlq_gemm_kernel(const Ge
         }
     }
     if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    GEMM_STAMP(15);
 }
 
 // Kernels that need more than 64 KiB of dynamic LDS must be told so once per device (the
@@ -738,13 +718,6 @@ int dispatch_gemm(const GemmArgs &a, int bits, bool g64, hipStream_t stream)
 }  // namespace
 
 extern "C" {
-
-#ifdef HLQ_TIMING
-int elutq_debug_set_gemm_stamps(void *d_buf)
-{
-    return hipMemcpyToSymbol(HIP_SYMBOL(g_gemm_stamps), &d_buf, sizeof(d_buf)) == hipSuccess ? 0 : -1;
-}
-#endif
 
 // y[M][N] = x[M][K] W^T + bias.  M == 1 goes to the LUT GEMV; larger M to the MFMA kernel in
 // chunks of up to 64 rows.

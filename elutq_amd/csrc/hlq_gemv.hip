@@ -66,11 +66,6 @@ constexpr int depth_of(int bits) { return bits == 3 ? 6 : (bits == 4 ? 8 : 4); }
 template <int BITS, bool G64, int NSLOT, bool MULTI, int VAR, bool PAIRED>
 __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, int ncb_run, unsigned char *smem, int &red_sel)
 {
-    HLQ_STAMP_DECL;
-#ifdef HLQ_TIMING_ENTRY
-    HLQ_STAMP(7);
-    asm volatile("" ::: "memory");
-#endif
     constexpr bool PLAIN = VAR != GEMV_FUSED;
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
@@ -93,7 +88,6 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     const uint32_t lut_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lut;
 
     __builtin_amdgcn_s_setprio(3);
-    HLQ_STAMP(0);
     // Activations first, then the weight stream.  Every load below is unconditional (a wave
     // whose run is shorter than NSLOT re-reads its last sub-task), so the number of loads
     // behind the activations is a compile-time constant and the table build waits for the
@@ -166,12 +160,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         else
             build_chunk(prologue, raw, raw2, rstd, lut + (size_t)ci * TBL_BYTES, xs_inv + (ci >> 4), (ci & 15) == 0, lane);
     }
-    HLQ_STAMP(1);
     // The tables were written by this wave and are read by this wave: LDS executes a wave's
     // operations in order, so no barrier -- only keep the compiler from reordering.
     asm volatile("" ::: "memory");
     __builtin_amdgcn_wave_barrier();
-    HLQ_STAMP(2);
 
     // Combine the waves of this workgroup, then the slices of this column block.  The wave that
     // does it waits for its partial-sum stores to be acknowledged, and that wait covers every load
@@ -192,7 +184,6 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                 for (int w = 0; w < nw; w++) total += red[w * HLQ_CB + lane];
             }
         }
-        HLQ_STAMP(4);
         if (a.ksplit == 1) {
             if (wave == fin && n < a.N) {
                 if (a.bias) total += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
@@ -211,16 +202,13 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         // the slices meet through device memory (slices_meet): all but the last store and leave
         if (wave == fin) {
             float sum;
-            HLQ_STAMP(5);
             if (slices_meet(a, cbf, slice, npad, n, lane, total, sum)) {
-                HLQ_STAMP(6);
                 if (n < a.N) {
                     if (a.bias) sum += (float)__builtin_bit_cast(_Float16, MULTI ? a.bias[n] : pre_bias);
                     if (residual) sum += (float)__builtin_bit_cast(_Float16, MULTI ? residual[n] : pre_res);
                     if (extra) sum += MULTI ? extra[n] : pre_extra;
                     a.y[n] = __builtin_bit_cast(uint16_t, (_Float16)sum);
                 }
-                HLQ_STAMP(7);
             }
         }
     };
@@ -246,7 +234,6 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         for (int c = 0; c < ncb_run; c++) {
             const CbBase next = cb_base<BITS>(a, min(cb + c + 1, cb + ncb_run - 1), u0);   // past the run: a reload nobody reads
             float accc = 0.f;
-            HLQ_STAMP(2);
             if (s_begin < s_end)                              // wave-uniform; a wave without sub-tasks loads nothing here
                 static_for<0, NSLOT>([&](auto dc) __attribute__((always_inline)) {
                     constexpr int d = decltype(dc)::value;
@@ -255,11 +242,8 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                     if (st < s_end) accc = run_slot(dc, st, accc);
                     load_slot<BITS, G64, PAIRED, d>(slot[d], next, u0, min(st, s_last), lane);
                 });
-            HLQ_STAMP(3);
             finish(cb + c, accc);
-            HLQ_STAMP(6);
         }
-        HLQ_STAMP_FLUSH;
         return;
     }
 
@@ -275,9 +259,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                 load_slot<BITS, G64, PAIRED, d>(slot[d], here, u0, min(st + NSLOT, s_last), lane);
         });
     }
-    HLQ_STAMP(3);
     finish(cb, acc);
-    HLQ_STAMP_FLUSH;
 }
 
 template <int BITS, bool G64, int NSLOT, bool PAIRED, int VAR>
@@ -646,13 +628,6 @@ size_t shape_lds_bytes(const LaunchShape &sh, int bits)
 }  // namespace
 
 extern "C" {
-
-#ifdef HLQ_TIMING
-int elutq_debug_set_stamps(void *d_buf)
-{
-    return hipMemcpyToSymbol(HIP_SYMBOL(g_hlq_stamps), &d_buf, sizeof(d_buf)) == hipSuccess ? 0 : -1;
-}
-#endif
 
 size_t elutq_hlq_workspace_bytes(int K, int N, int bits, int group, int M)
 {

@@ -61,24 +61,6 @@ struct GemvArgs {
     int drop_slice;                       // -1; tests only: this slice leaves without storing its sums, so that the wait runs out
 };
 
-#ifdef HLQ_TIMING
-// Profiling builds only: per-stage wall-clock stamps (100 MHz) of every wave (up to 16) of every
-// workgroup, kept in registers and written once when the tile is done.
-__device__ unsigned long long *g_hlq_stamps = nullptr;
-#define HLQ_STAMP_DECL unsigned long long hlq_t[8] = {0, 0, 0, 0, 0, 0, 0, 0}
-#define HLQ_STAMP(i) hlq_t[i] = wall_clock64()
-#define HLQ_STAMP_FLUSH                                                                           \
-    do {                                                                                          \
-        if (g_hlq_stamps && (threadIdx.x & 63) == 0)                                              \
-            for (int hlq_i = 0; hlq_i < 8; hlq_i++)                                               \
-                g_hlq_stamps[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (threadIdx.x >> 6)) * 8 + hlq_i] = hlq_t[hlq_i]; \
-    } while (0)
-#else
-#define HLQ_STAMP_DECL do { } while (0)
-#define HLQ_STAMP(i) do { } while (0)
-#define HLQ_STAMP_FLUSH do { } while (0)
-#endif
-
 // One tile of a grouped launch (many independent GEMVs in one launch): a run of consecutive column blocks of one
 // K slice of one problem of the list.
 struct GroupItem {

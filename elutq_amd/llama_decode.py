@@ -10,12 +10,12 @@ pairs (j, j + d/2) with theta = pos * base^(-2j/d) and no frequency rescaling
 (arm_rotary.cpp:31-46), fp32 softmax, GQA map h_kv = h * n_kv / n_q
 (arm_attention.cpp:199-274), SiLU*up in fp32 (arm_activation.cpp:36-49).
 
-impl="hip": five fused launches per layer, final norm and greedy pick as kernels of the
-library, the fp16 lm_head (hipBLASLt) through PyTorch; impl="torch": the
-same model with PyTorch-ROCm ops around the HLQ projections (the parity partner).  The step
-is captured in a HIP graph (token id and position live in device tensors), so one replay =
-one token.  q|k|v and gate|up are fused along N, which in the kernel layout is a
-concatenation of the packed buffers.
+Five fused launches per layer, embedding gather, final norm, lm_head and greedy pick as kernels
+of the library.  The step is captured in a HIP graph (token id and position live in device
+tensors), so one replay = one token.  q|k|v and gate|up are fused along N, which in the kernel
+layout is a concatenation of the packed buffers.  (The same step written with PyTorch ops around
+plain HLQLinear calls, the parity partner of this path, lives with the tests:
+tests/torch_glue_decode.py.)
 """
 from __future__ import annotations
 
@@ -24,7 +24,6 @@ import time
 from dataclasses import dataclass
 
 import torch
-import torch.nn.functional as F
 from torch import nn
 
 from . import _lib
@@ -95,11 +94,6 @@ def concat_sparse(mods: list[HLQLinear]):
     return (torch.cat(blocks).view(nblk, 32, group // 8), torch.cat(scales), index)
 
 
-def rms_norm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
-    xf = x.float()
-    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(torch.float16)
-
-
 class DecoderLayer(nn.Module):
     def __init__(self, s: LlamaShape, linears: dict, norms: tuple, fuse: bool = True):
         super().__init__()
@@ -117,37 +111,6 @@ class DecoderLayer(nn.Module):
         self.register_buffer("k_cache", torch.zeros(s.max_seq, s.n_kv_heads, s.head_dim, dtype=torch.float16,
                                                     device=norms[0].device))
         self.register_buffer("v_cache", torch.zeros_like(self.k_cache))
-
-    def forward(self, x, pos, cos, sin, mask):
-        """x [1, hidden] fp16; pos int64 [1] (device); cos/sin [1, head_dim/2] fp32 at pos;
-        mask [1, 1, max_seq] additive fp32 (0 up to pos, -inf beyond)."""
-        s = self.s
-        d, nq, nkv = s.head_dim, s.n_heads, s.n_kv_heads
-        h = rms_norm(x, self.ln1, s.rms_eps)
-        if self.fused:
-            qkv = self.qkv(h)
-            q, k, v = qkv.split([nq * d, nkv * d, nkv * d], dim=-1)
-        else:
-            q, k, v = self.q_proj(h), self.k_proj(h), self.v_proj(h)
-        q = rope(q.view(nq, d), cos, sin)
-        k = rope(k.view(nkv, d), cos, sin)
-        self.k_cache.index_copy_(0, pos, k.unsqueeze(0))
-        self.v_cache.index_copy_(0, pos, v.reshape(1, nkv, d))
-        # single-token GQA attention over the whole cache buffer, masked beyond pos
-        qg = q.view(nkv, nq // nkv, d).float()
-        kc = self.k_cache.permute(1, 2, 0).float()                 # [nkv, d, L]
-        scores = torch.matmul(qg, kc) * (d ** -0.5) + mask         # [nkv, nq/nkv, L]
-        p = torch.softmax(scores, dim=-1)
-        ctx = torch.matmul(p, self.v_cache.permute(1, 0, 2).float())   # [nkv, nq/nkv, d]
-        attn = ctx.to(torch.float16).reshape(1, nq * d)
-        x = x + self.o_proj(attn)
-        h = rms_norm(x, self.ln2, s.rms_eps)
-        if self.fused:
-            g, u = self.gate_up(h).split([s.ffn, s.ffn], dim=-1)
-        else:
-            g, u = self.gate_proj(h), self.up_proj(h)
-        act = (F.silu(g.float()) * u.float()).to(torch.float16)
-        return x + self.down_proj(act)
 
 
 class FusedBuffers:
@@ -232,13 +195,6 @@ def fused_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tensor) 
     layer.down_proj.gemv_fused(b.gu, b.xa, b.ws, prologue=2, residual=b.xb)
 
 
-def rope(t: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
-    """Half-split rotation: pairs (j, j + d/2)."""
-    d2 = t.shape[-1] // 2
-    a, b = t[..., :d2].float(), t[..., d2:].float()
-    return torch.cat([a * cos - b * sin, b * cos + a * sin], dim=-1).to(torch.float16)
-
-
 PROJ_DIRS = {"q_proj": "self_attn.q_proj", "k_proj": "self_attn.k_proj", "v_proj": "self_attn.v_proj",
              "o_proj": "self_attn.o_proj", "gate_proj": "mlp.gate_proj", "up_proj": "mlp.up_proj",
              "down_proj": "mlp.down_proj"}
@@ -312,16 +268,16 @@ def parts_from_export(root: str, s: LlamaShape, dev, sparse_mode: str = "auto") 
 class LlamaDecoder(nn.Module):
     """Random-init LLaMA-shaped decoder for the decode benchmark and its parity test."""
 
-    def __init__(self, s: LlamaShape, device="cuda", seed: int = 0, fuse: bool = True, impl: str = "hip",
+    FUSED_LAUNCHES = True      # (a subclass that steps through other operators sets this to False: no launch buffers)
+
+    def __init__(self, s: LlamaShape, device="cuda", seed: int = 0, fuse: bool = True,
                  parts: dict | None = None, qkv_to_attention: bool = True):
-        """impl "hip": five fused launches per layer through the C ABI (needs fuse=True);
-        impl "torch": the same step with PyTorch ops around plain HLQLinear calls.
+        """Five fused launches per layer through the C ABI (q|k|v and gate|up fused along N: fuse=True).
         qkv_to_attention: run q|k|v in two K slices that the attention launch sums (head_dim 128) rather than
         on the narrow-tile kernel (measured on MI355X at the LLaMA-3-8B shape: 835 against 817 tokens/s)."""
         super().__init__()
-        assert impl in ("hip", "torch") and (fuse or impl == "torch")
+        assert fuse or not self.FUSED_LAUNCHES
         self.s = s
-        self.impl = impl
         dev = torch.device(device)
         d = s.head_dim
         if parts is None:
@@ -347,7 +303,7 @@ class LlamaDecoder(nn.Module):
         # logits are bit for bit those of fused_layer_step.  Set before capture().
         self.defer_slices = True
         self.defer_qkv = False             # likewise q|k|v -> attention (set by the constructor, see qkv_to_attention)
-        if impl == "hip":
+        if self.FUSED_LAUNCHES:
             ws = max(m.workspace_bytes for m in self.modules() if isinstance(m, HLQLinear))
             ws = max(ws, _lib.lib().elutq_decode_attn_workspace_bytes(s.n_heads, s.head_dim, 0))
             self._buf = FusedBuffers(s, ws, dev)
@@ -380,11 +336,10 @@ class LlamaDecoder(nn.Module):
                     layer.down_proj.ksplit = _lib.GEMV_WIDE
 
     @classmethod
-    def from_export(cls, root: str, s: LlamaShape, device="cuda", fuse: bool = True, impl: str = "hip",
+    def from_export(cls, root: str, s: LlamaShape, device="cuda", fuse: bool = True,
                     sparse_mode: str = "auto") -> "LlamaDecoder":
         """A decoder over a genuinely exported model (bits and group size come from the files)."""
-        return cls(s, device=device, fuse=fuse, impl=impl,
-                   parts=parts_from_export(root, s, torch.device(device), sparse_mode))
+        return cls(s, device=device, fuse=fuse, parts=parts_from_export(root, s, torch.device(device), sparse_mode))
 
     @torch.no_grad()
     def fill_cache(self, n_tokens: int, seed: int = 1) -> None:
@@ -401,51 +356,37 @@ class LlamaDecoder(nn.Module):
     def step(self) -> torch.Tensor:
         """One decode step from the device-resident (token, pos); stores the greedy next token
         and pos + 1 back.  Returns the logits [1, vocab] (fp16)."""
-        if self.impl == "hip":
-            b = self._buf
-            _lib.check(_lib.lib().elutq_decode_embed_f16(self.embed.data_ptr(), self.token.data_ptr(), b.xa.data_ptr(),
-                                                         self.s.hidden, self.s.vocab,
-                                                         torch.cuda.current_stream().cuda_stream), "elutq_decode_embed_f16")
-            if self.defer_slices:
-                x, free, pending = b.xa, b.xb, 0
-                for i, layer in enumerate(self.layers):
-                    x, free, pending = deferred_layer_step(layer, b, self.pos, x, free, pending,
-                                                           last=i == len(self.layers) - 1, defer_qkv=self.defer_qkv,
-                                                           defer_down=self._defer_down[i])
-            else:
-                for layer in self.layers:
-                    fused_layer_step(layer, b, self.pos)
-                x, free = b.xa, b.xb
+        b = self._buf
+        _lib.check(_lib.lib().elutq_decode_embed_f16(self.embed.data_ptr(), self.token.data_ptr(), b.xa.data_ptr(),
+                                                     self.s.hidden, self.s.vocab,
+                                                     torch.cuda.current_stream().cuda_stream), "elutq_decode_embed_f16")
+        if self.defer_slices:
+            x, free, pending = b.xa, b.xb, 0
+            for i, layer in enumerate(self.layers):
+                x, free, pending = deferred_layer_step(layer, b, self.pos, x, free, pending,
+                                                       last=i == len(self.layers) - 1, defer_qkv=self.defer_qkv,
+                                                       defer_down=self._defer_down[i])
         else:
-            x = self.embed.index_select(0, self.token)
-            cos = self.cos_t.index_select(0, self.pos)
-            sin = self.sin_t.index_select(0, self.pos)
-            mask = torch.where(self.arange <= self.pos, 0.0, float("-inf")).view(1, 1, -1)
             for layer in self.layers:
-                x = layer(x, self.pos, cos, sin, mask)
-        if self.impl == "hip":
-            L, stream = _lib.lib(), torch.cuda.current_stream().cuda_stream
-            if self.lm_head_q is not None:       # the final norm rides in the GEMV's prologue
-                logits = self.lm_head_q.gemv_fused(x, b.logits, b.ws, prologue=1, norm_weight=self.norm,
-                                                   eps=self.s.rms_eps)
-            elif self.s.hidden % 8 == 0 and self.s.hidden <= 32768 and self.lm_head.data_ptr() % 16 == 0:
-                # the unquantized lm_head: the library's dense fp16 GEMV, the final norm in the same launch
-                logits = b.logits
-                _lib.check(L.elutq_fp16_gemv_f16(self.lm_head.data_ptr(), None, x.data_ptr(), logits.data_ptr(), self.s.hidden,
-                                                 self.s.vocab, self.norm.data_ptr(), self.s.rms_eps, stream),
-                           "elutq_fp16_gemv_f16")
-            else:
-                _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), free.data_ptr(),
-                                                      self.s.hidden, self.s.rms_eps, stream), "elutq_decode_rmsnorm_f16")
-                logits = torch.mm(free, self.lm_head.t(), out=b.logits)
-            _lib.check(L.elutq_decode_argmax_ws_f16(logits.data_ptr(), self.s.vocab, self.token.data_ptr(),
-                                                    self.pos.data_ptr(), b.ws.data_ptr(), b.ws.numel(), stream),
-                       "elutq_decode_argmax_ws_f16")
-            return logits
-        xn = rms_norm(x, self.norm, self.s.rms_eps)
-        logits = self.lm_head_q(xn) if self.lm_head_q is not None else F.linear(xn, self.lm_head)
-        self.token.copy_(logits.argmax(-1))
-        self.pos.add_(1)
+                fused_layer_step(layer, b, self.pos)
+            x, free = b.xa, b.xb
+        L, stream = _lib.lib(), torch.cuda.current_stream().cuda_stream
+        if self.lm_head_q is not None:       # the final norm rides in the GEMV's prologue
+            logits = self.lm_head_q.gemv_fused(x, b.logits, b.ws, prologue=1, norm_weight=self.norm,
+                                               eps=self.s.rms_eps)
+        elif self.s.hidden % 8 == 0 and self.s.hidden <= 32768 and self.lm_head.data_ptr() % 16 == 0:
+            # the unquantized lm_head: the library's dense fp16 GEMV, the final norm in the same launch
+            logits = b.logits
+            _lib.check(L.elutq_fp16_gemv_f16(self.lm_head.data_ptr(), None, x.data_ptr(), logits.data_ptr(), self.s.hidden,
+                                             self.s.vocab, self.norm.data_ptr(), self.s.rms_eps, stream),
+                       "elutq_fp16_gemv_f16")
+        else:
+            _lib.check(L.elutq_decode_rmsnorm_f16(x.data_ptr(), self.norm.data_ptr(), free.data_ptr(),
+                                                  self.s.hidden, self.s.rms_eps, stream), "elutq_decode_rmsnorm_f16")
+            logits = torch.mm(free, self.lm_head.t(), out=b.logits)
+        _lib.check(L.elutq_decode_argmax_ws_f16(logits.data_ptr(), self.s.vocab, self.token.data_ptr(),
+                                                self.pos.data_ptr(), b.ws.data_ptr(), b.ws.numel(), stream),
+                   "elutq_decode_argmax_ws_f16")
         return logits
 
     @torch.no_grad()
@@ -472,7 +413,7 @@ class LlamaDecoder(nn.Module):
 
 
 def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | None = None,
-                 impl: str = "hip", hlq_lm_head: bool = False) -> dict:
+                 hlq_lm_head: bool = False) -> dict:
     """Decode tokens/s of the random-init model: n_gen greedy tokens after an n_ctx-token
     cache; the first generated token is excluded, as in the reference
     ((generate_num - 1) / elapsed, main.cpp:110).  `hlq_lm_head`: see random_parts."""
@@ -481,7 +422,7 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
         # the attention launch of a position beyond the cache returns at once (NaN output): such tokens must not be timed
         raise ValueError(f"n_ctx + n_gen = {n_ctx + n_gen} exceeds the cache of {s.max_seq} positions")
     dev = torch.device(device)
-    model = LlamaDecoder(s, device=dev, seed=0, impl=impl, parts=random_parts(s, dev, 0, hlq_lm_head))
+    model = LlamaDecoder(s, device=dev, seed=0, parts=random_parts(s, dev, 0, hlq_lm_head))
     model.fill_cache(n_ctx)
     model.token.fill_(1)
     model.capture()
@@ -509,10 +450,8 @@ def bench_decode(device, n_ctx: int = 512, n_gen: int = 50, shape: LlamaShape | 
             "GBps": (hlq_bytes + lm_bytes + kv_bytes) / (ms * 1e-3) / 1e9,
             "model": f"LLaMA-3-8B-shaped random init, {s.n_layers} layers, HLQ w{s.bits}g{s.group}, "
                      + (f"HLQ w{s.bits}g{s.group} lm_head" if hlq_lm_head else "fp16 lm_head"),
-            "glue": ("5 launches per layer (rmsnorm+qkv | rope+cache+attention | o+residual | rmsnorm+gate|up | "
-                     "silu*up+down+residual; the K slices of q|k|v and of down are summed by the launch that reads "
-                     "them), " if impl == "hip" else "PyTorch-ROCm ops around the HLQ GEMVs, ")
-                    + ("own embedding gather and argmax kernels, "
-                       + ("HLQ GEMV lm_head, " if hlq_lm_head else "own dense fp16 GEMV lm_head, ") + "the final norm inside the lm_head launch, "
-                       if impl == "hip" else "torch embedding / final norm / hipBLASLt fp16 lm_head / argmax, ")
+            "glue": "5 launches per layer (rmsnorm+qkv | rope+cache+attention | o+residual | rmsnorm+gate|up | "
+                    "silu*up+down+residual; the K slices of q|k|v and of down are summed by the launch that reads "
+                    "them), own embedding gather and argmax kernels, "
+                    + ("HLQ GEMV lm_head, " if hlq_lm_head else "own dense fp16 GEMV lm_head, ") + "the final norm inside the lm_head launch, "
                     + "one HIP graph per token"}

@@ -442,17 +442,6 @@ int elutq_hlq_sparse_gemv_fused_f16(const void *d_planes, const void *d_scales, 
 int elutq_hlq_sparse_dequant_add_f16(const void *d_blocks, const void *d_blk_scales, const void *d_index, int nblk,
                                      void *d_w, int K, int N, int group, void *stream);
 
-/*
- * Measurement aid with no counterpart in the reference: one workgroup of `waves` (1..16) wavefronts per compute
- * unit (`waves` = 32: two workgroups of 16) does `passes` (even) x 16 lookups per wavefront in 16-entry LDS tables
- * and nothing else.  sequence = 0: bare ds_read_b32 instructions in the LUT GEMV's access pattern -- what the LDS
- * of a compute unit delivers; sequence = 1: the LUT GEMV's own instruction sequence for a sub-task (address
- * formation, lookups, integer sums, scaling) on plane words held in registers -- what that sequence reaches when it
- * never waits for memory.  Launch time / (passes * 16 * waves) = time per wavefront lookup of one compute unit.
- * d_out: 256 * waves * 64 uint32 (written, contents meaningless).  bench.py --mode lds-rate times both.
- */
-int elutq_diag_lds_lookup_rate(int sequence, int waves, int passes, void *d_out, void *stream);
-
 #ifdef __cplusplus
 }
 #endif

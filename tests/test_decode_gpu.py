@@ -8,6 +8,7 @@ import torch.nn.functional as F
 
 from elutq_amd.hlq_linear import HLQLinear
 from elutq_amd.llama_decode import LlamaDecoder, LlamaShape, fuse_along_n
+from torch_glue_decode import TorchGlueDecoder, make_decoder, rms_norm, rope
 from elutq_amd.synth import make_device_layer
 
 pytestmark = pytest.mark.gpu
@@ -47,8 +48,8 @@ def test_fuse_along_n_is_concatenation(cuda):
 
 @pytest.mark.parametrize("fuse,impl", [(True, "hip"), (True, "torch"), (False, "torch")])
 def test_decode_step_matches_dense_model(cuda, fuse, impl):
-    hlq = LlamaDecoder(SMALL, device=cuda, seed=3, fuse=fuse, impl=impl)
-    ref = densify(LlamaDecoder(SMALL, device=cuda, seed=3, fuse=fuse, impl="torch"))
+    hlq = make_decoder(impl, SMALL, device=cuda, seed=3, fuse=fuse)
+    ref = densify(TorchGlueDecoder(SMALL, device=cuda, seed=3, fuse=fuse))
     for m in (hlq, ref):
         m.fill_cache(20, seed=5)
         m.token.fill_(7)
@@ -67,8 +68,8 @@ def test_decode_step_matches_dense_model(cuda, fuse, impl):
 def test_fused_launches_match_torch_glue(cuda):
     """The five fused launches per layer against the same HLQ model run with PyTorch glue:
     same tokens, logits within fp16 rounding of the intermediate activations."""
-    a = LlamaDecoder(SMALL, device=cuda, seed=6, impl="hip")
-    b = LlamaDecoder(SMALL, device=cuda, seed=6, impl="torch")
+    a = LlamaDecoder(SMALL, device=cuda, seed=6)
+    b = TorchGlueDecoder(SMALL, device=cuda, seed=6)
     for m in (a, b):
         m.fill_cache(33, seed=8)
         m.token.fill_(11)
@@ -83,8 +84,8 @@ def test_fused_launches_match_torch_glue(cuda):
 
 @pytest.mark.parametrize("impl", ["hip", "torch"])
 def test_graph_replay_equals_eager(cuda, impl):
-    eager = LlamaDecoder(SMALL, device=cuda, seed=4, impl=impl)
-    graph = LlamaDecoder(SMALL, device=cuda, seed=4, impl=impl)
+    eager = make_decoder(impl, SMALL, device=cuda, seed=4)
+    graph = make_decoder(impl, SMALL, device=cuda, seed=4)
     for m in (eager, graph):
         m.fill_cache(10, seed=2)
         m.token.fill_(3)
@@ -122,7 +123,6 @@ def test_rope_cache_attention_kernel_long_context(cuda, d, nq, nkv, splits, pos)
 
 def check_rope_cache_attention(cuda, d, nq, nkv, splits, pos, max_seq):
     from elutq_amd import _lib
-    from elutq_amd.llama_decode import rope
     g = torch.Generator(device=cuda).manual_seed(pos * 7 + d)
     base = 10000.0
     L = _lib.lib()
@@ -253,7 +253,6 @@ def test_argmax_kernel(cuda, n, split):
 def test_final_rmsnorm_kernel(cuda, n):
     """elutq_decode_rmsnorm_f16 against the fp32 restatement of arm_rmsnorm.cpp:25-84."""
     from elutq_amd import _lib
-    from elutq_amd.llama_decode import rms_norm
     g = torch.Generator(device=cuda).manual_seed(n)
     x = (torch.randn(1, n, generator=g, device=cuda) * 3).half()
     w = (1 + 0.1 * torch.randn(n, generator=g, device=cuda)).half()

@@ -14,6 +14,7 @@ import torch
 
 from elutq_amd.hlq_linear import HLQLinear
 from elutq_amd.llama_decode import LlamaDecoder, LlamaShape
+from torch_glue_decode import TorchGlueDecoder
 from elutq_amd.synth import make_layer
 from oracle import hlq_oracle as O
 from test_decode_gpu import densify
@@ -87,12 +88,12 @@ def test_decode_step_at_full_llama3_8b_width(cuda):
     against the same HLQ model under PyTorch glue and against the dense fp32 model, eager steps and graph
     replays, with the K slices handed to the consuming launch and summed by the producer."""
     print("decode step at full width: building models", flush=True)
-    hip = LlamaDecoder(FULL, device=cuda, seed=5, impl="hip")
-    hip_nd = LlamaDecoder(FULL, device=cuda, seed=5, impl="hip")
+    hip = LlamaDecoder(FULL, device=cuda, seed=5)
+    hip_nd = LlamaDecoder(FULL, device=cuda, seed=5)
     hip_nd.defer_slices = hip_nd.defer_qkv = False
-    graph = LlamaDecoder(FULL, device=cuda, seed=5, impl="hip")
-    glue = LlamaDecoder(FULL, device=cuda, seed=5, impl="torch")
-    dense = densify(LlamaDecoder(FULL, device=cuda, seed=5, impl="torch"))
+    graph = LlamaDecoder(FULL, device=cuda, seed=5)
+    glue = TorchGlueDecoder(FULL, device=cuda, seed=5)
+    dense = densify(TorchGlueDecoder(FULL, device=cuda, seed=5))
     models = (hip, hip_nd, graph, glue, dense)
     for m in models:
         m.fill_cache(512, seed=9)

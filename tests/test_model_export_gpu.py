@@ -6,6 +6,7 @@ import torch
 
 from elutq_amd.hlq_linear import HLQLinear
 from elutq_amd.llama_decode import LlamaDecoder
+from torch_glue_decode import TorchGlueDecoder, decoder_from_export, make_decoder
 from elutq_amd.repack import repack_tree
 
 from model_export_fixture import TINY, write_tiny_export
@@ -34,9 +35,9 @@ def test_decoder_from_export_tree(cuda, tmp_path, kind, impl):
     src, dst = str(tmp_path / "export"), str(tmp_path / "repacked")
     arrays = write_tiny_export(src, lm_head=kind)
     repack_tree(src, dst)
-    models = [LlamaDecoder.from_export(src, TINY, device=cuda, impl=impl),
-              LlamaDecoder.from_export(dst, TINY, device=cuda, impl=impl),
-              LlamaDecoder(TINY, device=cuda, impl=impl, parts=in_memory_parts(arrays, cuda))]
+    models = [decoder_from_export(impl, src, TINY, device=cuda),
+              decoder_from_export(impl, dst, TINY, device=cuda),
+              make_decoder(impl, TINY, device=cuda, parts=in_memory_parts(arrays, cuda))]
     assert (models[0].lm_head_q is not None) == (kind == "hlq")
     if kind == "tied":
         assert torch.equal(models[0].lm_head, models[0].embed)
@@ -54,7 +55,7 @@ def test_decoder_from_export_tree(cuda, tmp_path, kind, impl):
     assert all(0 <= t < TINY.vocab for t in outs[0][0]) and int(models[0].pos) == 13
     if impl == "hip":
         # the fused step (with an HLQ lm_head: final norm inside its GEMV) against the PyTorch-glue step
-        glue = LlamaDecoder.from_export(src, TINY, device=cuda, fuse=False, impl="torch")
+        glue = TorchGlueDecoder.from_export(src, TINY, device=cuda, fuse=False)
         glue.fill_cache(9, seed=3)
         glue.token.fill_(5)
         first = glue.step().float()
@@ -71,9 +72,9 @@ def test_decoder_with_sparse_extra_planes(cuda, tmp_path):
     write_tiny_export(plain)
     repack_tree(src, dst)
     outs = []
-    for root, kw in ((src, dict(impl="hip")), (dst, dict(impl="hip")), (src, dict(fuse=False, impl="torch", sparse_mode="blocks")),
-                     (plain, dict(impl="hip")), (src, dict(impl="hip", sparse_mode="blocks"))):
-        m = LlamaDecoder.from_export(root, TINY, device=cuda, **kw)
+    for root, impl, kw in ((src, "hip", {}), (dst, "hip", {}), (src, "torch", dict(fuse=False, sparse_mode="blocks")),
+                           (plain, "hip", {}), (src, "hip", dict(sparse_mode="blocks"))):
+        m = decoder_from_export(impl, root, TINY, device=cuda, **kw)
         m.fill_cache(9, seed=3)
         m.token.fill_(5)
         logits = torch.cat([m.step().clone() for _ in range(3)])
