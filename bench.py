@@ -230,9 +230,10 @@ def gemm_leg(torch, lib, dev, steps):
 
 def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
     """Batch-1 GEMV of w2g128 layers that carry a block-sparse extra plane on `density` of their
-    (32 channels x 128 inputs) blocks, held as blocks -- two launches: the plane's fp32 term, then the
-    dense GEMV that adds it -- next to the same dense layers alone and to layers of one more dense
-    plane (the form the loader gives the plane by default).  Weight rings of `ring_len` layers per shape."""
+    (32 channels x 128 inputs) blocks, held as blocks: looked up inside the dense launch (the inline form) and as
+    two launches (the plane's fp32 term, then the dense GEMV that adds it), next to the same dense layers alone and to
+    layers of one more dense plane (the form the loader gives the plane by default).  Weight rings of `ring_len`
+    layers per shape."""
     import numpy as np
 
     from elutq_amd.hlq_linear import sparse_index
@@ -285,7 +286,18 @@ def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
         def launch_fused_dense(stream):
             launch_fused(stream, [mod for mod, _, _ in ring])
 
-        t_fu = time_graph(torch, launch_fused, steps, warmup) / ring_len
+        def launch_inline(stream):                  # plain call, the blocks looked up inside the dense launch
+            for m in fused:
+                m.gemv_fused(x, y, ws)
+
+        assert all(m.sparse_inline is not None for m in fused)
+        t_in = time_graph(torch, launch_inline, steps, warmup) / ring_len
+        t_fi = time_graph(torch, launch_fused, steps, warmup) / ring_len
+        HLQLinear.use_sparse_inline = False         # the plane as a launch of its own in front of the dense one
+        try:
+            t_fu = time_graph(torch, launch_fused, steps, warmup) / ring_len
+        finally:
+            HLQLinear.use_sparse_inline = True
         t_fd = time_graph(torch, launch_fused_dense, steps, warmup) / ring_len
         # the plane written out as one more dense plane (scale 0 where no block exists): what the loader does
         # by default -- it costs what any layer with one more plane costs
@@ -297,9 +309,10 @@ def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
 
         t_wi = time_graph(torch, launch_wide, steps, warmup) / ring_len
         sparse_bytes = nblk * (32 * GROUP // 8 + 64 + 4) + 4 * (n // 32 + 1) + 8 * n      # blocks, scales, index, fp32 term out and in
-        out[f"{k}x{n}"] = {"blocks": nblk, "density": density, "sparse_layer_us": t_sp * 1e6, "dense_layer_us": t_de * 1e6,
-                           "as_one_more_dense_plane_us": t_wi * 1e6,
-                           "rmsnorm_residual_sparse_layer_us": t_fu * 1e6, "rmsnorm_residual_dense_layer_us": t_fd * 1e6,
+        out[f"{k}x{n}"] = {"blocks": nblk, "density": density, "inline_layer_us": t_in * 1e6, "two_launch_layer_us": t_sp * 1e6,
+                           "dense_layer_us": t_de * 1e6, "as_one_more_dense_plane_us": t_wi * 1e6,
+                           "rmsnorm_residual_inline_layer_us": t_fi * 1e6, "rmsnorm_residual_two_launch_layer_us": t_fu * 1e6,
+                           "rmsnorm_residual_dense_layer_us": t_fd * 1e6,
                            "sparse_plane_bytes": sparse_bytes, "dense_bytes": algorithmic_bytes(k, n, BITS, GROUP)}
     out["decode"] = sparse_decode_leg(torch, dev, density)
     return out
@@ -307,7 +320,7 @@ def sparse_leg(torch, lib, dev, steps, warmup, density=0.1, ring_len=16):
 
 def sparse_decode_leg(torch, dev, density, n_ctx=512, n_gen=50):
     """Decode tokens/s of the LLaMA-3-8B-shaped w2g128 model whose every projection carries a sparse extra plane on
-    `density` of its blocks, held as blocks: the fused step with one launch of the plane in front of each projection."""
+    `density` of its blocks, held as blocks and looked up inside the projections' own launches."""
     from elutq_amd.llama_decode import LlamaDecoder, LlamaShape, random_parts
     from elutq_amd.synth import with_device_sparse_plane
     s = LlamaShape()
@@ -335,7 +348,7 @@ def sparse_decode_leg(torch, dev, density, n_ctx=512, n_gen=50):
     sec = time.perf_counter() - t0
     return {"tokens_per_s": (n_gen - 1) / sec, "ms_per_token": sec / (n_gen - 1) * 1e3, "blocks": nblk, "density": density,
             "model": "LLaMA-3-8B-shaped random init, 32 layers, HLQ w2g128 + sparse extra plane held as blocks on every "
-                     "projection, fp16 lm_head", "n_ctx": n_ctx, "n_gen": n_gen}
+                     "projection (inline form: one launch per projection), fp16 lm_head", "n_ctx": n_ctx, "n_gen": n_gen}
 
 
 def counter_mode(a, torch, lib, dev):

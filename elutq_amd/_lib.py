@@ -59,6 +59,9 @@ SIGNATURES = {
     "elutq_hlq_sparse_gemm_f16": (_ci, [_vp] * 7 + [_ci] + [_vp] * 2 + [_ci] * 5 + [_vp, _sz, _vp]),
     "elutq_hlq_sparse_gemv_fused_f16": (_ci, [_vp] * 7 + [_ci] + [_vp] * 2 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
     "elutq_hlq_sparse_dequant_add_f16": (_ci, [_vp] * 3 + [_ci, _vp] + [_ci] * 3 + [_vp]),
+    "elutq_hlq_sparse_inline_bytes": (_sz, [_ci] * 4),
+    "elutq_hlq_sparse_inline_host": (_ci, [_vp, _ci, _vp, _vp, _ci, _ci, _ci, _vp, _vp]),
+    "elutq_hlq_sparse_gemv_inline_f16": (_ci, [_vp] * 7 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
 }
 
 
@@ -113,6 +116,7 @@ def lib() -> ctypes.CDLL:
 GEMV_ENGINES = {"auto": 0, "lut": 1, "mfma": 2}
 # values of the `ksplit` tuning argument that name a kernel instead of a slice count (include/elutq_hip.h)
 GEMV_NARROW16, GEMV_NARROW32, GEMV_WIDE = -16, -32, -64
+ERR_SPARSE = -8        # ELUTQ_ERR_SPARSE: a block list that a form of the sparse extra plane cannot hold
 
 
 def set_gemv_engine(name: str) -> None:

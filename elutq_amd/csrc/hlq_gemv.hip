@@ -66,10 +66,11 @@ constexpr int depth_of(int bits) { return bits == 3 ? 6 : (bits == 4 ? 8 : 4); }
 template <int BITS, bool G64, int NSLOT, bool MULTI, int VAR, bool PAIRED>
 __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, int ncb_run, unsigned char *smem, int &red_sel)
 {
-    constexpr bool PLAIN = VAR != GEMV_FUSED;
+    constexpr bool SPARSE = VAR == GEMV_SPARSE;
+    constexpr bool PLAIN = VAR != GEMV_FUSED && !SPARSE;
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
-    const HLQ_GLOBAL float *extra = (VAR == GEMV_FUSED || VAR == GEMV_EXTRA) ? a.extra : nullptr;
+    const HLQ_GLOBAL float *extra = (VAR == GEMV_FUSED || VAR == GEMV_EXTRA || SPARSE) ? a.extra : nullptr;
     const int tid = threadIdx.x, lane = tid & 63, nw = blockDim.x >> 6;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int u0 = slice * a.ups, nU = min(u0 + a.ups, a.U) - u0;
@@ -119,6 +120,36 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     // (where K ends half way through the last unit, the chunks of the absent half re-read the last one and count as zeros)
     const size_t kfirst = hlq_x_first_k(k0, nchunks, lane);
     load_chunk<PLAIN>(a, prologue, K, hlq_x_load_k(kfirst, K), raw, raw2);
+    // Block-sparse extra plane: a unit's blocks are looked up by the wave that has the unit's plane 0 in its run, in the
+    // tables it builds anyway.  The record numbers of the first two units of the run come in with the activations, the
+    // records themselves are requested once the tables stand and arrive while the dense planes are looked up.
+    // (Dealing the units that have blocks evenly to the waves, whichever wave built their tables, was measured: the
+    // barrier it needs in front of the lookups costs more than the uneven work -- 8.1 against 7.5 us at 4096 x 14336.)
+    int scell[2] = {-1, -1};
+    bool sown[2] = {false, false};
+    Sub sp[2];
+    auto sp_cells_load = [&](int cbx, int (&out)[2]) __attribute__((always_inline)) {
+        const HLQ_GLOBAL int32_t *row = a.sp_cells + ((size_t)cbx * a.U + u0);
+#pragma unroll
+        for (int j = 0; j < 2; j++) out[j] = row[min(ub + j, nU - 1)];
+    };
+    auto sp_recs_load = [&](int (&cell)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            cell[j] = sown[j] ? __builtin_amdgcn_readfirstlane(cell[j]) : -1;
+            if (cell[j] >= 0) {                                            // wave-uniform
+                const HLQ_GLOBAL unsigned char *r = a.sp_recs + (size_t)cell[j] * HLQ_SP_REC_BYTES;
+                const u32x4 v = __builtin_nontemporal_load((const HLQ_GLOBAL u32x4 *)(r + (uint32_t)lane * 16u));
+                sp[j].w = make_uint4(v.x, v.y, v.z, v.w);
+                sp[j].sc = *(const HLQ_GLOBAL uint32_t *)(r + 1024u + (uint32_t)lane * 4u);
+            }
+        }
+    };
+    if constexpr (SPARSE) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) sown[j] = j < nuw && s_begin <= (ub + j) * BITS && (ub + j) * BITS < s_end;
+        sp_cells_load(cb, scell);
+    }
     asm volatile("" ::: "memory");      // keep both activation loads ahead of the weight loads
 
     float acc = 0.f;
@@ -134,6 +165,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
     // the combined chunk replaces the base's (a wave without a run sits at the end of the slice: clamped)
     if (sliced) raw = stage[hlq_stage_first_index(k0, nchunks, lane, K)];
     if (kfirst >= (size_t)K) raw = make_uint2(0u, 0u);
+    if constexpr (SPARSE) sp_recs_load(scell);      // (the record numbers came in with the activations)
 
     // ... the tables are built as soon as the activations are in (a wave that first queued all
     // its weight loads would sit in the memory pipeline's back-pressure instead) ...
@@ -230,9 +262,32 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         }
     };
 
+    // the blocks of column block `cbx`: records in `sp` for the first two units of the run, the (rare) further units
+    // of a long run fetched here
+    auto sp_process = [&](int cbx, const int (&cell)[2], float accv) __attribute__((always_inline)) -> float {
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+            if (cell[j] >= 0) accv = process_sub<true>(sp[j].w, sp[j].sc, 0u, j, 1, 0, lut_base, xs_inv, accv);
+        for (int j = 2; j < nuw; j++) {
+            if (!(s_begin <= (ub + j) * BITS && (ub + j) * BITS < s_end)) continue;
+            const int cj = __builtin_amdgcn_readfirstlane(a.sp_cells[(size_t)cbx * a.U + u0 + ub + j]);
+            if (cj < 0) continue;
+            const HLQ_GLOBAL unsigned char *r = a.sp_recs + (size_t)cj * HLQ_SP_REC_BYTES;
+            const u32x4 v = *(const HLQ_GLOBAL u32x4 *)(r + (uint32_t)lane * 16u);
+            const uint32_t scj = *(const HLQ_GLOBAL uint32_t *)(r + 1024u + (uint32_t)lane * 4u);
+            accv = process_sub<true>(make_uint4(v.x, v.y, v.z, v.w), scj, 0u, j, 1, 0, lut_base, xs_inv, accv);
+        }
+        return accv;
+    };
+
     if (MULTI) {
         for (int c = 0; c < ncb_run; c++) {
             const CbBase next = cb_base<BITS>(a, min(cb + c + 1, cb + ncb_run - 1), u0);   // past the run: a reload nobody reads
+            int ncell[2] = {-1, -1};
+            if constexpr (SPARSE) {
+                if (c > 0) sp_recs_load(scell);
+                sp_cells_load(min(cb + c + 1, cb + ncb_run - 1), ncell);
+            }
             float accc = 0.f;
             if (s_begin < s_end)                              // wave-uniform; a wave without sub-tasks loads nothing here
                 static_for<0, NSLOT>([&](auto dc) __attribute__((always_inline)) {
@@ -242,6 +297,10 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                     if (st < s_end) accc = run_slot(dc, st, accc);
                     load_slot<BITS, G64, PAIRED, d>(slot[d], next, u0, min(st, s_last), lane);
                 });
+            if constexpr (SPARSE) {
+                accc = sp_process(cb + c, scell, accc);
+                scell[0] = ncell[0]; scell[1] = ncell[1];
+            }
             finish(cb + c, accc);
         }
         return;
@@ -259,6 +318,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
                 load_slot<BITS, G64, PAIRED, d>(slot[d], here, u0, min(st + NSLOT, s_last), lane);
         });
     }
+    if constexpr (SPARSE) acc = sp_process(cb, scell, acc);
     finish(cb, acc);
 }
 
@@ -273,13 +333,13 @@ __global__ __launch_bounds__(1024) void hlq_gemv_kernel(const GemvArgs a)
 // One GEMV with more column blocks than the chip has CUs: every workgroup takes a run of
 // consecutive column blocks (tables built once, weights prefetched across the blocks) instead
 // of the launch holding two workgroups per CU that each build the same tables.
-template <int BITS, bool G64, int NSLOT, bool PAIRED, bool PLAIN>
+template <int BITS, bool G64, int NSLOT, bool PAIRED, int VAR>
 __global__ __launch_bounds__(1024) void hlq_gemv_run_kernel(const GemvArgs a, int run)
 {
     extern __shared__ __align__(256) unsigned char smem[];
     const int cb0 = blockIdx.y * run;               // grid = (slices, runs of column blocks)
     int sel = 0;
-    gemv_tile<BITS, G64, NSLOT, true, PLAIN ? GEMV_PLAIN : GEMV_FUSED, PAIRED>(a, cb0, blockIdx.x, min(run, a.ncb - cb0), smem, sel);
+    gemv_tile<BITS, G64, NSLOT, true, VAR, PAIRED>(a, cb0, blockIdx.x, min(run, a.ncb - cb0), smem, sel);
 }
 
 // Many independent GEMVs in one launch: the tiles of all of them form one list that the
@@ -337,14 +397,14 @@ bool paired_ok(int spw, int ups, int ksplit)
 template <int BITS, bool G64, int NSLOT, bool PAIRED, int VAR>
 int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
-    constexpr bool PLAIN = VAR == GEMV_PLAIN;
+    constexpr int RUN_VAR = VAR == GEMV_PLAIN ? GEMV_PLAIN : (VAR == GEMV_SPARSE ? GEMV_SPARSE : GEMV_FUSED);
     auto kern = hlq_gemv_kernel<BITS, G64, NSLOT, PAIRED, VAR>;
     static bool big_lds_done[64] = {};        // per template instance
     if (!allow_big_lds((const void *)kern, lds, MAX_LDS, big_lds_done)) return ELUTQ_ERR_HIP;
     // more tiles than CUs and runs that fit the slots: runs of column blocks, one workgroup per CU
     const int run = (a.ncb * a.ksplit + NUM_CU_RUN - 1) / NUM_CU_RUN;
     if (VAR != GEMV_EXTRA && VAR != GEMV_INT8 && run > 1 && a.spw <= NSLOT && waves == 16) {       // (plain plus extra term, int8 tables: no run instances)
-        auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT, PAIRED, PLAIN>;
+        auto kern_run = hlq_gemv_run_kernel<BITS, G64, NSLOT, PAIRED, RUN_VAR>;
         static bool big_lds_run_done[64] = {};
         if (!allow_big_lds((const void *)kern_run, lds, MAX_LDS, big_lds_run_done)) return ELUTQ_ERR_HIP;
         const int groups = (a.ncb + run - 1) / run;
@@ -358,6 +418,10 @@ int launch_gemv_pp(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 template <int BITS, bool G64, int NSLOT, bool PAIRED>
 int launch_gemv_p(const GemvArgs &a, int waves, size_t lds, hipStream_t stream)
 {
+    if constexpr (BITS <= 3) {     // a layer with the extra plane has at most four planes in all
+        if (a.sp_cells) return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_SPARSE>(a, waves, lds, stream);
+    }
+    if (a.sp_cells) return ELUTQ_ERR_BITS;
     if (a.extra && a.prologue == 0 && !a.residual)
         return launch_gemv_pp<BITS, G64, NSLOT, PAIRED, GEMV_EXTRA>(a, waves, lds, stream);
     if (a.prologue == 0 && !a.residual && !a.extra && !a.defer && a.n_slices_in == 0)      // the plain instances read none of these fields
@@ -663,16 +727,17 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
 static int gemv_launch(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
                        const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
                        size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,
-                       int waves, const float *d_extra, bool lut_int8)
+                       int waves, const float *d_extra, bool lut_int8, const void *d_sp_inline = nullptr)
 {
     int rc = check_shape(K, N, bits, group);
     if (rc != ELUTQ_OK) return rc;
     if (!d_planes || !d_scales || !d_zeros || !d_x || !d_y) return ELUTQ_ERR_NULL;
     const HlqGeo g = hlq_geo(K, N, bits, group);
     LaunchShape sh;
+    // (a block-sparse plane held in its inline form is looked up by the LUT kernels)
     const bool allow_narrow = !(fusion && fusion->d_slices_out) && !lut_int8;
     const bool own_shape = ksplit == 0 && waves == 0;              // the library chooses the launch shape
-    rc = plan_launch(g, bits, ksplit, waves, allow_narrow, sh, lut_int8);
+    rc = plan_launch(g, bits, ksplit, waves, allow_narrow, sh, lut_int8 || d_sp_inline != nullptr);
     if (rc != ELUTQ_OK) return rc;
     if (lut_int8 && (sh.mfma || sh.narrow || fusion || d_extra)) return ELUTQ_ERR_TUNING;
     ksplit = sh.ksplit; waves = sh.waves;
@@ -683,7 +748,7 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
     // Measured on MI355X against the LUT kernel's runs of column blocks with K slices: 8192 x 28672 17.7 against
     // 21.2 us, 14336 x 32768 29.2 against 51.8 us; at K = 4096, where the LUT kernel needs no slices, the two are level
     // (4096 x 128256: 31.0 against 30.6 us) and the LUT kernel stays.
-    const bool wide = g_gemv_engine != ELUTQ_GEMV_ENGINE_LUT && !lut_int8 && !fusion && !d_extra && own_shape &&
+    const bool wide = g_gemv_engine != ELUTQ_GEMV_ENGINE_LUT && !lut_int8 && !fusion && !d_extra && !d_sp_inline && own_shape &&
                       g.K % HLQ_UNIT == 0 && g.ncb > NUM_CU && (g.U > 32 || g_gemv_engine == ELUTQ_GEMV_ENGINE_MFMA);
     if (wide) sh.ksplit = 1;
     ksplit = sh.ksplit;
@@ -701,7 +766,7 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
     a.partial = nullptr; a.counters = nullptr; a.meet_slots = 0;
     a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
     a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr; a.lut_int8 = 0;
-    a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1;
+    a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1; a.sp_cells = nullptr; a.sp_recs = nullptr;
     if (fusion) {
         if (fusion->prologue < 0 || fusion->prologue > 2) return ELUTQ_ERR_TUNING;
         if (fusion->prologue == 1 && !fusion->d_norm_weight) return ELUTQ_ERR_NULL;
@@ -712,6 +777,10 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
     }
     a.extra = (const HLQ_GLOBAL float *)d_extra;
     a.lut_int8 = lut_int8 ? 1 : 0;
+    if (d_sp_inline) {
+        a.sp_cells = (const HLQ_GLOBAL int32_t *)((const unsigned char *)d_sp_inline + HLQ_SP_HEAD_BYTES);
+        a.sp_recs = (const HLQ_GLOBAL unsigned char *)d_sp_inline + hlq_sp_recs_offset(g.ncb, g.U);
+    }
     size_t stage_bytes = 0;
     if (fusion && fusion->n_slices_in != 0) {
         // x arrives as a base vector plus the unsummed K slices of the launch that produced it
@@ -772,6 +841,16 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
 {
     return gemv_launch(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace, workspace_bytes,
                        stream, fusion, ksplit, waves, d_extra, false);
+}
+
+int hlq_gemv_with_inline_sparse(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                                const void *d_sp_inline, const void *d_x, void *d_y, int K, int N, int bits, int group,
+                                void *d_workspace, size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion,
+                                int ksplit, int waves)
+{
+    if (!d_sp_inline) return ELUTQ_ERR_NULL;
+    return gemv_launch(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace, workspace_bytes,
+                       stream, fusion, ksplit, waves, nullptr, false, d_sp_inline);
 }
 
 extern "C" int elutq_hlq_gemv_int8lut_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
@@ -974,7 +1053,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
         }
         a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
         a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr; a.lut_int8 = 0;
-        a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1;
+        a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1; a.sp_cells = nullptr; a.sp_recs = nullptr;
         const int ns = a.spw < depth_of(bits) ? a.spw : depth_of(bits);
         if (ns > nslot) nslot = ns;
         if (mfma) continue;                          // its tile list is made below, over all layers at once

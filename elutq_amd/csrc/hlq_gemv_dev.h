@@ -59,6 +59,10 @@ struct GemvArgs {
     HLQ_GLOBAL unsigned *fault;           // the library's count of meetings that gave up (never null when meet_slots)
     int spin_limit;                       // polls before a waiting wave gives up
     int drop_slice;                       // -1; tests only: this slice leaves without storing its sums, so that the wait runs out
+    // block-sparse extra plane looked up in the tables the tile has built anyway (GEMV_SPARSE instances; hlq_layout.h:
+    // the inline form of a sparse plane): record index per (column block, unit) or -1, and the records
+    const HLQ_GLOBAL int32_t *sp_cells;        // [ncb][U]
+    const HLQ_GLOBAL unsigned char *sp_recs;   // [records][HLQ_SP_REC_BYTES]
 };
 
 // One tile of a grouped launch (many independent GEMVs in one launch): a run of consecutive column blocks of one
@@ -570,7 +574,8 @@ __device__ __forceinline__ void progress_prio(int done, int total)
 //   GEMV_PLAIN  none of them (their fields are not read)
 //   GEMV_EXTRA  plain, plus the fp32 term `extra` added before the output is rounded
 //   GEMV_INT8   plain, with the tables quantized to int8 per group (build_chunk_int8)
-enum { GEMV_FUSED = 0, GEMV_PLAIN = 1, GEMV_EXTRA = 2, GEMV_INT8 = 3 };
+//   GEMV_SPARSE fused, plus the blocks of a block-sparse extra plane looked up in the unit's tables (sp_cells, sp_recs)
+enum { GEMV_FUSED = 0, GEMV_PLAIN = 1, GEMV_EXTRA = 2, GEMV_INT8 = 3, GEMV_SPARSE = 4 };
 
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
 template <int B, int E, typename F>

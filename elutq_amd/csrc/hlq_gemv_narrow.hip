@@ -80,11 +80,14 @@ __device__ __forceinline__ float process_sub_lane(const uint4 &w, uint32_t sc_ra
 
 // grid = ceil(N / 64) * (64 / CW) workgroups of ceil(U / NU) waves; workgroup nb owns columns
 // 64 * (nb / UL) + CW * (nb % UL) + [0, CW) over all of K.
-template <int BITS, bool G64, int CW, int R, bool PLAIN>
+// VAR: GEMV_PLAIN (no prologue, residual or extra term), GEMV_FUSED (as the argument block says), GEMV_SPARSE (fused, plus
+// the blocks of a block-sparse extra plane in its inline form: every lane looks its own unit's record up in that unit's tables).
+template <int BITS, bool G64, int CW, int R, int VAR>
 __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
 {
     using Geo = NarrowGeo<CW, R>;
     constexpr int UL = Geo::UL, NU = Geo::NU, PASSES = Geo::PASSES;
+    constexpr bool PLAIN = VAR == GEMV_PLAIN, SPARSE = VAR == GEMV_SPARSE;
     extern __shared__ __align__(256) unsigned char smem[];
     const int prologue = PLAIN ? 0 : a.prologue;
     const HLQ_GLOBAL uint16_t *residual = PLAIN ? nullptr : a.residual;
@@ -127,6 +130,12 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     for (int p = 0; p < PASSES; p++) {
         load_chunk<PLAIN>(a, prologue, K, (size_t)hlq_narrow_x_chunk(ub, p * 64 + lane, K) * 4, raw[p], raw2[p]);
     }
+    // the record of this lane's unit in every round (-1: no block on its column block and unit), with the activations
+    int cell[R];
+    if constexpr (SPARSE) {
+#pragma unroll
+        for (int r = 0; r < R; r++) cell[r] = a.sp_cells[(size_t)cb * a.U + hlq_narrow_unit(ub, r, UL, ul, a.U)];
+    }
     asm volatile("" ::: "memory");      // the activation loads stay ahead of the weight loads
 
     // every weight load of the wave, unconditional (units past the end re-read the last one)
@@ -162,6 +171,25 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     for (int p = 0; p < PASSES; p++)
         if ((ub * 32 + p * 64 + lane) * 4 >= K) raw[p] = make_uint2(0u, 0u);
 
+    // the records of the units that have blocks: requested before the tables are built, looked up after the dense planes
+    uint4 spw[R];
+    uint32_t spsc[R];
+    bool sp_any[R];
+    if constexpr (SPARSE) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const bool has = cell[r] >= 0 && ub + r * UL + ul < a.U;
+            sp_any[r] = __builtin_amdgcn_ballot_w64(has) != 0;              // wave-uniform
+            spw[r] = make_uint4(0u, 0u, 0u, 0u);
+            spsc[r] = 0u;
+            if (has) {
+                const HLQ_GLOBAL unsigned char *rec = a.sp_recs + (size_t)cell[r] * HLQ_SP_REC_BYTES;
+                const u32x4 v = *(const HLQ_GLOBAL u32x4 *)(rec + (uint32_t)col * 16u);
+                spw[r] = make_uint4(v.x, v.y, v.z, v.w);
+                spsc[r] = *(const HLQ_GLOBAL uint32_t *)(rec + 1024u + (uint32_t)col * 4u);
+            }
+        }
+    }
     // the wave's own tables: chunk ci of the wave belongs to unit ci / 32, half unit ci / 16
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
@@ -182,6 +210,10 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
 #pragma unroll
         for (int b = 0; b < BITS; b++)
             t = process_sub_lane<G64>(w[r][b], sc[r][b], zz[r], base, xs_inv + 2 * lu, b, ul & 1, t);
+        if constexpr (SPARSE) {
+            // lanes without a block look up entry 0 of every table (the empty subset: 0) with scale 0
+            if (sp_any[r]) t = process_sub_lane<true>(spw[r], spsc[r], 0u, base, xs_inv + 2 * lu, 1, 0, t);
+        }
         acc += ub + lu < a.U ? t : 0.f;
     }
 
@@ -202,7 +234,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     }
 }
 
-template <int BITS, bool G64, int CW, int R, bool PLAIN>
+template <int BITS, bool G64, int CW, int R, int VAR>
 int launch_narrow_v(const GemvArgs &a, size_t stage_bytes, hipStream_t stream)
 {
     using Geo = NarrowGeo<CW, R>;
@@ -210,7 +242,7 @@ int launch_narrow_v(const GemvArgs &a, size_t stage_bytes, hipStream_t stream)
     const size_t lds = narrow_lds_bytes<CW, R>(waves) + stage_bytes;
     if (waves < 1 || waves > 16) return ELUTQ_ERR_TUNING;
     if (lds > (size_t)MAX_LDS) return ELUTQ_ERR_SHAPE;
-    auto kern = hlq_gemv_narrow_kernel<BITS, G64, CW, R, PLAIN>;
+    auto kern = hlq_gemv_narrow_kernel<BITS, G64, CW, R, VAR>;
     static bool big_lds_done[64] = {};        // per template instance
     if (lds > 64 * 1024) {
         int dev = 0;
@@ -228,8 +260,12 @@ int launch_narrow_v(const GemvArgs &a, size_t stage_bytes, hipStream_t stream)
 template <int BITS, bool G64, int CW, int R>
 int launch_narrow_r(const GemvArgs &a, size_t stage_bytes, hipStream_t stream)
 {
-    if (a.prologue == 0 && !a.residual && !a.extra) return launch_narrow_v<BITS, G64, CW, R, true>(a, stage_bytes, stream);
-    return launch_narrow_v<BITS, G64, CW, R, false>(a, stage_bytes, stream);
+    if constexpr (BITS <= 3) {        // a layer with the extra plane has at most four planes in all
+        if (a.sp_cells) return launch_narrow_v<BITS, G64, CW, R, GEMV_SPARSE>(a, stage_bytes, stream);
+    }
+    if (a.sp_cells) return ELUTQ_ERR_BITS;
+    if (a.prologue == 0 && !a.residual && !a.extra) return launch_narrow_v<BITS, G64, CW, R, GEMV_PLAIN>(a, stage_bytes, stream);
+    return launch_narrow_v<BITS, G64, CW, R, GEMV_FUSED>(a, stage_bytes, stream);
 }
 
 template <int BITS, bool G64>

@@ -34,6 +34,22 @@
 #define HLQ_GEMM_WAVES 8               /* waves per GEMM workgroup */
 #define HLQ_GEMM_MAX_M 64              /* rows per GEMM launch; more rows run in chunks of this many (weights re-streamed) */
 
+// Inline form of a block-sparse extra plane (blocks of 32 output channels x G inputs on the group grid, at most one per
+// cell): what a GEMV tile needs to look the blocks up in the activation tables it has built for the dense planes.
+//   header   int32 [8]          magic, K, N, group, U, ncb, records, 0
+//   cells    int32 [ncb][U]     record of (column block, unit), or -1             at HLQ_SP_HEAD_BYTES
+//   records  [records][1280 B]  uint4 [64]: lane n's 128 plane bits of the unit, laid out and rotated like a dense plane's,
+//                               zero where n's half of the column block (or, at G = 64, a 64-k half) has no block;
+//                               uint32 [64]: fp16 scales of n for the unit's two 64-k halves (0 where there is no block)
+//                                                                                   at hlq_sp_recs_offset(ncb, U)
+#define HLQ_SP_MAGIC 0x53504c31
+#define HLQ_SP_HEAD_BYTES 32
+#define HLQ_SP_REC_BYTES 1280
+static inline size_t hlq_sp_recs_offset(int ncb, int U)
+{
+    return ((size_t)HLQ_SP_HEAD_BYTES + (size_t)ncb * U * sizeof(int32_t) + 255) & ~(size_t)255;
+}
+
 struct HlqGeo {
     int K, N, bits, group;
     int U;      // units per column

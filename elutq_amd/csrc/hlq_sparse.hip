@@ -22,6 +22,8 @@
 // block is one contiguous 32*G/8-byte read -- and the pair list becomes an index by channel tile.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <string.h>
+#include <vector>
 
 #include "../../include/elutq_hip.h"
 #include "hlq_layout.h"
@@ -458,6 +460,77 @@ int elutq_hlq_sparse_gemv_fused_f16(const void *d_planes, const void *d_scales, 
     if (rc != ELUTQ_OK) return rc;
     return hlq_gemv_with_extra(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace, dense,
                                stream, fusion, ksplit, waves, extra);
+}
+
+// ---- the inline form of a plane: blocks looked up inside the dense GEMV launch ------------------------------------
+size_t elutq_hlq_sparse_inline_bytes(int K, int N, int group, int nblk)
+{
+    if (check_sparse_call(K, N, group, nblk) != ELUTQ_OK) return 0;
+    const HlqGeo g = hlq_geo(K, N, 1, group);
+    return hlq_sp_recs_offset(g.ncb, g.U) + (size_t)nblk * HLQ_SP_REC_BYTES;
+}
+
+int elutq_hlq_sparse_inline_host(const uint32_t *h_mask, int mask_len, const void *h_blocks, const void *h_blk_scales,
+                                 int K, int N, int group, void *h_out, size_t *bytes_used)
+{
+    if (mask_len < 0 || mask_len % 2) return ELUTQ_ERR_SPARSE;
+    const int nblk = mask_len / 2;
+    int rc = check_sparse_call(K, N, group, nblk);
+    if (rc != ELUTQ_OK) return rc;
+    if (!h_out || (nblk && (!h_mask || !h_blocks || !h_blk_scales))) return ELUTQ_ERR_NULL;
+    const HlqGeo g = hlq_geo(K, N, 1, group);
+    const size_t recs_off = hlq_sp_recs_offset(g.ncb, g.U);
+    int32_t *head = (int32_t *)h_out, *cells = (int32_t *)((unsigned char *)h_out + HLQ_SP_HEAD_BYTES);
+    unsigned char *recs = (unsigned char *)h_out + recs_off;
+    memset(h_out, 0, recs_off);
+    for (size_t i = 0; i < (size_t)g.ncb * g.U; i++) cells[i] = -1;
+    std::vector<unsigned char> taken;                 // per record: which (channel half, 64-k half) quarters hold a block
+    const int bpr = group / 8;                        // bytes per channel of a block
+    int nrec = 0;
+    for (int i = 0; i < nblk; i++) {
+        const uint32_t c = h_mask[2 * i], k = h_mask[2 * i + 1];
+        // the inline form needs the blocks on the grid of the quantization groups: anything else keeps the block form
+        if (c % SP_TILE || c >= (uint32_t)N || k % (uint32_t)group || (uint64_t)k + (uint32_t)group > (uint32_t)K)
+            return ELUTQ_ERR_SPARSE;
+        const int cb = (int)(c / HLQ_CB), half = (int)(c / SP_TILE) & 1, u = (int)(k / HLQ_UNIT), g2 = (int)(k % HLQ_UNIT) / 64;
+        int32_t &cell = cells[(size_t)cb * g.U + u];
+        if (cell < 0) {
+            cell = nrec++;
+            memset(recs + (size_t)cell * HLQ_SP_REC_BYTES, 0, HLQ_SP_REC_BYTES);
+            taken.push_back(0);
+        }
+        const unsigned char quarters = group == 128 ? (unsigned char)(3u << (2 * half)) : (unsigned char)(1u << (2 * half + g2));
+        if (taken[cell] & quarters) return ELUTQ_ERR_SPARSE;          // two blocks on one cell
+        taken[cell] |= quarters;
+        uint32_t *w = (uint32_t *)(recs + (size_t)cell * HLQ_SP_REC_BYTES);
+        uint32_t *sc = w + HLQ_CB * 4;
+        for (int r = 0; r < SP_TILE; r++) {
+            const int lane = SP_TILE * half + r;
+            const unsigned char *src = (const unsigned char *)h_blocks + ((size_t)i * SP_TILE + r) * bpr;
+            for (int d = 0; d < bpr / 4; d++) {
+                uint32_t v;
+                memcpy(&v, src + 4 * d, 4);                            // little-endian dword: bit j <-> k = 32 d + j of the block
+                v = (v << HLQ_ROT) | (v >> (32 - HLQ_ROT));
+                w[lane * 4 + (group == 128 ? d : 2 * g2 + d)] = v;
+            }
+            const uint32_t s = ((const uint16_t *)h_blk_scales)[(size_t)i * SP_TILE + r];
+            if (group == 128) sc[lane] = s | (s << 16);
+            else sc[lane] |= s << (16 * g2);
+        }
+    }
+    head[0] = HLQ_SP_MAGIC; head[1] = K; head[2] = N; head[3] = group; head[4] = g.U; head[5] = g.ncb; head[6] = nrec; head[7] = 0;
+    if (bytes_used) *bytes_used = recs_off + (size_t)nrec * HLQ_SP_REC_BYTES;
+    return ELUTQ_OK;
+}
+
+int elutq_hlq_sparse_gemv_inline_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                                     const void *d_inline, const void *d_x, void *d_y, int K, int N, int bits, int group,
+                                     void *d_workspace, size_t workspace_bytes, void *stream,
+                                     const elutq_gemv_fusion *fusion, int ksplit, int waves)
+{
+    if (bits > 3) return ELUTQ_ERR_BITS;              // the extra plane is the layer's fourth at most
+    return hlq_gemv_with_inline_sparse(d_planes, d_scales, d_zeros, d_bias, d_inline, d_x, d_y, K, N, bits, group,
+                                       d_workspace, workspace_bytes, stream, fusion, ksplit, waves);
 }
 
 int elutq_hlq_sparse_gemv_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,

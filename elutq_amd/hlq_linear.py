@@ -77,6 +77,25 @@ def unpack_to_export_arrays(planes, scales, zeros, k: int, n: int, bits: int, gr
     return w_quant, w_scale, w_zero
 
 
+def sparse_inline(mask, blocks, scales, k: int, n: int, group: int) -> np.ndarray | None:
+    """The inline form of a sparse extra plane (elutq_hlq_sparse_inline_host): what the batch-1 GEMV needs to look
+    the blocks up inside its own launch.  None where the block list does not fit that form (blocks off the grid of
+    the quantization groups, or two on one cell): such a plane runs as a launch of its own."""
+    L = _lib.lib()
+    mask = np.ascontiguousarray(mask, dtype=np.uint32).reshape(-1)
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    scales = np.ascontiguousarray(scales, dtype=np.float16)
+    out = np.zeros(L.elutq_hlq_sparse_inline_bytes(k, n, group, mask.size // 2), dtype=np.uint8)
+    used = ctypes.c_size_t(0)
+    vp = ctypes.c_void_p
+    rc = L.elutq_hlq_sparse_inline_host(mask.ctypes.data_as(vp), mask.size, blocks.ctypes.data_as(vp), scales.ctypes.data_as(vp),
+                                        k, n, group, out.ctypes.data_as(vp), ctypes.byref(used))
+    if rc == _lib.ERR_SPARSE:
+        return None
+    _lib.check(rc, "elutq_hlq_sparse_inline_host")
+    return out[:used.value].copy()
+
+
 def sparse_index(mask, k: int, n: int, group: int) -> np.ndarray:
     """(channel start, k start) pairs of a sparse extra plane -> the int32 index the kernels read
     (elutq_hlq_sparse_index_host; raises on a malformed list)."""
@@ -95,6 +114,8 @@ class HLQLinear(nn.Module):
     `sparse`: optional block-sparse extra plane of a ``use_sparse`` export as device tensors
     (blocks uint8 [nblk, 32, G/8], scales fp16 [nblk, 32], index int32 from `sparse_index`);
     `bits` counts the dense planes only, as ``base_bit`` does in the export's json."""
+
+    use_sparse_inline = True    # batch-1 calls look a sparse extra plane up inside the dense launch where its blocks allow it
 
     def __init__(self, in_features: int, out_features: int, bits: int, group_size: int,
                  planes: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor,
@@ -118,6 +139,14 @@ class HLQLinear(nn.Module):
                     or sp_blocks.numel() != self.sparse_count * 32 * self.group_size // 8):
                 raise ValueError("sparse buffers do not match the layer: need blocks uint8 [nblk, 32, G/8], "
                                  "scales fp16 [nblk, 32] and the int32 index of sparse_index()")
+        # the inline form of the plane, where its blocks fit it: batch-1 calls then take one launch (the blocks are
+        # looked up in the dense GEMV's own tables) instead of two; `use_sparse_inline = False` keeps the two launches
+        self.register_buffer("sparse_inline", None)
+        if self.sparse_count and self.bits <= 3:
+            form = sparse_inline(self.sparse_pairs(), sp_blocks.cpu().numpy(), sp_scales.cpu().numpy(), self.in_features,
+                                 self.out_features, self.group_size)
+            if form is not None:
+                self.sparse_inline = torch.from_numpy(form).to(sp_blocks.device)
         self._ws_bytes = _lib.lib().elutq_hlq_workspace_bytes(self.in_features, self.out_features,
                                                               self.bits, self.group_size, 1)
         if self._ws_bytes == 0:
@@ -250,7 +279,13 @@ class HLQLinear(nn.Module):
             ws = _workspace(x.device, need)
             stream = torch.cuda.current_stream(x.device).cuda_stream
             bias = self.bias.data_ptr() if self.bias is not None else None
-            if self.sparse_count:
+            if m == 1 and self._inline():
+                rc = L.elutq_hlq_sparse_gemv_inline_f16(self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
+                                                        bias, self.sparse_inline.data_ptr(), x2.data_ptr(), y.data_ptr(),
+                                                        self.in_features, self.out_features, self.bits, self.group_size,
+                                                        ws.data_ptr(), ws.numel(), stream, None, self.ksplit, self.waves)
+                _lib.check(rc, "elutq_hlq_sparse_gemv_inline_f16")
+            elif self.sparse_count:
                 rc = L.elutq_hlq_sparse_gemm_f16(self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
                                                  bias, self.sparse_blocks.data_ptr(), self.sparse_scales.data_ptr(),
                                                  self.sparse_index.data_ptr(), self.sparse_count, x2.data_ptr(),
@@ -271,6 +306,16 @@ class HLQLinear(nn.Module):
                 _lib.check(rc, "elutq_hlq_gemm_f16")
         y = y.reshape(*x.shape[:-1], self.out_features)
         return y if in_dtype == torch.float16 else y.to(in_dtype)
+
+    def _inline(self) -> bool:
+        """Whether batch-1 calls look the sparse extra plane up inside the dense launch."""
+        return bool(self.sparse_count) and self.sparse_inline is not None and self.use_sparse_inline
+
+    @property
+    def sparse_own_launch(self) -> bool:
+        """A sparse extra plane that runs as a launch of its own in front of the dense one (such a layer neither
+        takes nor leaves K slices)."""
+        return bool(self.sparse_count) and not self._inline()
 
     def gemv_int8lut(self, x: torch.Tensor) -> torch.Tensor:
         """Batch-1 GEMV with the lookup tables quantized to int8 per group, as the reference's int8-LUT variant
@@ -305,8 +350,8 @@ class HLQLinear(nn.Module):
         A layer with a sparse extra plane held as blocks takes two launches (the plane's fp32 term with
         the same prologue, then the dense kernel, elutq_hlq_sparse_gemv_fused_f16), `ws` of
         self.workspace_bytes, and no slices in either direction."""
-        if self.sparse_count and (slices_out is not None or slices_in is not None):
-            raise ValueError("a layer with a sparse extra plane held as blocks neither takes nor leaves K slices")
+        if self.sparse_count and not self._inline() and (slices_out is not None or slices_in is not None):
+            raise ValueError("a layer whose sparse extra plane runs as a launch of its own neither takes nor leaves K slices")
         f = _lib.GemvFusion(prologue, eps, norm_weight.data_ptr() if norm_weight is not None else None,
                             residual.data_ptr() if residual is not None else None,
                             slices_out.data_ptr() if slices_out is not None else None,
@@ -320,6 +365,14 @@ class HLQLinear(nn.Module):
         if slices_in is not None and (slices_in.dtype != torch.float32 or slices_in.dim() != 2
                                       or slices_in.shape[1] != self.in_features or not slices_in.is_contiguous()):
             raise ValueError("slices_in must be contiguous fp32 [S, in_features]")
+        if self._inline():
+            rc = _lib.lib().elutq_hlq_sparse_gemv_inline_f16(
+                self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
+                self.bias.data_ptr() if self.bias is not None else None, self.sparse_inline.data_ptr(), x.data_ptr(),
+                out.data_ptr(), self.in_features, self.out_features, self.bits, self.group_size, ws.data_ptr(), ws.numel(),
+                torch.cuda.current_stream(x.device).cuda_stream, ctypes.byref(f), self.ksplit, self.waves)
+            _lib.check(rc, "elutq_hlq_sparse_gemv_inline_f16")
+            return out
         if self.sparse_count:
             rc = _lib.lib().elutq_hlq_sparse_gemv_fused_f16(
                 self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),

@@ -150,7 +150,7 @@ def deferred_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tenso
     s = layer.s
     n_q = layer.qkv.slices
     defer_qkv = (defer_qkv and s.head_dim == 128 and 2 <= n_q <= MAX_DEFERRED_SLICES and layer.qkv.bias is None
-                 and not layer.qkv.sparse_count)
+                 and not layer.qkv.sparse_own_launch)
     layer.qkv.gemv_fused(cur, b.qkv, b.ws, prologue=1, norm_weight=layer.ln1, eps=s.rms_eps,
                          slices_in=b.sd[:pending] if pending else None, x_out=other if pending else None,
                          slices_out=b.sq if defer_qkv else None)
@@ -173,7 +173,7 @@ def deferred_layer_step(layer: "DecoderLayer", b: FusedBuffers, pos: torch.Tenso
     cur, other = other, cur
     n_d = layer.down_proj.slices
     if (not last and defer_down and 2 <= n_d <= MAX_DEFERRED_SLICES and layer.down_proj.bias is None
-            and not layer.down_proj.sparse_count):
+            and not layer.down_proj.sparse_own_launch):
         layer.down_proj.gemv_fused(b.gu, other, b.ws, prologue=2, slices_out=b.sd)
         return cur, other, n_d
     layer.down_proj.gemv_fused(b.gu, other, b.ws, prologue=2, residual=cur)
@@ -316,7 +316,7 @@ class LlamaDecoder(nn.Module):
             if self.defer_qkv:
                 for layer in self.layers:
                     q = layer.qkv
-                    if q.sparse_count:
+                    if q.sparse_own_launch:
                         continue                         # its plane's launch reads the stored input: no slices
                     if q.bias is None and q.slices == 1 and 2 * ((q.out_features + 63) // 64) <= 256:
                         q.ksplit, q.waves = 2, 16
@@ -326,7 +326,7 @@ class LlamaDecoder(nn.Module):
             # with more tiles than compute units, or tables that leave no room for the staged activations,
             # does not): decided here, once, so that a step never meets a refusing launch
             self._defer_down = [i + 1 < len(self.layers) and 2 <= layer.down_proj.slices <= MAX_DEFERRED_SLICES
-                                and not layer.down_proj.sparse_count and not self.layers[i + 1].qkv.sparse_count
+                                and not layer.down_proj.sparse_own_launch and not self.layers[i + 1].qkv.sparse_own_launch
                                 and self.layers[i + 1].qkv.accepts_slices(layer.down_proj.slices)
                                 for i, layer in enumerate(self.layers)]
             # a launch that leaves its K slices to the next one runs on the wide-tile kernel: a down that may do so

@@ -422,6 +422,18 @@ int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void
  * llama.cpp:204-617).  The plane's launch forms the projection's input from the same stored vectors
  * with the same operations as the dense launch's prologue.  K slices handed over by, or left to,
  * another launch (d_slices_in / d_slices_out) are refused: ELUTQ_ERR_TUNING.
+ *
+ * The inline form -- one launch per layer.  Where every block lies on the grid of the quantization groups (k start a
+ * multiple of `group`) and no two blocks share a cell, the batch-1 GEMV can look the blocks up in the activation tables
+ * it builds for the dense planes anyway, as t_mac_g4_float_update_sparse_impl (arm_t_mac_kernal.cpp:678-788) looks
+ * them up in the LUT of the dense update.  elutq_hlq_sparse_inline_host writes that form (per (column block, unit) a
+ * record number, per record the 64 lanes' plane bits in the dense planes' layout and their fp16 scales) into h_out,
+ * elutq_hlq_sparse_inline_bytes(K, N, group, nblk) bytes at most, *bytes_used of them used (may be NULL); copy it to
+ * the device unchanged.  ELUTQ_ERR_SPARSE for a block list the form cannot hold (off the grid, repeated, malformed):
+ * such a layer keeps the two-launch entry points above.  elutq_hlq_sparse_gemv_inline_f16 is elutq_hlq_gemv_fused_f16
+ * (fusion may be NULL; prologues, residual, K slices handed over or left to the next launch as there) on such a layer,
+ * `bits` = base_bit <= 3, on the table-lookup kernels (wide or narrow tiles as for a dense layer); the workspace is that of the dense layer.  The
+ * result is the dense fp32 sum plus the blocks' terms, rounded once.
  */
 size_t elutq_hlq_sparse_index_bytes(int N, int nblk);
 int elutq_hlq_sparse_index_host(const uint32_t *h_mask, int mask_len, int K, int N, int group, void *h_index_out);
@@ -441,6 +453,13 @@ int elutq_hlq_sparse_gemv_fused_f16(const void *d_planes, const void *d_scales, 
                                     const elutq_gemv_fusion *fusion, int ksplit, int waves);
 int elutq_hlq_sparse_dequant_add_f16(const void *d_blocks, const void *d_blk_scales, const void *d_index, int nblk,
                                      void *d_w, int K, int N, int group, void *stream);
+size_t elutq_hlq_sparse_inline_bytes(int K, int N, int group, int nblk);
+int elutq_hlq_sparse_inline_host(const uint32_t *h_mask, int mask_len, const void *h_blocks, const void *h_blk_scales,
+                                 int K, int N, int group, void *h_out, size_t *bytes_used);
+int elutq_hlq_sparse_gemv_inline_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
+                                     const void *d_inline, const void *d_x, void *d_y, int K, int N, int bits, int group,
+                                     void *d_workspace, size_t workspace_bytes, void *stream,
+                                     const elutq_gemv_fusion *fusion, int ksplit, int waves);
 
 #ifdef __cplusplus
 }

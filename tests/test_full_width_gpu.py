@@ -126,3 +126,39 @@ def test_decode_step_at_full_llama3_8b_width(cuda):
         assert (a.v_cache[512:516].float() - b.v_cache[512:516].float()).abs().max() <= 2e-2
     for a, b in zip(hip.layers, graph.layers):
         assert torch.equal(a.k_cache, b.k_cache) and torch.equal(a.v_cache, b.v_cache)
+
+
+def test_the_32_layer_step_the_benchmark_times(cuda):
+    """The decode configuration itself: 32 layers at the LLaMA-3-8B shape, 512-token cache, one HIP graph per
+    token (what `bench.py` times) against eager steps of the same fused path, bit for bit, and against the same
+    HLQ model under PyTorch glue -- every projection through the C ABI one call at a time, norms, RoPE, attention
+    and residual adds as PyTorch operators in fp32 -- to within 3e-2 of the logits' rms after 32 layers."""
+    shape = LlamaShape(n_layers=32, hidden=4096, n_heads=32, n_kv_heads=8, ffn=14336, vocab=128256, max_seq=640)
+    print("32-layer decode step: building models", flush=True)
+    graph = LlamaDecoder(shape, device=cuda, seed=11)
+    eager = LlamaDecoder(shape, device=cuda, seed=11)
+    glue = TorchGlueDecoder(shape, device=cuda, seed=11)
+    for m in (graph, eager, glue):
+        m.fill_cache(512, seed=3)
+        m.token.fill_(77)
+    graph.capture()
+    worst = 0.0
+    for step in range(3):
+        print(f"32-layer decode step: step {step}", flush=True)
+        le = eager.step().float()
+        lg = glue.step().float()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(graph._logits.float(), le), step
+        assert int(graph.token) == int(eager.token) and int(graph.pos) == 513 + step
+        assert torch.isfinite(le).all()
+        d = float((le - lg).abs().max() / lg.pow(2).mean().sqrt())
+        worst = max(worst, d)
+        assert d <= 3e-2, (step, d)
+        # the greedy pick of the fused path is among the glue path's best few (random weights give near ties)
+        assert int(eager.token) in torch.topk(lg.flatten(), 5).indices.tolist(), step
+        glue.token.copy_(eager.token)
+    print(f"32-layer decode step: fused - glue, max over logits / rms = {worst:.3e}", flush=True)
+    for a, b in zip(eager.layers, graph.layers):
+        assert torch.equal(a.k_cache, b.k_cache) and torch.equal(a.v_cache, b.v_cache)

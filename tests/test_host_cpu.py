@@ -202,3 +202,56 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout == ""
+
+
+@pytest.mark.parametrize("k,n,group", [(512, 128, 128), (768, 96, 64), (448, 64, 64), (1024, 100, 128)])
+def test_sparse_inline_form_holds_every_block_where_the_kernel_looks(k, n, group):
+    """elutq_hlq_sparse_inline_host against a bit-by-bit reconstruction: per (column block, unit) a record, in it lane n's
+    plane bits at the dense planes' positions (dword d = k 32d..32d+31 of the unit, rotated left by 2) and the fp16
+    scales of the unit's two 64-k halves; zero wherever no block lies."""
+    from elutq_amd.hlq_linear import sparse_inline
+    from elutq_amd.synth import make_sparse_plane, pack_bits_lsb_first
+    npad = (n + 31) // 32 * 32
+    bits, scale, mask = make_sparse_plane(k // group * group, npad, group, 0.4, seed=k + n)
+    keep = mask[:, 0] < n
+    bits, scale, mask = bits[keep], scale[keep], mask[keep]
+    form = sparse_inline(mask, pack_bits_lsb_first(bits), scale, k, n, group)
+    assert form is not None
+    U, ncb = (k + 127) // 128, (n + 63) // 64
+    head = form[:32].view(np.int32)
+    assert head[0] == 0x53504c31 and list(head[1:6]) == [k, n, group, U, ncb]
+    cells = form[32:32 + 4 * ncb * U].view(np.int32).reshape(ncb, U)
+    recs_off = (32 + 4 * ncb * U + 255) // 256 * 256
+    nrec = int(head[6])
+    assert form.size == recs_off + 1280 * nrec
+    recs = form[recs_off:].reshape(nrec, 1280)
+    # the plane as a dense [npad64, U * 128] bit matrix and a per-(channel, 64-k half) scale matrix
+    want_bits = np.zeros((ncb * 64, U * 128), np.uint8)
+    want_scale = np.zeros((ncb * 64, U * 2), np.float16)
+    for b, s, (c, k0) in zip(bits, scale, mask):
+        want_bits[c:c + 32, k0:k0 + group] = b
+        for h in range(k0 // 64, (k0 + group) // 64):
+            want_scale[c:c + 32, h] = s
+    used = set()
+    for cb in range(ncb):
+        for u in range(U):
+            blk = want_bits[64 * cb:64 * cb + 64, 128 * u:128 * u + 128]
+            sc = want_scale[64 * cb:64 * cb + 64, 2 * u:2 * u + 2]
+            c = cells[cb, u]
+            if c < 0:
+                assert not blk.any() and not sc.any()
+                continue
+            assert 0 <= c < nrec and c not in used
+            used.add(int(c))
+            w = recs[c, :1024].view(np.uint32).reshape(64, 4)
+            w = (w >> 2) | (w << 30)                                    # rotation undone
+            got = ((w[:, :, None] >> np.arange(32, dtype=np.uint32)) & 1).astype(np.uint8).reshape(64, 128)
+            assert np.array_equal(got, blk)
+            got_sc = recs[c, 1024:].view(np.float16).reshape(64, 2)
+            assert np.array_equal(got_sc, sc)
+    assert len(used) == nrec
+    # what the form cannot hold comes back as None: a block off the grid of the groups, two blocks on one cell
+    one = pack_bits_lsb_first(bits[:1])
+    assert sparse_inline(np.array([[0, 4]], np.uint32), one, scale[:1], k, n, group) is None
+    two = pack_bits_lsb_first(bits[[0, 0]])
+    assert sparse_inline(np.array([[0, 0], [0, 0]], np.uint32), two, scale[[0, 0]], k, n, group) is None

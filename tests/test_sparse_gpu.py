@@ -21,6 +21,14 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
+@pytest.fixture(params=["inline", "own_launch"], autouse=True)
+def plane_launch(request, monkeypatch):
+    """Every test runs twice: with the plane's blocks looked up inside the dense batch-1 launch (where the block list
+    fits the inline form and the layer has at most three dense planes), and with the plane as a launch of its own."""
+    monkeypatch.setattr(HLQLinear, "use_sparse_inline", request.param == "inline")
+    return request.param
+
+
 def build(k, n, bits, group, density, seed, dev, m=1, bias=True, mode="blocks"):
     """mode "blocks": the plane in its file form (the block kernels); "dense": written out as one more plane."""
     L = make_layer(k, n, bits, group, m=m, seed=seed, bias=bias)
@@ -226,7 +234,7 @@ FUSED_SHAPES = [(4096, 64, 2, 64, 1.0), (1024, 256, 2, 128, 0.3), (512, 96, 3, 6
 @pytest.mark.parametrize("k,n,bits,group,density", FUSED_SHAPES)
 @pytest.mark.parametrize("ksplit,waves", [(0, 0), (1, 4), (2, 16), (_lib.GEMV_NARROW16, 0), (_lib.GEMV_NARROW32, 0),
                                           (_lib.GEMV_WIDE, 0)])
-def test_fused_rmsnorm_prologue_and_residual(cuda, k, n, bits, group, density, ksplit, waves):
+def test_fused_rmsnorm_prologue_and_residual(cuda, plane_launch, k, n, bits, group, density, ksplit, waves):
     """The layer inside a decode step: RMSNorm in front (formed by both launches, the plane's and the dense one's),
     bias, the plane's fp32 term and the residual behind, one rounding."""
     L, sp, mod, g, res, out, ws = _fused_case(k, n, bits, group, density, k + n + 3, cuda)
@@ -258,7 +266,7 @@ def test_fused_rmsnorm_prologue_and_residual(cuda, k, n, bits, group, density, k
 @pytest.mark.parametrize("k,n,bits,group,density", [(1024, 256, 2, 128, 0.3), (1536, 192, 4, 64, 0.2), (960, 96, 2, 64, 0.5),
                                                      (14336, 4096, 2, 128, 0.02)])
 @pytest.mark.parametrize("ksplit", [0, _lib.GEMV_NARROW32, _lib.GEMV_WIDE])
-def test_fused_silu_mul_prologue(cuda, k, n, bits, group, density, ksplit):
+def test_fused_silu_mul_prologue(cuda, plane_launch, k, n, bits, group, density, ksplit):
     import torch.nn.functional as F
     if ksplit == _lib.GEMV_NARROW32 and k > 8192:
         pytest.skip("the narrow-tile kernel holds the tables of at most 8192 activations")
@@ -324,7 +332,9 @@ def test_fused_integer_inputs_bit_exact(cuda):
     assert np.array_equal(out.cpu().numpy().astype(np.float64), want)
 
 
-def test_fused_refuses_slices_and_group_refuses_sparse(cuda):
+def test_fused_refuses_slices_and_group_refuses_sparse(cuda, plane_launch):
+    if plane_launch == "inline":
+        pytest.skip("a plane looked up inside the dense launch takes part in handed-over slices: test_inline_*")
     L, sp, mod = build(256, 64, 2, 128, 0.5, 81, cuda)
     x = torch.from_numpy(L.x).to(cuda)
     out = torch.empty(1, 64, dtype=torch.float16, device=cuda)
@@ -338,3 +348,74 @@ def test_fused_refuses_slices_and_group_refuses_sparse(cuda):
         mod.gemv_fused(x, out, ws[:mod._ws_bytes])
     with pytest.raises(NotImplementedError):
         GemvGroup([mod], [x], [out])
+
+
+# ---- the inline form: blocks looked up inside the dense launch ---------------------------------------------------------
+
+def test_inline_form_exists_where_the_blocks_allow_it(cuda, plane_launch):
+    L, sp, mod = build(512, 128, 2, 128, 0.3, 5, cuda)
+    assert mod.sparse_inline is not None
+    four = build(384, 96, 4, 128, 0.5, 6, cuda)[2]                       # the plane would be a fifth: no instance
+    assert four.sparse_inline is None
+    # off the grid of the groups / two blocks on one cell: the form cannot hold them, the layer keeps its own launch
+    k, n, group = 384, 64, 64
+    L2 = make_layer(k, n, 2, group, seed=41)
+    r = np.random.default_rng(1)
+    for mk in (np.array([[0, 4]], np.uint32), np.array([[0, 64], [0, 64]], np.uint32)):
+        b = r.integers(0, 2, (len(mk), 32, group), dtype=np.uint8)
+        s = r.uniform(0.02, 0.08, (len(mk), 32)).astype(np.float16)
+        m2 = HLQLinear.from_export_arrays(L2.w_quant, L2.w_scale, L2.w_zero, group, None, cuda,
+                                          SparseBlocks(O.SparsePlane(b, s, mk, group).packed, s, mk), sparse_mode="blocks")
+        assert m2.sparse_count == len(mk) and m2.sparse_inline is None
+        y = run(m2, L2.x, cuda)[0]
+        assert O.rel_err(y, O.gemv_sparse_f64(L2.x[0], L2.w_quant, L2.w_scale, L2.w_zero, O.SparsePlane(b, s, mk, group))) <= TOL
+
+
+@pytest.mark.parametrize("k,n,bits,group,density", [(512, 128, 2, 128, 0.3), (1024, 256, 3, 64, 0.2), (4096, 4096, 2, 128, 0.1),
+                                                     (14336, 4096, 2, 128, 0.1), (4096, 14336, 2, 64, 0.1), (8128, 192, 1, 64, 0.5)])
+def test_inline_and_own_launch_agree(cuda, monkeypatch, k, n, bits, group, density):
+    """The two ways of running the plane add the same terms in fp32 before the one rounding: results within one fp16
+    step of each other, and both within the oracle's bar."""
+    L, sp, mod = build(k, n, bits, group, density, k + n + 9, cuda, bias=False)
+    assert mod.sparse_inline is not None
+    monkeypatch.setattr(HLQLinear, "use_sparse_inline", True)
+    yi = run(mod, L.x, cuda)[0]
+    monkeypatch.setattr(HLQLinear, "use_sparse_inline", False)
+    yo = run(mod, L.x, cuda)[0]
+    ref = O.gemv_sparse_f64(L.x[0], L.w_quant, L.w_scale, L.w_zero, sp)
+    assert O.rel_err(yi, ref) <= TOL and O.rel_err(yo, ref) <= TOL
+    assert np.max(np.abs(yi.astype(np.float64) - yo.astype(np.float64))) <= 2.0 ** -9 * max(1.0, np.max(np.abs(ref)))
+
+
+def test_inline_plane_with_handed_over_slices(cuda, monkeypatch):
+    """down -> q|k|v of a decode step with a plane on both layers: the producer leaves its K slices unsummed (the
+    blocks' terms are part of each slice's sum), the consumer adds them up in its RMSNorm prologue."""
+    monkeypatch.setattr(HLQLinear, "use_sparse_inline", True)
+    kd, hid, nq = 14336, 4096, 6144
+    Ld, spd, down = build(kd, hid, 2, 128, 0.05, 301, cuda, bias=False)
+    Lq, spq, qkv = build(hid, nq, 2, 128, 0.1, 302, cuda, bias=False)
+    down.ksplit = _lib.GEMV_WIDE
+    qkv.ksplit, qkv.waves = 2, 16
+    g = torch.Generator(device=cuda).manual_seed(7)
+    gu = torch.randn(1, 2 * kd, generator=g, device=cuda).half()
+    res = torch.randn(1, hid, generator=g, device=cuda).half()
+    w = (1 + 0.1 * torch.randn(hid, generator=g, device=cuda)).half()
+    ws = torch.zeros(max(down.workspace_bytes, qkv.workspace_bytes), dtype=torch.uint8, device=cuda)
+    # the producer summing for itself
+    x1 = torch.empty(1, hid, dtype=torch.float16, device=cuda)
+    down.gemv_fused(gu, x1, ws, prologue=2, residual=res)
+    y1 = torch.empty(1, nq, dtype=torch.float16, device=cuda)
+    qkv.gemv_fused(x1, y1, ws, prologue=1, norm_weight=w, eps=1e-5)
+    # the slices handed over
+    assert down.slices >= 2
+    sl = torch.zeros(down.slices, hid, dtype=torch.float32, device=cuda)
+    dummy = torch.empty(1, hid, dtype=torch.float16, device=cuda)
+    down.gemv_fused(gu, dummy, ws, prologue=2, slices_out=sl)
+    y2 = torch.empty(1, nq, dtype=torch.float16, device=cuda)
+    x2 = torch.empty(1, hid, dtype=torch.float16, device=cuda)
+    qkv.gemv_fused(res, y2, ws, prologue=1, norm_weight=w, eps=1e-5, slices_in=sl, x_out=x2)
+    assert torch.equal(x1, x2) and torch.equal(y1, y2)
+    import torch.nn.functional as F
+    act = (F.silu(gu[:, :kd].float()) * gu[:, kd:].float()).half()
+    ref = O.gemv_sparse_f64(act.cpu().numpy()[0], Ld.w_quant, Ld.w_scale, Ld.w_zero, spd) + res.cpu().numpy()[0].astype(np.float64)
+    assert O.rel_err(x1.cpu().numpy()[0], ref) <= TOL
