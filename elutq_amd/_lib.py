@@ -61,7 +61,7 @@ SIGNATURES = {
     "elutq_hlq_sparse_dequant_add_f16": (_ci, [_vp] * 3 + [_ci, _vp] + [_ci] * 3 + [_vp]),
     "elutq_hlq_sparse_inline_bytes": (_sz, [_ci] * 4),
     "elutq_hlq_sparse_inline_host": (_ci, [_vp, _ci, _vp, _vp, _ci, _ci, _ci, _vp, _vp]),
-    "elutq_hlq_sparse_gemv_inline_f16": (_ci, [_vp] * 7 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
+    "elutq_hlq_sparse_gemv_inline_f16": (_ci, [_vp] * 5 + [_sz] + [_vp] * 2 + [_ci] * 4 + [_vp, _sz, _vp, _vp, _ci, _ci]),
 }
 
 

@@ -137,6 +137,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             cell[j] = sown[j] ? __builtin_amdgcn_readfirstlane(cell[j]) : -1;
+            if (cell[j] >= a.sp_nrec) cell[j] = -1;
             if (cell[j] >= 0) {                                            // wave-uniform
                 const HLQ_GLOBAL unsigned char *r = a.sp_recs + (size_t)cell[j] * HLQ_SP_REC_BYTES;
                 const u32x4 v = __builtin_nontemporal_load((const HLQ_GLOBAL u32x4 *)(r + (uint32_t)lane * 16u));
@@ -271,7 +272,7 @@ __device__ __forceinline__ void gemv_tile(const GemvArgs &a, int cb, int slice, 
         for (int j = 2; j < nuw; j++) {
             if (!(s_begin <= (ub + j) * BITS && (ub + j) * BITS < s_end)) continue;
             const int cj = __builtin_amdgcn_readfirstlane(a.sp_cells[(size_t)cbx * a.U + u0 + ub + j]);
-            if (cj < 0) continue;
+            if (cj < 0 || cj >= a.sp_nrec) continue;
             const HLQ_GLOBAL unsigned char *r = a.sp_recs + (size_t)cj * HLQ_SP_REC_BYTES;
             const u32x4 v = *(const HLQ_GLOBAL u32x4 *)(r + (uint32_t)lane * 16u);
             const uint32_t scj = *(const HLQ_GLOBAL uint32_t *)(r + 1024u + (uint32_t)lane * 4u);
@@ -727,7 +728,7 @@ int elutq_hlq_gemv_fused_f16(const void *d_planes, const void *d_scales, const v
 static int gemv_launch(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
                        const void *d_x, void *d_y, int K, int N, int bits, int group, void *d_workspace,
                        size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion, int ksplit,
-                       int waves, const float *d_extra, bool lut_int8, const void *d_sp_inline = nullptr)
+                       int waves, const float *d_extra, bool lut_int8, const void *d_sp_inline = nullptr, size_t sp_inline_bytes = 0)
 {
     int rc = check_shape(K, N, bits, group);
     if (rc != ELUTQ_OK) return rc;
@@ -766,7 +767,7 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
     a.partial = nullptr; a.counters = nullptr; a.meet_slots = 0;
     a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
     a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr; a.lut_int8 = 0;
-    a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1; a.sp_cells = nullptr; a.sp_recs = nullptr;
+    a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1; a.sp_cells = nullptr; a.sp_recs = nullptr; a.sp_nrec = 0;
     if (fusion) {
         if (fusion->prologue < 0 || fusion->prologue > 2) return ELUTQ_ERR_TUNING;
         if (fusion->prologue == 1 && !fusion->d_norm_weight) return ELUTQ_ERR_NULL;
@@ -778,8 +779,14 @@ static int gemv_launch(const void *d_planes, const void *d_scales, const void *d
     a.extra = (const HLQ_GLOBAL float *)d_extra;
     a.lut_int8 = lut_int8 ? 1 : 0;
     if (d_sp_inline) {
+        // the form's size is the caller's word for how many records lie behind the cell table: a record number beyond
+        // them is treated as "no block", and a buffer too small for the layer's cell table is refused
+        const size_t recs_off = hlq_sp_recs_offset(g.ncb, g.U);
+        if (sp_inline_bytes < recs_off) return ELUTQ_ERR_WORKSPACE;
         a.sp_cells = (const HLQ_GLOBAL int32_t *)((const unsigned char *)d_sp_inline + HLQ_SP_HEAD_BYTES);
-        a.sp_recs = (const HLQ_GLOBAL unsigned char *)d_sp_inline + hlq_sp_recs_offset(g.ncb, g.U);
+        a.sp_recs = (const HLQ_GLOBAL unsigned char *)d_sp_inline + recs_off;
+        const size_t nrec = (sp_inline_bytes - recs_off) / HLQ_SP_REC_BYTES;
+        a.sp_nrec = nrec > 0x7fffffffu ? 0x7fffffff : (int)nrec;
     }
     size_t stage_bytes = 0;
     if (fusion && fusion->n_slices_in != 0) {
@@ -844,13 +851,13 @@ int hlq_gemv_with_extra(const void *d_planes, const void *d_scales, const void *
 }
 
 int hlq_gemv_with_inline_sparse(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
-                                const void *d_sp_inline, const void *d_x, void *d_y, int K, int N, int bits, int group,
+                                const void *d_sp_inline, size_t sp_inline_bytes, const void *d_x, void *d_y, int K, int N, int bits, int group,
                                 void *d_workspace, size_t workspace_bytes, void *stream, const elutq_gemv_fusion *fusion,
                                 int ksplit, int waves)
 {
     if (!d_sp_inline) return ELUTQ_ERR_NULL;
     return gemv_launch(d_planes, d_scales, d_zeros, d_bias, d_x, d_y, K, N, bits, group, d_workspace, workspace_bytes,
-                       stream, fusion, ksplit, waves, nullptr, false, d_sp_inline);
+                       stream, fusion, ksplit, waves, nullptr, false, d_sp_inline, sp_inline_bytes);
 }
 
 extern "C" int elutq_hlq_gemv_int8lut_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
@@ -1053,7 +1060,7 @@ int elutq_hlq_gemv_group_create(const elutq_gemv_problem *problems, int count, i
         }
         a.prologue = 0; a.eps = 0.f; a.norm_w = nullptr; a.residual = nullptr; a.extra = nullptr;
         a.defer = 0; a.n_slices_in = 0; a.slices_in = nullptr; a.x_out = nullptr; a.lut_int8 = 0;
-        a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1; a.sp_cells = nullptr; a.sp_recs = nullptr;
+        a.fault = nullptr; a.spin_limit = SLICE_SPIN_LIMIT; a.drop_slice = -1; a.sp_cells = nullptr; a.sp_recs = nullptr; a.sp_nrec = 0;
         const int ns = a.spw < depth_of(bits) ? a.spw : depth_of(bits);
         if (ns > nslot) nslot = ns;
         if (mfma) continue;                          // its tile list is made below, over all layers at once

@@ -63,6 +63,7 @@ struct GemvArgs {
     // the inline form of a sparse plane): record index per (column block, unit) or -1, and the records
     const HLQ_GLOBAL int32_t *sp_cells;        // [ncb][U]
     const HLQ_GLOBAL unsigned char *sp_recs;   // [records][HLQ_SP_REC_BYTES]
+    int sp_nrec;                               // records behind sp_recs: a number outside [0, sp_nrec) counts as "no block"
 };
 
 // One tile of a grouped launch (many independent GEMVs in one launch): a run of consecutive column blocks of one

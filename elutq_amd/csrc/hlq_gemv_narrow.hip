@@ -178,7 +178,7 @@ __global__ __launch_bounds__(1024) void hlq_gemv_narrow_kernel(const GemvArgs a)
     if constexpr (SPARSE) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const bool has = cell[r] >= 0 && ub + r * UL + ul < a.U;
+            const bool has = cell[r] >= 0 && cell[r] < a.sp_nrec && ub + r * UL + ul < a.U;
             sp_any[r] = __builtin_amdgcn_ballot_w64(has) != 0;              // wave-uniform
             spw[r] = make_uint4(0u, 0u, 0u, 0u);
             spsc[r] = 0u;

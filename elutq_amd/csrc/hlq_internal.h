@@ -16,9 +16,9 @@ HLQ_INTERNAL int hlq_gemv_with_extra(const void *d_planes, const void *d_scales,
                                      int waves, const float *d_extra);
 
 // elutq_hlq_gemv_fused_f16 on a layer whose block-sparse extra plane is held in its inline form (hlq_layout.h) on the
-// device: one launch of the wide-tile LUT kernel, which looks the blocks up in the tables it has built.
+// device (`sp_inline_bytes` of it): one launch of a LUT kernel, which looks the blocks up in the tables it has built.
 HLQ_INTERNAL int hlq_gemv_with_inline_sparse(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
-                                             const void *d_sp_inline, const void *d_x, void *d_y, int K, int N, int bits,
+                                             const void *d_sp_inline, size_t sp_inline_bytes, const void *d_x, void *d_y, int K, int N, int bits,
                                              int group, void *d_workspace, size_t workspace_bytes, void *stream,
                                              const elutq_gemv_fusion *fusion, int ksplit, int waves);
 

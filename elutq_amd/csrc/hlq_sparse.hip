@@ -524,12 +524,12 @@ int elutq_hlq_sparse_inline_host(const uint32_t *h_mask, int mask_len, const voi
 }
 
 int elutq_hlq_sparse_gemv_inline_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
-                                     const void *d_inline, const void *d_x, void *d_y, int K, int N, int bits, int group,
-                                     void *d_workspace, size_t workspace_bytes, void *stream,
+                                     const void *d_inline, size_t inline_bytes, const void *d_x, void *d_y, int K, int N,
+                                     int bits, int group, void *d_workspace, size_t workspace_bytes, void *stream,
                                      const elutq_gemv_fusion *fusion, int ksplit, int waves)
 {
     if (bits > 3) return ELUTQ_ERR_BITS;              // the extra plane is the layer's fourth at most
-    return hlq_gemv_with_inline_sparse(d_planes, d_scales, d_zeros, d_bias, d_inline, d_x, d_y, K, N, bits, group,
+    return hlq_gemv_with_inline_sparse(d_planes, d_scales, d_zeros, d_bias, d_inline, inline_bytes, d_x, d_y, K, N, bits, group,
                                        d_workspace, workspace_bytes, stream, fusion, ksplit, waves);
 }
 

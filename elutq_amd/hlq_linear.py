@@ -281,7 +281,7 @@ class HLQLinear(nn.Module):
             bias = self.bias.data_ptr() if self.bias is not None else None
             if m == 1 and self._inline():
                 rc = L.elutq_hlq_sparse_gemv_inline_f16(self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
-                                                        bias, self.sparse_inline.data_ptr(), x2.data_ptr(), y.data_ptr(),
+                                                        bias, self.sparse_inline.data_ptr(), self.sparse_inline.numel(), x2.data_ptr(), y.data_ptr(),
                                                         self.in_features, self.out_features, self.bits, self.group_size,
                                                         ws.data_ptr(), ws.numel(), stream, None, self.ksplit, self.waves)
                 _lib.check(rc, "elutq_hlq_sparse_gemv_inline_f16")
@@ -368,7 +368,7 @@ class HLQLinear(nn.Module):
         if self._inline():
             rc = _lib.lib().elutq_hlq_sparse_gemv_inline_f16(
                 self.planes.data_ptr(), self.scales.data_ptr(), self.zeros.data_ptr(),
-                self.bias.data_ptr() if self.bias is not None else None, self.sparse_inline.data_ptr(), x.data_ptr(),
+                self.bias.data_ptr() if self.bias is not None else None, self.sparse_inline.data_ptr(), self.sparse_inline.numel(), x.data_ptr(),
                 out.data_ptr(), self.in_features, self.out_features, self.bits, self.group_size, ws.data_ptr(), ws.numel(),
                 torch.cuda.current_stream(x.device).cuda_stream, ctypes.byref(f), self.ksplit, self.waves)
             _lib.check(rc, "elutq_hlq_sparse_gemv_inline_f16")

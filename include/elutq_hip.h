@@ -432,7 +432,9 @@ int elutq_hlq_dequant_f16(const void *d_planes, const void *d_scales, const void
  * the device unchanged.  ELUTQ_ERR_SPARSE for a block list the form cannot hold (off the grid, repeated, malformed):
  * such a layer keeps the two-launch entry points above.  elutq_hlq_sparse_gemv_inline_f16 is elutq_hlq_gemv_fused_f16
  * (fusion may be NULL; prologues, residual, K slices handed over or left to the next launch as there) on such a layer,
- * `bits` = base_bit <= 3, on the table-lookup kernels (wide or narrow tiles as for a dense layer); the workspace is that of the dense layer.  The
+ * `bits` = base_bit <= 3, on the table-lookup kernels (wide or narrow tiles as for a dense layer); the workspace is that of the dense layer;
+ * `inline_bytes` = the bytes of the form on the device (*bytes_used): less than the layer's cell table is ELUTQ_ERR_WORKSPACE, and a
+ * record number that points beyond it counts as "no block" instead of being followed.  The
  * result is the dense fp32 sum plus the blocks' terms, rounded once.
  */
 size_t elutq_hlq_sparse_index_bytes(int N, int nblk);
@@ -457,8 +459,8 @@ size_t elutq_hlq_sparse_inline_bytes(int K, int N, int group, int nblk);
 int elutq_hlq_sparse_inline_host(const uint32_t *h_mask, int mask_len, const void *h_blocks, const void *h_blk_scales,
                                  int K, int N, int group, void *h_out, size_t *bytes_used);
 int elutq_hlq_sparse_gemv_inline_f16(const void *d_planes, const void *d_scales, const void *d_zeros, const void *d_bias,
-                                     const void *d_inline, const void *d_x, void *d_y, int K, int N, int bits, int group,
-                                     void *d_workspace, size_t workspace_bytes, void *stream,
+                                     const void *d_inline, size_t inline_bytes, const void *d_x, void *d_y, int K, int N,
+                                     int bits, int group, void *d_workspace, size_t workspace_bytes, void *stream,
                                      const elutq_gemv_fusion *fusion, int ksplit, int waves);
 
 #ifdef __cplusplus

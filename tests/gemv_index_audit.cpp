@@ -17,6 +17,7 @@
 #include <vector>
 
 #include "hlq_gemv_index.h"
+#include "hlq_layout.h"
 
 namespace {
 
@@ -95,6 +96,21 @@ void audit(int bits, bool g64, int waves, int U, int ups, int ncb, int n_slices_
                     CHECK(((size_t)cb * NT + row) * (CB * 4) + 63 * 4 + 4 <= zero_bytes, "zeros");
                 }
             }
+            // inline sparse plane: record numbers of the run's first two units (fetched by every wave, clamped into the
+            // slice), of its further units only where the wave has their plane 0; the lookups use the unit's own tables
+            for (int cb = 0; cb < ncb; cb += (ncb > 1 ? ncb - 1 : 1)) {
+                for (int j = 0; j < 2; j++) {
+                    const int uj = r.ub + j < nU - 1 ? r.ub + j : nU - 1;
+                    CHECK(uj >= 0 && (size_t)cb * U + u0 + uj < (size_t)ncb * U, "sparse-cell");
+                    const bool own = j < r.nuw && r.s_begin <= (r.ub + j) * bits && (r.ub + j) * bits < r.s_end;
+                    if (own) CHECK(lut + (uint32_t)j * HLQ_UNIT_LUT_BYTES + 3 * 8 * 64 + 7 * 64 + 60 + 4 <= xs, "sparse-lookup");
+                }
+                for (int j = 2; j < r.nuw; j++) {
+                    if (!(r.s_begin <= (r.ub + j) * bits && (r.ub + j) * bits < r.s_end)) continue;
+                    CHECK(r.ub + j < nU && (size_t)cb * U + u0 + r.ub + j < (size_t)ncb * U, "sparse-cell");
+                    CHECK(lut + (uint32_t)j * HLQ_UNIT_LUT_BYTES + 3 * 8 * 64 + 7 * 64 + 60 + 4 <= xs, "sparse-lookup");
+                }
+            }
             // cross-wave sums (two alternating buffers), reduction scratch of the RMSNorm prologue
             for (int sel = 0; sel < 2; sel++)
                 CHECK(lm.red + ((uint32_t)(sel * waves + wave) * 64 + 63) * 4 + 4 <= lm.rstd, "lds-red");
@@ -157,6 +173,10 @@ void audit_narrow(int bits, bool g64, int cw, int rounds, int U, int ncb, bool r
                         CHECK(row < NT && ((size_t)cb * NT * bits + (size_t)row * bits + b) * (CB * 4) + 63 * 4 + 4 <= scale_bytes, "n-scales");
                         CHECK(((size_t)cb * NT + row) * (CB * 4) + 63 * 4 + 4 <= zero_bytes, "n-zeros");
                     }
+                // inline sparse plane: the record number of the lane's unit, the lane's 20 bytes of a 1280-byte record
+                for (int cb = 0; cb < ncb; cb += (ncb > 1 ? ncb - 1 : 1)) CHECK((size_t)cb * U + u < (size_t)ncb * U, "n-sparse-cell");
+                for (int part = 0; part < ul_count; part++)
+                    CHECK((size_t)(part * cw + cw - 1) * 16 + 16 <= 1024 && 1024 + (size_t)(part * cw + cw - 1) * 4 + 4 <= HLQ_SP_REC_BYTES, "n-sparse-rec");
             }
         CHECK(lm.red + ((uint32_t)wave * 64 + 63) * 4 + 4 <= lm.rstd, "n-lds-red");
         CHECK(lm.rstd + (uint32_t)((waves * 64 - 1) >> 4) * 4 + 4 <= lm.rstd + 64 * 4 && lm.rstd + 64 * 4 + 4 <= lm.stage, "n-lds-rstd");

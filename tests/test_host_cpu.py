@@ -255,3 +255,17 @@ def test_sparse_inline_form_holds_every_block_where_the_kernel_looks(k, n, group
     assert sparse_inline(np.array([[0, 4]], np.uint32), one, scale[:1], k, n, group) is None
     two = pack_bits_lsb_first(bits[[0, 0]])
     assert sparse_inline(np.array([[0, 0], [0, 0]], np.uint32), two, scale[[0, 0]], k, n, group) is None
+
+
+def test_inline_sparse_call_checks_the_size_of_the_form():
+    """A form smaller than the layer's cell table is refused before anything is launched (no GPU needed for the
+    refusal: the argument checks come first)."""
+    L = _lib.lib()
+    one = ctypes.c_void_p(256)          # never dereferenced
+    need = 32 + 4 * (4096 // 64) * (4096 // 128)
+    rc = L.elutq_hlq_sparse_gemv_inline_f16(one, one, one, None, one, need - 1, one, one, 4096, 4096, 2, 128, one, 1 << 20,
+                                            None, None, 0, 0)
+    assert rc == -5, rc                 # ELUTQ_ERR_WORKSPACE
+    rc = L.elutq_hlq_sparse_gemv_inline_f16(one, one, one, None, one, 1 << 20, one, one, 4096, 4096, 4, 128, one, 1 << 20,
+                                            None, None, 0, 0)
+    assert rc == -3, rc                 # ELUTQ_ERR_BITS: the plane would be a fifth
